@@ -1,0 +1,102 @@
+/*
+ * ringattr.h -- C ABI of the MI355X (gfx950) leaky ring-attractor time loop.
+ *
+ * One shared library (libringattr.so) exports the forward recurrence and its
+ * reverse-time BPTT.  All tensors are fp32, contiguous, row-major DEVICE
+ * pointers owned by the caller; the library allocates nothing inside the
+ * ringattr_* entry points (the caller brings the workspace).  Work is enqueued
+ * on the HIP stream passed as `stream` (a hipStream_t, NULL = the null stream)
+ * and the calls return without synchronising.
+ *
+ * Shapes (B = batch_size, T = seq_len, k = a_dim, N = neurons):
+ *   A            [B,T,k]   action signal
+ *   Wa           [k,N,N]   action-modulated weight bank
+ *   Wo           [N,N]     recurrent weights
+ *   r_init       [B,N]     initial state (never modified)
+ *   bump_history [T,B,N]   state after every step (forward output)
+ *   grad_output  [T,B,N]   dL/d bump_history
+ *   grad_Wa [k,N,N], grad_Wo [N,N]   ACCUMULATED into (caller zeroes them)
+ *
+ * Math per sample b and step t (r_prev = r_init at t = 0):
+ *   re  = J0*sum_j r_prev[j] + J1*(Wo r_prev) + sum_c A[b,t,c]*(Wa[c] r_prev)
+ *   r_t = (1-alpha)*r_prev + alpha*F(re),   F in {relu, gelu(erf), tanh, silu}
+ *
+ * activation_type: 0 relu, 1 gelu, 2 tanh, 3 silu
+ * (reference: cpp/ring_rnn_cuda.py:63, cpp/cuda_common.cuh:56).
+ *
+ * Every int-returning entry point returns RINGATTR_OK or an error code;
+ * ringattr_last_error() gives the message.  Nothing here ever exits the process
+ * (the reference's CHECK_CUDA_ERROR does, cpp/cuda_common.cuh:30-39).
+ */
+#ifndef RINGATTR_H
+#define RINGATTR_H
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define RINGATTR_API __attribute__((visibility("default")))
+
+#define RINGATTR_OK 0
+#define RINGATTR_ERR_INVALID 1   /* bad shape, null pointer, unknown activation */
+#define RINGATTR_ERR_WORKSPACE 2 /* workspace pointer null or too small */
+#define RINGATTR_ERR_HIP 3       /* a HIP runtime call or kernel launch failed */
+
+/* Library version (major*1000 + minor). */
+RINGATTR_API int ringattr_version(void);
+
+/* Message of the last failing call made on the calling thread ("" if none). */
+RINGATTR_API const char* ringattr_last_error(void);
+
+/* Bytes of the "saved activations" buffer the forward pass fills for training:
+ * F'(re) as fp16 and the bf16 operand copy of r_prev, both in the kernels'
+ * private tile order.  Opaque to the caller: allocate, pass to ringattr_fwd,
+ * keep until ringattr_bwd.  Replaces the reference's re_history slot
+ * (cpp/ring_rnn_cuda.py:106, cpp/bwd.cu:12). */
+RINGATTR_API size_t ringattr_saved_bytes(int N, int a_dim, int seq_len, int batch_size);
+
+/* Scratch bytes needed by ringattr_fwd / ringattr_bwd.  have_saved = 1 when the
+ * forward's saved buffer will be handed to the backward, 0 when the backward
+ * must rebuild it from bump_history (then the workspace also holds it).
+ * Replaces the fixed workspace list of cpp/ring_rnn_cuda.py:108-114. */
+RINGATTR_API size_t ringattr_fwd_workspace_bytes(int N, int a_dim, int seq_len, int batch_size);
+RINGATTR_API size_t ringattr_bwd_workspace_bytes(int N, int a_dim, int seq_len, int batch_size, int have_saved);
+
+/* Forward recurrence over all T steps in one persistent launch.
+ * Replaces fwd_cuda (cpp/fwd.cu:21-50) and the pybind shim cpp/fwd.cpp:20-47.
+ * `saved` may be NULL (inference: nothing but bump_history is written). */
+RINGATTR_API int ringattr_fwd(const void* A, const void* Wa, float J0, float J1, const void* Wo,
+                 const void* r_init, void* bump_history, float alpha,
+                 int N, int a_dim, int seq_len, int batch_size, int activation_type,
+                 void* saved, void* workspace, size_t workspace_bytes, void* stream);
+
+/* Reverse-time BPTT + weight gradients.
+ * Replaces bwd_cuda (cpp/bwd.cu:4-52) and cpp/bwd.cpp:34-99.
+ * `saved` may be NULL: F'(re) is then recomputed from bump_history.
+ * grad_A [B,T,k] and grad_r_init [B,N] are optional outputs (NULL = skip); the
+ * reference returns None for both (cpp/ring_rnn_cuda.py:144). */
+RINGATTR_API int ringattr_bwd(const void* grad_output, const void* A, const void* Wa, float J0, float J1,
+                 const void* Wo, const void* bump_history, const void* r_init,
+                 void* grad_Wa, void* grad_Wo, float alpha,
+                 int N, int a_dim, int seq_len, int batch_size, int activation_type,
+                 const void* saved, void* grad_A, void* grad_r_init,
+                 void* workspace, size_t workspace_bytes, void* stream);
+
+/* Reference-signature entry points, argument for argument (cpp/fwd.cu:21-35,
+ * cpp/bwd.cu:4-30).  They run on the null stream, obtain their scratch with
+ * hipMalloc/hipFree around the call, ignore the reference's workspace pointers
+ * and cublas_handle, and report failures on stderr without exiting. */
+RINGATTR_API void fwd_cuda(void* A, void* Wa, float J0, float J1, void* Wo, void* r_init, void* bump_history,
+              float alpha, int N, int a_dim, int seq_len, int batch_size, int activation_type);
+RINGATTR_API void bwd_cuda(void* grad_output, void* A, void* Wa, float J0, float J1, void* Wo,
+              void* bump_history, void* re_history, void* r_init, void* grad_Wa, void* grad_Wo,
+              float alpha, int N, int a_dim, int seq_len, int batch_size, int activation_type,
+              void* grad_r, void* W_eff_temp, void* grad_re_temp, void* grad_W_eff_temp_bf16,
+              void* A_t_temp_bf16, void* grad_re_temp_T, void* cublas_handle);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* RINGATTR_H */

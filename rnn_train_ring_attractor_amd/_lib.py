@@ -1,0 +1,77 @@
+"""ctypes binding of libringattr.so (the C ABI declared in include/ringattr.h).
+
+The library is looked up next to this file (prebuilt, in-tree); if it is absent it is built once
+with hipcc (same prebuilt-then-build order as the reference's cpp/ring_rnn_cuda.py:6-16).  There is
+no CPU fallback: a missing or unloadable library raises.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+import threading
+
+import torch  # noqa: F401  (loads torch's libamdhip64 first so the library binds to the same HIP runtime)
+
+from . import build as _build
+
+_lock = threading.Lock()
+_lib = None
+
+c_void_p, c_int, c_float, c_size_t, c_char_p = (ctypes.c_void_p, ctypes.c_int, ctypes.c_float,
+                                                ctypes.c_size_t, ctypes.c_char_p)
+
+# name -> (restype, argtypes): one entry per prototype in include/ringattr.h
+PROTOTYPES = {
+    "ringattr_version": (c_int, []),
+    "ringattr_last_error": (c_char_p, []),
+    "ringattr_saved_bytes": (c_size_t, [c_int] * 4),
+    "ringattr_fwd_workspace_bytes": (c_size_t, [c_int] * 4),
+    "ringattr_bwd_workspace_bytes": (c_size_t, [c_int] * 5),
+    "ringattr_fwd": (c_int, [c_void_p, c_void_p, c_float, c_float, c_void_p, c_void_p, c_void_p, c_float,
+                             c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_size_t, c_void_p]),
+    "ringattr_bwd": (c_int, [c_void_p, c_void_p, c_void_p, c_float, c_float, c_void_p, c_void_p, c_void_p,
+                             c_void_p, c_void_p, c_float, c_int, c_int, c_int, c_int, c_int,
+                             c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
+    "fwd_cuda": (None, [c_void_p, c_void_p, c_float, c_float, c_void_p, c_void_p, c_void_p, c_float,
+                        c_int, c_int, c_int, c_int, c_int]),
+    "bwd_cuda": (None, [c_void_p, c_void_p, c_void_p, c_float, c_float, c_void_p, c_void_p, c_void_p, c_void_p,
+                        c_void_p, c_void_p, c_float, c_int, c_int, c_int, c_int, c_int,
+                        c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
+}
+
+
+def library_path() -> str:
+    return _build.LIB_PATH
+
+
+def load():
+    """Return the loaded library, building it first if no prebuilt file exists."""
+    global _lib
+    with _lock:
+        if _lib is not None:
+            return _lib
+        path = library_path()
+        if not os.path.exists(path):
+            _build.build_library()
+        lib = ctypes.CDLL(path)
+        for name, (res, args) in PROTOTYPES.items():
+            fn = getattr(lib, name)          # AttributeError if the library lacks a declared symbol
+            fn.restype = res
+            fn.argtypes = args
+        _lib = lib
+        return lib
+
+
+def last_error() -> str:
+    return load().ringattr_last_error().decode("utf-8", "replace")
+
+
+def check(rc: int) -> None:
+    """Turn a status code into a Python exception (the reference exits the process instead,
+    cpp/cuda_common.cuh:30-39)."""
+    if rc == 0:
+        return
+    msg = last_error()
+    if rc == 1:
+        raise ValueError(msg)
+    raise RuntimeError(msg)

@@ -1,0 +1,187 @@
+// Shared device helpers for the gfx950 ring-attractor kernels: vector types, tile geometry,
+// activation math, LDS operand exchange, and the private "tile order" used for side buffers.
+//
+// Tile geometry (all kernels).  A workgroup is 4 wavefronts (256 lanes) and owns 16 batch rows.
+// Neurons are padded to NPAD = 64*NC; wave w owns the 16*NC contiguous neurons starting at
+// 16*NC*w and splits them into NC MFMA column tiles of 16: tile c, column n <-> neuron
+// 16*NC*w + NC*n + c.  A lane (q = lane/16, n = lane%16) therefore holds, after a 16x16 MFMA,
+// batch rows 4q..4q+3 of NC CONSECUTIVE neurons -- which makes the fp32 history stores, the bf16
+// operand write-back and the side-buffer stores all contiguous per lane.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+
+enum : int { ACT_RELU = 0, ACT_GELU = 1, ACT_TANH = 2, ACT_SILU = 3 };  // cpp/cuda_common.cuh:56
+
+template <int NC_>
+struct Tile {
+  static constexpr int NC = NC_;
+  static constexpr int NPAD = 64 * NC;          // padded neuron count
+  static constexpr int KCH = 2 * NC;            // K chunks of 32 along the contraction
+  static constexpr int KG = KCH < 8 ? KCH : 8;  // chunks staged per register group
+  static constexpr int NKG = KCH / KG;
+  static constexpr int GW = (NC % 4 == 0) ? 4 : ((NC % 2 == 0) ? 2 : 1);  // LDS write granule
+  static constexpr int SLOTS = KCH * 64;        // 16-byte operand slots per LDS buffer
+};
+
+// D = A(16x32 bf16) * B(32x16 bf16) + C(16x16 fp32).  Lane (q,n): A row n, B column n, both with
+// K slots 8q..8q+7; C/D rows 4q..4q+3 of column n.
+__device__ __forceinline__ f32x4 mfma16(bf16x8 a, bf16x8 b, f32x4 c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+}
+
+// F(x) and F'(x).  gelu is the exact erf form (train/train_ring_attractor.py:16), its derivative
+// uses the normal density 1/sqrt(2*pi) as the torch path does (legacy/bwd_fp32.py:455-457).
+__device__ __forceinline__ void act_eval(int act, float x, float& F, float& D) {
+  switch (act) {
+    case ACT_RELU:
+      F = fmaxf(x, 0.f);
+      D = x > 0.f ? 1.f : 0.f;
+      break;
+    case ACT_GELU: {
+      float cdf = 0.5f * erfcf(-x * 0.70710678118654752f);
+      float pdf = 0.39894228040143268f * __expf(-0.5f * x * x);
+      F = x * cdf;
+      D = cdf + x * pdf;
+      break;
+    }
+    case ACT_TANH: {
+      float th = tanhf(x);
+      F = th;
+      D = 1.f - th * th;
+      break;
+    }
+    default: {  // ACT_SILU
+      float s = 1.f / (1.f + __expf(-x));
+      F = x * s;
+      D = s * (1.f + x * (1.f - s));
+      break;
+    }
+  }
+}
+
+// Sum over the 16 lanes that share q (one MFMA column group); every lane gets the total.
+__device__ __forceinline__ float row16_sum(float v) {
+  v += __shfl_xor(v, 1, 16);
+  v += __shfl_xor(v, 2, 16);
+  v += __shfl_xor(v, 4, 16);
+  v += __shfl_xor(v, 8, 16);
+  return v;
+}
+
+// LDS operand buffer: slot(kc,q,b) = (kc*4+q)*16 + b holds the 8 bf16 values
+// x[b][32kc+8q .. +7]; an MFMA A-operand read by lane (q,b) is slot(kc,q,b): the 64 lanes read
+// 1 KiB contiguous.  This writes the lane's [4 rows][NC neurons] fp32 values as bf16.
+template <int NC>
+__device__ __forceinline__ void write_operand(bf16x8* xb, const float (&v)[4][NC], int w, int q, int n) {
+  constexpr int G = Tile<NC>::GW;
+  char* base = reinterpret_cast<char*>(xb);
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const int b = 4 * q + e;
+#pragma unroll
+    for (int c0 = 0; c0 < NC; c0 += G) {
+      const int j = 16 * NC * w + NC * n + c0;
+      const int slot = (((j >> 5) * 4 + ((j >> 3) & 3)) * 16 + b);
+      char* dst = base + slot * 16 + (j & 7) * 2;
+      if constexpr (G == 4) {
+        bf16x4 pk = {(__bf16)v[e][c0], (__bf16)v[e][c0 + 1], (__bf16)v[e][c0 + 2], (__bf16)v[e][c0 + 3]};
+        *reinterpret_cast<bf16x4*>(dst) = pk;
+      } else if constexpr (G == 2) {
+        bf16x2 pk = {(__bf16)v[e][c0], (__bf16)v[e][c0 + 1]};
+        *reinterpret_cast<bf16x2*>(dst) = pk;
+      } else {
+        *reinterpret_cast<__bf16*>(dst) = (__bf16)v[e][c0];
+      }
+    }
+  }
+}
+
+// Side buffers (saved F', bf16 operand copies of r_prev and g) use the private tile order
+//   S[t][bt][w][lane][c][e],  element = X[t][16*bt + 4q + e][16*NC*w + NC*n + c]
+// so each lane moves 4*NC contiguous 2-byte values and the weight-gradient GEMM can load MFMA
+// fragments (8 samples of one neuron = rows 4q..4q+3 of two time steps) without a transpose.
+template <int NC>
+__device__ __forceinline__ size_t side_offset(int t, int nbt, int bt, int w, int lane) {
+  return ((((size_t)t * nbt + bt) * 4 + w) * 64 + lane) * (size_t)(4 * NC);
+}
+
+template <int NC, typename V4, typename S>
+__device__ __forceinline__ void side_store(S* dst, const float (&v)[4][NC]) {
+#pragma unroll
+  for (int c = 0; c < NC; ++c) {
+    V4 pk = {(S)v[0][c], (S)v[1][c], (S)v[2][c], (S)v[3][c]};
+    *reinterpret_cast<V4*>(dst + 4 * c) = pk;
+  }
+}
+
+template <int NC>
+__device__ __forceinline__ void side_load_f16(const _Float16* src, float (&v)[4][NC]) {
+#pragma unroll
+  for (int c = 0; c < NC; ++c) {
+    f16x4 pk = *reinterpret_cast<const f16x4*>(src + 4 * c);
+    v[0][c] = (float)pk[0];
+    v[1][c] = (float)pk[1];
+    v[2][c] = (float)pk[2];
+    v[3][c] = (float)pk[3];
+  }
+}
+
+// Masked fp32 [rows][N] <-> lane registers.  slab points at row 0 of a [B][N] matrix.
+template <int NC>
+__device__ __forceinline__ void rows_load(const float* slab, int N, int B, int b0, int i0, float (&v)[4][NC]) {
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const int b = b0 + e;
+    if constexpr (NC % 4 == 0) {
+      if ((N & 3) == 0 && i0 + NC <= N && b < B) {
+        const float* row = slab + (size_t)b * N + i0;
+#pragma unroll
+        for (int c = 0; c < NC; c += 4) {
+          f32x4 pk = *reinterpret_cast<const f32x4*>(row + c);
+          v[e][c] = pk[0];
+          v[e][c + 1] = pk[1];
+          v[e][c + 2] = pk[2];
+          v[e][c + 3] = pk[3];
+        }
+        continue;
+      }
+    }
+#pragma unroll
+    for (int c = 0; c < NC; ++c) {
+      const int i = i0 + c;
+      v[e][c] = (b < B && i < N) ? slab[(size_t)b * N + i] : 0.f;
+    }
+  }
+}
+
+template <int NC>
+__device__ __forceinline__ void rows_store(float* slab, int N, int B, int b0, int i0, const float (&v)[4][NC]) {
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const int b = b0 + e;
+    if (b >= B) continue;
+    float* row = slab + (size_t)b * N + i0;
+    if constexpr (NC % 4 == 0) {
+      // rows start 16-byte aligned when N % 4 == 0 (i0 is a multiple of NC)
+      if ((N & 3) == 0 && i0 + NC <= N) {
+#pragma unroll
+        for (int c = 0; c < NC; c += 4) {
+          f32x4 pk = {v[e][c], v[e][c + 1], v[e][c + 2], v[e][c + 3]};
+          *reinterpret_cast<f32x4*>(row + c) = pk;
+        }
+        continue;
+      }
+    }
+#pragma unroll
+    for (int c = 0; c < NC; ++c)
+      if (i0 + c < N) row[c] = v[e][c];
+  }
+}

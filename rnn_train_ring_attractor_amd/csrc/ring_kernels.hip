@@ -1,0 +1,461 @@
+// gfx950 kernels of the leaky ring-attractor time loop: weight packing, the persistent forward
+// recurrence, the reverse-time BPTT recurrence, the rebuild of saved activations from the state
+// history, and the split-K weight-gradient contraction with its fixed-order reduction.
+//
+// The per-step product r @ [Wo|Wa_0|..]^T is a dense bf16 MFMA contraction with fp32 accumulation;
+// the reference instead rebuilds W_eff per sample (cpp/kernels/fwd_1loop_tc_idx.cuh:50-232,
+// cpp/kernels/bwd_mixed_precision_aggressive.cuh:53-318).
+#include "ring_common.hpp"
+#include "ring_kernels.hpp"
+
+// ------------------------------------------------------------------------------------------------
+// Weight packing: fp32 [N][N] matrices -> bf16 MFMA B-operand fragments, zero padded to NPAD.
+//   out[mm][w][c][kc][lane][8]; lane (q,n) owns output column 16*NC*w + NC*n + c and the eight
+//   contraction indices 32kc+8q .. +7.  transposed = 0: value = W[col][contr] (forward, re = W r);
+//   transposed = 1: value = W[contr][col] (backward, g @ W).
+// ------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void ring_pack_weights_kernel(const float* __restrict__ Wo,
+                                                                const float* __restrict__ Wa,
+                                                                bf16x8* __restrict__ out, int N, int k, int NC,
+                                                                int transposed) {
+  const int KCH = 2 * NC;
+  const size_t total = (size_t)(1 + k) * 4 * NC * KCH * 64;
+  for (size_t u = (size_t)blockIdx.x * blockDim.x + threadIdx.x; u < total; u += (size_t)gridDim.x * blockDim.x) {
+    const int lane = (int)(u & 63);
+    size_t v = u >> 6;
+    const int kc = (int)(v % KCH);
+    v /= KCH;
+    const int c = (int)(v % NC);
+    v /= NC;
+    const int w = (int)(v & 3);
+    const int mm = (int)(v >> 2);
+    const int q = lane >> 4, n = lane & 15;
+    const int col = 16 * NC * w + NC * n + c;
+    const int k0 = 32 * kc + 8 * q;
+    const float* W = (mm == 0) ? Wo : Wa + (size_t)(mm - 1) * N * N;
+    bf16x8 pk;
+#pragma unroll
+    for (int x = 0; x < 8; ++x) {
+      const int kk = k0 + x;
+      float val = 0.f;
+      if (col < N && kk < N) val = transposed ? W[(size_t)kk * N + col] : W[(size_t)col * N + kk];
+      pk[x] = (__bf16)val;
+    }
+    out[u] = pk;
+  }
+}
+
+// ------------------------------------------------------------------------------------------------
+// Gated products for one step:  acc[c][e] = sum_mm coef_mm[e] * (X @ W_mm)[row 4q+e][tile c]
+// X is read as MFMA A-operand fragments from the LDS operand buffer, W_mm streams from the packed
+// global copy (L2 resident).  coef_0 = J1, coef_{1+j}[e] = A[b_e, t, j].
+// ------------------------------------------------------------------------------------------------
+template <int NC>
+__device__ __forceinline__ void gated_products(const bf16x8* __restrict__ xb, const bf16x8* __restrict__ Wp,
+                                               const float* __restrict__ A, int k, int T, int B, int t, int b0,
+                                               float J1, int w, int lane, f32x4 (&acc)[NC]) {
+  using TL = Tile<NC>;
+  const int q = lane >> 4, n = lane & 15;
+#pragma unroll
+  for (int c = 0; c < NC; ++c) acc[c] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  for (int mm = 0; mm <= k; ++mm) {
+    float coef[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const int b = b0 + e;
+      coef[e] = (mm == 0) ? J1 : ((b < B) ? A[((size_t)b * T + t) * k + (mm - 1)] : 0.f);
+    }
+    f32x4 p[NC];
+#pragma unroll
+    for (int c = 0; c < NC; ++c) p[c] = f32x4{0.f, 0.f, 0.f, 0.f};
+    const bf16x8* wm = Wp + ((size_t)(mm * 4 + w) * NC) * TL::KCH * 64 + lane;
+#pragma unroll
+    for (int kg = 0; kg < TL::NKG; ++kg) {
+      bf16x8 af[TL::KG];
+#pragma unroll
+      for (int u = 0; u < TL::KG; ++u) af[u] = xb[((kg * TL::KG + u) * 4 + q) * 16 + n];
+      bf16x8 wf[2][TL::KG];
+#pragma unroll
+      for (int u = 0; u < TL::KG; ++u) wf[0][u] = wm[(size_t)(0 * TL::KCH + kg * TL::KG + u) * 64];
+#pragma unroll
+      for (int c = 0; c < NC; ++c) {
+        if (c + 1 < NC) {
+#pragma unroll
+          for (int u = 0; u < TL::KG; ++u)
+            wf[(c + 1) & 1][u] = wm[(size_t)((c + 1) * TL::KCH + kg * TL::KG + u) * 64];
+        }
+#pragma unroll
+        for (int u = 0; u < TL::KG; ++u) p[c] = mfma16(af[u], wf[c & 1][u], p[c]);
+      }
+    }
+#pragma unroll
+    for (int c = 0; c < NC; ++c)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) acc[c][e] += coef[e] * p[c][e];
+  }
+}
+
+// Row sums over neurons: per-wave partials go to psum[w][16]; readers add the four in wave order.
+template <int NC>
+__device__ __forceinline__ void publish_rowsum(float* psum, const float (&v)[4][NC], int w, int q, int n) {
+  float s[4];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    float a = 0.f;
+#pragma unroll
+    for (int c = 0; c < NC; ++c) a += v[e][c];
+    s[e] = row16_sum(a);
+  }
+  if (n == 0) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) psum[w * 16 + 4 * q + e] = s[e];
+  }
+}
+
+__device__ __forceinline__ void read_rowsum(const float* psum, int q, float (&s)[4]) {
+#pragma unroll
+  for (int e = 0; e < 4; ++e)
+    s[e] = ((psum[0 * 16 + 4 * q + e] + psum[1 * 16 + 4 * q + e]) + psum[2 * 16 + 4 * q + e]) + psum[3 * 16 + 4 * q + e];
+}
+
+// ------------------------------------------------------------------------------------------------
+// Forward: one workgroup = 16 batch rows for all T steps.  r lives in fp32 registers; its bf16 copy
+// is exchanged between the four waves through a double-buffered LDS operand buffer (one barrier
+// per step).  Writes bump_history [T,B,N] fp32 and, when training, F'(re) (fp16) and the bf16
+// operand copy of r_prev in tile order.
+// ------------------------------------------------------------------------------------------------
+template <int NC>
+__global__ __launch_bounds__(256) void ring_fwd_kernel(RingFwdArgs p) {
+  using TL = Tile<NC>;
+  __shared__ bf16x8 xbuf[2][TL::SLOTS];
+  __shared__ float psum[2][64];
+
+  const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, q = lane >> 4, n = lane & 15;
+  const int bt = blockIdx.x;
+  const int b0 = 16 * bt + 4 * q;
+  const int i0 = 16 * NC * w + NC * n;
+  const int N = p.N, B = p.B, T = p.T;
+  const float oma = 1.f - p.alpha;
+
+  float r[4][NC];
+  rows_load<NC>(p.r_init, N, B, b0, i0, r);
+  write_operand<NC>(xbuf[0], r, w, q, n);
+  publish_rowsum<NC>(psum[0], r, w, q, n);
+  if (p.rfrag) side_store<NC, bf16x4, __bf16>(p.rfrag + side_offset<NC>(0, p.nbt, bt, w, lane), r);
+  __syncthreads();
+
+  for (int t = 0; t < T; ++t) {
+    const int cur = t & 1;
+    f32x4 acc[NC];
+    gated_products<NC>(xbuf[cur], (const bf16x8*)p.Wpack, p.A, p.k, T, B, t, b0, p.J1, w, lane, acc);
+    float s[4];
+    read_rowsum(psum[cur], q, s);
+    float d[4][NC];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+#pragma unroll
+      for (int c = 0; c < NC; ++c) {
+        const float x = acc[c][e] + p.J0 * s[e];
+        float F, D;
+        act_eval(p.act, x, F, D);
+        const bool ok = (b0 + e < B) && (i0 + c < N);
+        r[e][c] = ok ? (oma * r[e][c] + p.alpha * F) : 0.f;
+        d[e][c] = ok ? D : 0.f;
+      }
+    }
+    rows_store<NC>(p.hist + (size_t)t * B * N, N, B, b0, i0, r);
+    if (p.dfrag) side_store<NC, f16x4, _Float16>(p.dfrag + side_offset<NC>(t, p.nbt, bt, w, lane), d);
+    if (t + 1 < T) {
+      write_operand<NC>(xbuf[cur ^ 1], r, w, q, n);
+      publish_rowsum<NC>(psum[cur ^ 1], r, w, q, n);
+      if (p.rfrag) side_store<NC, bf16x4, __bf16>(p.rfrag + side_offset<NC>(t + 1, p.nbt, bt, w, lane), r);
+    }
+    __syncthreads();
+  }
+}
+
+// ------------------------------------------------------------------------------------------------
+// Rebuild of the saved activations from the state history (used when the forward's buffer was not
+// kept): one workgroup per (batch tile, step); no recurrence.
+// ------------------------------------------------------------------------------------------------
+template <int NC>
+__global__ __launch_bounds__(256) void ring_rebuild_saved_kernel(RingFwdArgs p) {
+  using TL = Tile<NC>;
+  __shared__ bf16x8 xbuf[TL::SLOTS];
+  __shared__ float psum[64];
+
+  const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, q = lane >> 4, n = lane & 15;
+  const int bt = blockIdx.x, t = blockIdx.y;
+  const int b0 = 16 * bt + 4 * q;
+  const int i0 = 16 * NC * w + NC * n;
+  const int N = p.N, B = p.B, T = p.T;
+
+  float r[4][NC];
+  const float* prev = (t == 0) ? p.r_init : p.hist + (size_t)(t - 1) * B * N;
+  rows_load<NC>(prev, N, B, b0, i0, r);
+  write_operand<NC>(xbuf, r, w, q, n);
+  publish_rowsum<NC>(psum, r, w, q, n);
+  side_store<NC, bf16x4, __bf16>(p.rfrag + side_offset<NC>(t, p.nbt, bt, w, lane), r);
+  __syncthreads();
+
+  f32x4 acc[NC];
+  gated_products<NC>(xbuf, (const bf16x8*)p.Wpack, p.A, p.k, T, B, t, b0, p.J1, w, lane, acc);
+  float s[4];
+  read_rowsum(psum, q, s);
+  float d[4][NC];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+#pragma unroll
+    for (int c = 0; c < NC; ++c) {
+      float F, D;
+      act_eval(p.act, acc[c][e] + p.J0 * s[e], F, D);
+      d[e][c] = ((b0 + e < B) && (i0 + c < N)) ? D : 0.f;
+    }
+  }
+  side_store<NC, f16x4, _Float16>(p.dfrag + side_offset<NC>(t, p.nbt, bt, w, lane), d);
+}
+
+// ------------------------------------------------------------------------------------------------
+// BPTT recurrence, reverse time.  carry = dL/dr_t flowing in from later steps (fp32 registers).
+//   G = carry + grad_output[t];  g = alpha * F'(re_t) * G  (bf16 copy -> LDS operand + gfrag)
+//   carry' = (1-alpha) G + J0 * sum_i g + J1 (g @ Wo) + sum_j A_j (g @ Wa_j)
+// legacy/bwd_fp32.py:86-109.  One barrier per step.
+// ------------------------------------------------------------------------------------------------
+template <int NC>
+__global__ __launch_bounds__(256) void ring_bptt_kernel(RingBpttArgs p) {
+  using TL = Tile<NC>;
+  __shared__ bf16x8 xbuf[2][TL::SLOTS];
+  __shared__ float psum[2][64];
+
+  const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, q = lane >> 4, n = lane & 15;
+  const int bt = blockIdx.x;
+  const int b0 = 16 * bt + 4 * q;
+  const int i0 = 16 * NC * w + NC * n;
+  const int N = p.N, B = p.B, T = p.T;
+  const float oma = 1.f - p.alpha;
+
+  float carry[4][NC];
+#pragma unroll
+  for (int e = 0; e < 4; ++e)
+#pragma unroll
+    for (int c = 0; c < NC; ++c) carry[e][c] = 0.f;
+
+  for (int t = T - 1; t >= 0; --t) {
+    const int cur = (T - 1 - t) & 1;
+    float G[4][NC], g[4][NC];
+    rows_load<NC>(p.grad_out + (size_t)t * B * N, N, B, b0, i0, G);
+    side_load_f16<NC>(p.dfrag + side_offset<NC>(t, p.nbt, bt, w, lane), g);
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+#pragma unroll
+      for (int c = 0; c < NC; ++c) {
+        G[e][c] += carry[e][c];
+        g[e][c] = p.alpha * g[e][c] * G[e][c];
+      }
+    write_operand<NC>(xbuf[cur], g, w, q, n);
+    publish_rowsum<NC>(psum[cur], g, w, q, n);
+    side_store<NC, bf16x4, __bf16>(p.gfrag + side_offset<NC>(t, p.nbt, bt, w, lane), g);
+    __syncthreads();
+
+    f32x4 acc[NC];
+    gated_products<NC>(xbuf[cur], (const bf16x8*)p.Wpack, p.A, p.k, T, B, t, b0, p.J1, w, lane, acc);
+    float s[4];
+    read_rowsum(psum[cur], q, s);
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+#pragma unroll
+      for (int c = 0; c < NC; ++c) {
+        const bool ok = (b0 + e < B) && (i0 + c < N);
+        carry[e][c] = ok ? (oma * G[e][c] + p.J0 * s[e] + acc[c][e]) : 0.f;
+      }
+  }
+  if (p.grad_r_init) rows_store<NC>(p.grad_r_init, N, B, b0, i0, carry);
+}
+
+// ------------------------------------------------------------------------------------------------
+// Weight gradients: dW_mm[i][j] = sum over samples (b,t) of coef_mm(b,t) * g[t,b,i] * r_prev[t,b,j]
+// (coef_0 = 1 here, J1 is applied in the reduction; coef_{1+c} = A[b,t,c]).
+// A K chunk is 16 batch rows x 2 time steps = 32 samples; MFMA fragments come straight from the
+// tile-ordered gfrag / rfrag buffers.  Each wave owns 2 row tiles x TJ column tiles x 3 matrices
+// over one K split and writes its fp32 partial; no atomics, fixed reduction order afterwards.
+// ------------------------------------------------------------------------------------------------
+__device__ __forceinline__ bf16x8 join8(bf16x4 lo, bf16x4 hi) {
+  return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+}
+
+__device__ __forceinline__ bf16x8 gate8(bf16x8 x, const float (&cf)[8]) {
+  bf16x8 o;
+#pragma unroll
+  for (int u = 0; u < 8; ++u) o[u] = (__bf16)((float)x[u] * cf[u]);
+  return o;
+}
+
+template <int NC, int TJ>
+__global__ __launch_bounds__(256) void ring_dw_kernel(RingDwArgs p) {
+  constexpr int NT = 4 * NC;       // 16-wide tiles per matrix side
+  constexpr int NIP = NT / 2;      // row-tile pairs
+  constexpr int NJO = NT / TJ;     // column-tile groups
+  const int lane = threadIdx.x & 63, q = lane >> 4;
+  const int nmg = (p.k + 3) / 3;   // groups of 3 matrices
+  long wid = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int ip = (int)(wid % NIP);
+  wid /= NIP;
+  const int jo = (int)(wid % NJO);
+  wid /= NJO;
+  const int mg = (int)(wid % nmg);
+  const int z = (int)(wid / nmg);
+  if (z >= p.nz) return;
+
+  const int T = p.T, B = p.B, k = p.k, nbt = p.nbt;
+  const int TP = (T + 1) / 2;
+  const long nchunk = (long)nbt * TP;
+  const long ch0 = nchunk * z / p.nz, ch1 = nchunk * (z + 1) / p.nz;
+
+  f32x4 acc[3][2][TJ];
+#pragma unroll
+  for (int a = 0; a < 3; ++a)
+#pragma unroll
+    for (int ii = 0; ii < 2; ++ii)
+#pragma unroll
+      for (int u = 0; u < TJ; ++u) acc[a][ii][u] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  const bf16x4 zero4 = {(__bf16)0.f, (__bf16)0.f, (__bf16)0.f, (__bf16)0.f};
+  for (long ch = ch0; ch < ch1; ++ch) {
+    const int bt = (int)(ch % nbt);
+    const int t0 = 2 * (int)(ch / nbt), t1 = t0 + 1;
+    const bool has1 = t1 < T;
+    bf16x8 ga[2], rb[TJ];
+#pragma unroll
+    for (int ii = 0; ii < 2; ++ii) {
+      const int it = 2 * ip + ii, wi = it / NC, ci = it % NC;
+      const bf16x4 lo = *reinterpret_cast<const bf16x4*>(p.gfrag + side_offset<NC>(t0, nbt, bt, wi, lane) + 4 * ci);
+      const bf16x4 hi = has1 ? *reinterpret_cast<const bf16x4*>(p.gfrag + side_offset<NC>(t1, nbt, bt, wi, lane) + 4 * ci) : zero4;
+      ga[ii] = join8(lo, hi);
+    }
+#pragma unroll
+    for (int u = 0; u < TJ; ++u) {
+      const int jt = jo * TJ + u, wj = jt / NC, cj = jt % NC;
+      const bf16x4 lo = *reinterpret_cast<const bf16x4*>(p.rfrag + side_offset<NC>(t0, nbt, bt, wj, lane) + 4 * cj);
+      const bf16x4 hi = has1 ? *reinterpret_cast<const bf16x4*>(p.rfrag + side_offset<NC>(t1, nbt, bt, wj, lane) + 4 * cj) : zero4;
+      rb[u] = join8(lo, hi);
+    }
+#pragma unroll
+    for (int a = 0; a < 3; ++a) {
+      const int mm = 3 * mg + a;
+      if (mm > k) break;
+      bf16x8 gg[2];
+      if (mm == 0) {
+        gg[0] = ga[0];
+        gg[1] = ga[1];
+      } else {
+        float cf[8];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int b = 16 * bt + 4 * q + e;
+          cf[e] = (b < B) ? p.A[((size_t)b * T + t0) * k + (mm - 1)] : 0.f;
+          cf[4 + e] = (b < B && has1) ? p.A[((size_t)b * T + t1) * k + (mm - 1)] : 0.f;
+        }
+        gg[0] = gate8(ga[0], cf);
+        gg[1] = gate8(ga[1], cf);
+      }
+#pragma unroll
+      for (int ii = 0; ii < 2; ++ii)
+#pragma unroll
+        for (int u = 0; u < TJ; ++u) acc[a][ii][u] = mfma16(gg[ii], rb[u], acc[a][ii][u]);
+    }
+  }
+
+#pragma unroll
+  for (int a = 0; a < 3; ++a) {
+    const int mm = 3 * mg + a;
+    if (mm > k) break;
+#pragma unroll
+    for (int ii = 0; ii < 2; ++ii)
+#pragma unroll
+      for (int u = 0; u < TJ; ++u) {
+        const int it = 2 * ip + ii, jt = jo * TJ + u;
+        p.partial[((((size_t)z * (k + 1) + mm) * NT + it) * NT + jt) * 64 + lane] = acc[a][ii][u];
+      }
+  }
+}
+
+// Fixed-order sum of the K-split partials, undoing the tile permutation, accumulated into the
+// caller's grad_Wo / grad_Wa (which the caller zeroed, cpp/ring_rnn_cuda.py:98-99).
+__global__ __launch_bounds__(256) void ring_dw_reduce_kernel(RingDwArgs p, int NC) {
+  const int NT = 4 * NC;
+  const size_t per_z = (size_t)(p.k + 1) * NT * NT * 64;
+  const size_t u = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (u >= per_z) return;
+  f32x4 s = {0.f, 0.f, 0.f, 0.f};
+  for (int z = 0; z < p.nz; ++z) s += p.partial[(size_t)z * per_z + u];
+  const int lane = (int)(u & 63);
+  size_t v = u >> 6;
+  const int jt = (int)(v % NT);
+  v /= NT;
+  const int it = (int)(v % NT);
+  const int mm = (int)(v / NT);
+  const int q = lane >> 4, n = lane & 15;
+  const int j = 16 * NC * (jt / NC) + NC * n + (jt % NC);
+  if (j >= p.N) return;
+  float* out = (mm == 0) ? p.grad_Wo : p.grad_Wa + (size_t)(mm - 1) * p.N * p.N;
+  const float scale = (mm == 0) ? p.J1 : 1.f;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const int i = 16 * NC * (it / NC) + NC * (4 * q + e) + (it % NC);
+    if (i < p.N) out[(size_t)i * p.N + j] += scale * s[e];
+  }
+}
+
+// ------------------------------------------------------------------------------------------------
+// Launchers (host).  NC is chosen by the caller as the smallest of {1,2,4,8} with 64*NC >= N.
+// ------------------------------------------------------------------------------------------------
+#define RING_DISPATCH_NC(NCv, CALL)                 \
+  switch (NCv) {                                    \
+    case 1: { constexpr int NC = 1; CALL; } break;  \
+    case 2: { constexpr int NC = 2; CALL; } break;  \
+    case 4: { constexpr int NC = 4; CALL; } break;  \
+    case 8: { constexpr int NC = 8; CALL; } break;  \
+    default: return hipErrorInvalidValue;           \
+  }
+
+hipError_t ring_launch_pack(const float* Wo, const float* Wa, void* out, int N, int k, int NC, int transposed,
+                            hipStream_t st) {
+  const size_t total = (size_t)(1 + k) * 4 * NC * 2 * NC * 64;
+  const int blocks = (int)((total + 255) / 256 < 4096 ? (total + 255) / 256 : 4096);
+  hipLaunchKernelGGL(ring_pack_weights_kernel, dim3(blocks), dim3(256), 0, st, Wo, Wa, (bf16x8*)out, N, k, NC,
+                     transposed);
+  return hipGetLastError();
+}
+
+hipError_t ring_launch_fwd(const RingFwdArgs& a, int NCv, hipStream_t st) {
+  RING_DISPATCH_NC(NCv, hipLaunchKernelGGL(ring_fwd_kernel<NC>, dim3(a.nbt), dim3(256), 0, st, a));
+  return hipGetLastError();
+}
+
+hipError_t ring_launch_rebuild(const RingFwdArgs& a, int NCv, hipStream_t st) {
+  RING_DISPATCH_NC(NCv, hipLaunchKernelGGL(ring_rebuild_saved_kernel<NC>, dim3(a.nbt, a.T), dim3(256), 0, st, a));
+  return hipGetLastError();
+}
+
+hipError_t ring_launch_bptt(const RingBpttArgs& a, int NCv, hipStream_t st) {
+  RING_DISPATCH_NC(NCv, hipLaunchKernelGGL(ring_bptt_kernel<NC>, dim3(a.nbt), dim3(256), 0, st, a));
+  return hipGetLastError();
+}
+
+hipError_t ring_launch_dw(const RingDwArgs& a, int NCv, hipStream_t st) {
+  const int NT = 4 * NCv;
+  const int TJ = NCv == 1 ? 4 : 8;
+  const long waves = (long)(NT / 2) * (NT / TJ) * ((a.k + 3) / 3) * a.nz;
+  const int blocks = (int)((waves + 3) / 4);
+  if (NCv == 1) {
+    hipLaunchKernelGGL((ring_dw_kernel<1, 4>), dim3(blocks), dim3(256), 0, st, a);
+  } else {
+    RING_DISPATCH_NC(NCv, if constexpr (NC >= 2) hipLaunchKernelGGL((ring_dw_kernel<NC, 8>), dim3(blocks), dim3(256), 0, st, a));
+  }
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return e;
+  const size_t per_z = (size_t)(a.k + 1) * NT * NT * 64;
+  hipLaunchKernelGGL(ring_dw_reduce_kernel, dim3((unsigned)((per_z + 255) / 256)), dim3(256), 0, st, a, NCv);
+  return hipGetLastError();
+}

@@ -1,0 +1,46 @@
+// Host-visible argument blocks and launchers of the ring-attractor kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+
+typedef float ring_f32x4 __attribute__((ext_vector_type(4)));
+
+struct RingFwdArgs {
+  const float* A;        // [B,T,k]
+  const void* Wpack;     // packed bf16 forward fragments
+  const float* r_init;   // [B,N]
+  float* hist;           // [T,B,N] (forward: output; rebuild: input)
+  _Float16* dfrag;       // F'(re) in tile order, or null
+  __bf16* rfrag;         // bf16 r_prev in tile order, or null
+  float J0, J1, alpha;
+  int N, k, T, B, nbt, act;
+};
+
+struct RingBpttArgs {
+  const float* A;
+  const void* Wpack;     // packed bf16 transposed fragments
+  const float* grad_out; // [T,B,N]
+  const _Float16* dfrag;
+  __bf16* gfrag;         // bf16 g in tile order (output)
+  float* grad_r_init;    // [B,N] or null
+  float J0, J1, alpha;
+  int N, k, T, B, nbt;
+};
+
+struct RingDwArgs {
+  const float* A;
+  const __bf16* gfrag;
+  const __bf16* rfrag;
+  ring_f32x4* partial;   // [nz][1+k][NT][NT][64] fp32x4
+  float* grad_Wo;        // [N,N], accumulated into
+  float* grad_Wa;        // [k,N,N], accumulated into
+  float J1;
+  int N, k, T, B, nbt, nz;
+};
+
+hipError_t ring_launch_pack(const float* Wo, const float* Wa, void* out, int N, int k, int NC, int transposed,
+                            hipStream_t st);
+hipError_t ring_launch_fwd(const RingFwdArgs& a, int NC, hipStream_t st);
+hipError_t ring_launch_rebuild(const RingFwdArgs& a, int NC, hipStream_t st);
+hipError_t ring_launch_bptt(const RingBpttArgs& a, int NC, hipStream_t st);
+hipError_t ring_launch_dw(const RingDwArgs& a, int NC, hipStream_t st);

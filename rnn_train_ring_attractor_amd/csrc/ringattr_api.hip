@@ -1,0 +1,291 @@
+// C ABI of libringattr.so: argument validation, workspace carving and kernel sequencing.
+// Entry points and the reference interfaces they replace are documented in include/ringattr.h.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+#include "ring_kernels.hpp"
+#include "ringattr.h"
+
+namespace {
+
+thread_local char g_err[512] = "";
+
+int fail(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
+int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+constexpr size_t kAlign = 256;
+size_t align_up(size_t x) { return (x + kAlign - 1) / kAlign * kAlign; }
+
+struct Geo {
+  int N, k, T, B, NC, NPAD, nbt, nz;
+  size_t wpack_bytes;    // one packed copy of [Wo|Wa] in bf16
+  size_t side_bytes;     // one tile-ordered 2-byte [T,16*nbt,NPAD] side buffer
+  size_t partial_bytes;  // split-K partials of the weight gradient
+};
+
+// Smallest supported neuron tiling with 64*NC >= N.
+int pick_nc(int N) {
+  for (int nc = 1; nc <= 8; nc *= 2)
+    if (64 * nc >= N) return nc;
+  return 0;
+}
+
+int make_geo(int N, int k, int T, int B, Geo& g) {
+  if (N <= 0 || k <= 0 || T <= 0 || B <= 0)
+    return fail(RINGATTR_ERR_INVALID, "N, a_dim, seq_len, batch_size must be positive (got %d, %d, %d, %d)", N, k, T, B);
+  const int nc = pick_nc(N);
+  if (nc == 0) return fail(RINGATTR_ERR_INVALID, "N = %d exceeds the supported maximum of 512 neurons", N);
+  g.N = N;
+  g.k = k;
+  g.T = T;
+  g.B = B;
+  g.NC = nc;
+  g.NPAD = 64 * nc;
+  g.nbt = (B + 15) / 16;
+  g.wpack_bytes = align_up((size_t)(1 + k) * g.NPAD * g.NPAD * 2);
+  g.side_bytes = align_up((size_t)T * g.nbt * 16 * g.NPAD * 2);
+  const int NT = 4 * nc, TJ = nc == 1 ? 4 : 8;
+  const long per_z = (long)(NT / 2) * (NT / TJ) * ((k + 3) / 3);  // wave work items per K split
+  const long nchunk = (long)g.nbt * ((T + 1) / 2);
+  long nz = (2048 + per_z - 1) / per_z;
+  if (nz > 128) nz = 128;
+  if (nz > nchunk) nz = nchunk;
+  if (nz < 1) nz = 1;
+  g.nz = (int)nz;
+  g.partial_bytes = align_up((size_t)g.nz * (1 + k) * g.NPAD * g.NPAD * 4);
+  return RINGATTR_OK;
+}
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+int check_act(int a) {
+  if (a < 0 || a > 3) return fail(RINGATTR_ERR_INVALID, "activation_type %d is not one of 0 relu, 1 gelu, 2 tanh, 3 silu", a);
+  return RINGATTR_OK;
+}
+
+int hip_fail(hipError_t e, const char* what) {
+  return fail(RINGATTR_ERR_HIP, "%s: %s", what, hipGetErrorString(e));
+}
+
+}  // namespace
+
+extern "C" {
+
+int ringattr_version(void) { return 1000; }
+
+const char* ringattr_last_error(void) { return g_err; }
+
+size_t ringattr_saved_bytes(int N, int a_dim, int seq_len, int batch_size) {
+  Geo g;
+  if (make_geo(N, a_dim, seq_len, batch_size, g) != RINGATTR_OK) return 0;
+  return 2 * g.side_bytes;
+}
+
+size_t ringattr_fwd_workspace_bytes(int N, int a_dim, int seq_len, int batch_size) {
+  Geo g;
+  if (make_geo(N, a_dim, seq_len, batch_size, g) != RINGATTR_OK) return 0;
+  return g.wpack_bytes;
+}
+
+size_t ringattr_bwd_workspace_bytes(int N, int a_dim, int seq_len, int batch_size, int have_saved) {
+  Geo g;
+  if (make_geo(N, a_dim, seq_len, batch_size, g) != RINGATTR_OK) return 0;
+  size_t s = g.wpack_bytes + g.side_bytes + g.partial_bytes;
+  if (!have_saved) s += g.wpack_bytes + 2 * g.side_bytes;
+  return s;
+}
+
+int ringattr_fwd(const void* A, const void* Wa, float J0, float J1, const void* Wo, const void* r_init,
+                 void* bump_history, float alpha, int N, int a_dim, int seq_len, int batch_size,
+                 int activation_type, void* saved, void* workspace, size_t workspace_bytes, void* stream) {
+  Geo g;
+  int rc = make_geo(N, a_dim, seq_len, batch_size, g);
+  if (rc) return rc;
+  if ((rc = check_act(activation_type))) return rc;
+  if (!A || !Wa || !Wo || !r_init || !bump_history) return fail(RINGATTR_ERR_INVALID, "ringattr_fwd: null tensor pointer");
+  if (!aligned16(A) || !aligned16(Wa) || !aligned16(Wo) || !aligned16(r_init) || !aligned16(bump_history) ||
+      !aligned16(saved) || !aligned16(workspace))
+    return fail(RINGATTR_ERR_INVALID, "ringattr_fwd: every pointer must be 16-byte aligned");
+  if (!workspace || workspace_bytes < g.wpack_bytes)
+    return fail(RINGATTR_ERR_WORKSPACE, "ringattr_fwd: workspace of %zu bytes needed, %zu given", g.wpack_bytes,
+                workspace ? workspace_bytes : (size_t)0);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+
+  hipError_t e = ring_launch_pack((const float*)Wo, (const float*)Wa, workspace, N, a_dim, g.NC, 0, st);
+  if (e != hipSuccess) return hip_fail(e, "pack weights");
+
+  RingFwdArgs a;
+  a.A = (const float*)A;
+  a.Wpack = workspace;
+  a.r_init = (const float*)r_init;
+  a.hist = (float*)bump_history;
+  a.dfrag = saved ? (_Float16*)saved : nullptr;
+  a.rfrag = saved ? (__bf16*)((char*)saved + g.side_bytes) : nullptr;
+  a.J0 = J0;
+  a.J1 = J1;
+  a.alpha = alpha;
+  a.N = N;
+  a.k = a_dim;
+  a.T = seq_len;
+  a.B = batch_size;
+  a.nbt = g.nbt;
+  a.act = activation_type;
+  e = ring_launch_fwd(a, g.NC, st);
+  if (e != hipSuccess) return hip_fail(e, "forward launch");
+  return RINGATTR_OK;
+}
+
+int ringattr_bwd(const void* grad_output, const void* A, const void* Wa, float J0, float J1, const void* Wo,
+                 const void* bump_history, const void* r_init, void* grad_Wa, void* grad_Wo, float alpha, int N,
+                 int a_dim, int seq_len, int batch_size, int activation_type, const void* saved, void* grad_A,
+                 void* grad_r_init, void* workspace, size_t workspace_bytes, void* stream) {
+  Geo g;
+  int rc = make_geo(N, a_dim, seq_len, batch_size, g);
+  if (rc) return rc;
+  if ((rc = check_act(activation_type))) return rc;
+  if (!grad_output || !A || !Wa || !Wo || !bump_history || !r_init || !grad_Wa || !grad_Wo)
+    return fail(RINGATTR_ERR_INVALID, "ringattr_bwd: null tensor pointer");
+  if (grad_A) return fail(RINGATTR_ERR_INVALID, "ringattr_bwd: grad_A output is not implemented yet; pass NULL");
+  if (!aligned16(grad_output) || !aligned16(A) || !aligned16(Wa) || !aligned16(Wo) || !aligned16(bump_history) ||
+      !aligned16(r_init) || !aligned16(grad_Wa) || !aligned16(grad_Wo) || !aligned16(saved) ||
+      !aligned16(grad_r_init) || !aligned16(workspace))
+    return fail(RINGATTR_ERR_INVALID, "ringattr_bwd: every pointer must be 16-byte aligned");
+  const size_t need = ringattr_bwd_workspace_bytes(N, a_dim, seq_len, batch_size, saved != nullptr);
+  if (!workspace || workspace_bytes < need)
+    return fail(RINGATTR_ERR_WORKSPACE, "ringattr_bwd: workspace of %zu bytes needed, %zu given", need,
+                workspace ? workspace_bytes : (size_t)0);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+
+  char* ws = (char*)workspace;
+  void* wb = ws;
+  ws += g.wpack_bytes;
+  __bf16* gfrag = (__bf16*)ws;
+  ws += g.side_bytes;
+  ring_f32x4* partial = (ring_f32x4*)ws;
+  ws += g.partial_bytes;
+
+  const _Float16* dfrag;
+  const __bf16* rfrag;
+  if (saved) {
+    dfrag = (const _Float16*)saved;
+    rfrag = (const __bf16*)((const char*)saved + g.side_bytes);
+  } else {
+    void* wf = ws;
+    ws += g.wpack_bytes;
+    _Float16* d = (_Float16*)ws;
+    ws += g.side_bytes;
+    __bf16* r = (__bf16*)ws;
+    hipError_t e = ring_launch_pack((const float*)Wo, (const float*)Wa, wf, N, a_dim, g.NC, 0, st);
+    if (e != hipSuccess) return hip_fail(e, "pack weights");
+    RingFwdArgs f;
+    f.A = (const float*)A;
+    f.Wpack = wf;
+    f.r_init = (const float*)r_init;
+    f.hist = (float*)const_cast<void*>(bump_history);  // read only in the rebuild kernel
+    f.dfrag = d;
+    f.rfrag = r;
+    f.J0 = J0;
+    f.J1 = J1;
+    f.alpha = alpha;
+    f.N = N;
+    f.k = a_dim;
+    f.T = seq_len;
+    f.B = batch_size;
+    f.nbt = g.nbt;
+    f.act = activation_type;
+    e = ring_launch_rebuild(f, g.NC, st);
+    if (e != hipSuccess) return hip_fail(e, "rebuild launch");
+    dfrag = d;
+    rfrag = r;
+  }
+
+  hipError_t e = ring_launch_pack((const float*)Wo, (const float*)Wa, wb, N, a_dim, g.NC, 1, st);
+  if (e != hipSuccess) return hip_fail(e, "pack transposed weights");
+
+  RingBpttArgs b;
+  b.A = (const float*)A;
+  b.Wpack = wb;
+  b.grad_out = (const float*)grad_output;
+  b.dfrag = dfrag;
+  b.gfrag = gfrag;
+  b.grad_r_init = (float*)grad_r_init;
+  b.J0 = J0;
+  b.J1 = J1;
+  b.alpha = alpha;
+  b.N = N;
+  b.k = a_dim;
+  b.T = seq_len;
+  b.B = batch_size;
+  b.nbt = g.nbt;
+  e = ring_launch_bptt(b, g.NC, st);
+  if (e != hipSuccess) return hip_fail(e, "BPTT launch");
+
+  RingDwArgs d;
+  d.A = (const float*)A;
+  d.gfrag = gfrag;
+  d.rfrag = rfrag;
+  d.partial = partial;
+  d.grad_Wo = (float*)grad_Wo;
+  d.grad_Wa = (float*)grad_Wa;
+  d.J1 = J1;
+  d.N = N;
+  d.k = a_dim;
+  d.T = seq_len;
+  d.B = batch_size;
+  d.nbt = g.nbt;
+  d.nz = g.nz;
+  e = ring_launch_dw(d, g.NC, st);
+  if (e != hipSuccess) return hip_fail(e, "weight-gradient launch");
+  return RINGATTR_OK;
+}
+
+void fwd_cuda(void* A, void* Wa, float J0, float J1, void* Wo, void* r_init, void* bump_history, float alpha, int N,
+              int a_dim, int seq_len, int batch_size, int activation_type) {
+  const size_t need = ringattr_fwd_workspace_bytes(N, a_dim, seq_len, batch_size);
+  void* ws = nullptr;
+  if (need == 0 || hipMalloc(&ws, need) != hipSuccess) {
+    fprintf(stderr, "fwd_cuda: %s\n", need ? "workspace allocation failed" : ringattr_last_error());
+    return;
+  }
+  if (ringattr_fwd(A, Wa, J0, J1, Wo, r_init, bump_history, alpha, N, a_dim, seq_len, batch_size, activation_type,
+                   nullptr, ws, need, nullptr) != RINGATTR_OK)
+    fprintf(stderr, "fwd_cuda: %s\n", ringattr_last_error());
+  (void)hipStreamSynchronize(nullptr);
+  (void)hipFree(ws);
+}
+
+void bwd_cuda(void* grad_output, void* A, void* Wa, float J0, float J1, void* Wo, void* bump_history,
+              void* re_history, void* r_init, void* grad_Wa, void* grad_Wo, float alpha, int N, int a_dim,
+              int seq_len, int batch_size, int activation_type, void* grad_r, void* W_eff_temp, void* grad_re_temp,
+              void* grad_W_eff_temp_bf16, void* A_t_temp_bf16, void* grad_re_temp_T, void* cublas_handle) {
+  (void)re_history;
+  (void)grad_r;
+  (void)W_eff_temp;
+  (void)grad_re_temp;
+  (void)grad_W_eff_temp_bf16;
+  (void)A_t_temp_bf16;
+  (void)grad_re_temp_T;
+  (void)cublas_handle;
+  const size_t need = ringattr_bwd_workspace_bytes(N, a_dim, seq_len, batch_size, 0);
+  void* ws = nullptr;
+  if (need == 0 || hipMalloc(&ws, need) != hipSuccess) {
+    fprintf(stderr, "bwd_cuda: %s\n", need ? "workspace allocation failed" : ringattr_last_error());
+    return;
+  }
+  if (ringattr_bwd(grad_output, A, Wa, J0, J1, Wo, bump_history, r_init, grad_Wa, grad_Wo, alpha, N, a_dim, seq_len,
+                   batch_size, activation_type, nullptr, nullptr, nullptr, ws, need, nullptr) != RINGATTR_OK)
+    fprintf(stderr, "bwd_cuda: %s\n", ringattr_last_error());
+  (void)hipStreamSynchronize(nullptr);
+  (void)hipFree(ws);
+}
+
+}  // extern "C"

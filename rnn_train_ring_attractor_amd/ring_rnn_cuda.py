@@ -1,0 +1,62 @@
+"""Autograd operator of the ring-attractor time loop, HIP-backed.
+
+Same public names, argument order and semantics as the reference's cpp/ring_rnn_cuda.py:18-144:
+`ring_rnn_cuda_func(action_signal, Wa, J0, J1, Wo, r_init, alpha, activation='relu')` returns
+bump_history [T,B,N] and is differentiable w.r.t. Wa and Wo.  A star-import also hands out `torch`,
+which the reference training script relies on (train_general_ring_no_gain.py:19, 40).
+"""
+import torch
+from torch.autograd import Function
+
+from .rnn_cuda import fwd_cuda, bwd_cuda, saved_nbytes
+
+_ACTIVATION_MAP = {'relu': 0, 'gelu': 1, 'tanh': 2, 'silu': 3}   # cpp/ring_rnn_cuda.py:63
+
+
+def _activation_id(name):
+    if name not in _ACTIVATION_MAP:
+        raise ValueError(f"Invalid activation '{name}'. Must be one of {list(_ACTIVATION_MAP.keys())}.")
+    return _ACTIVATION_MAP[name]
+
+
+def ring_rnn_cuda_func(action_signal, Wa, J0, J1, Wo, r_init, alpha, activation='relu'):
+    """Ring RNN forward pass on the GPU.
+
+    action_signal (B,T,k); Wa (k,N,N); J0, J1 scalars; Wo (N,N); r_init (B,N); alpha float;
+    activation in {'relu','gelu','tanh','silu'}.  Returns bump_history (T,B,N).
+    """
+    return RingRnnCudaFunc.apply(action_signal, Wa, J0, J1, Wo, r_init, alpha, activation)
+
+
+class RingRnnCudaFunc(Function):
+    @staticmethod
+    def forward(ctx, action_signal, Wa, J0, J1, Wo, r_init, alpha, activation_name):
+        activation_type = _activation_id(activation_name)
+        batch_size, seq_len, a_dim = action_signal.shape
+        N = Wa.shape[1]
+        action_signal = action_signal.contiguous()
+        Wa_c, Wo_c, r0 = Wa.contiguous(), Wo.contiguous(), r_init.contiguous()
+        bump_history = torch.empty(seq_len, batch_size, N, device=action_signal.device, dtype=action_signal.dtype)
+
+        # F'(re) and the bf16 operand copy of r_prev are only worth writing when a backward will follow
+        needs_grad = ctx.needs_input_grad[1] or ctx.needs_input_grad[4]
+        saved = None
+        if needs_grad:
+            saved = torch.empty(saved_nbytes(N, a_dim, seq_len, batch_size), dtype=torch.uint8,
+                                device=action_signal.device)
+        fwd_cuda.fwd(A=action_signal, Wa=Wa_c, J0=J0, J1=J1, Wo=Wo_c, r_init=r0, bump_history=bump_history,
+                     alpha=alpha, activation_type=activation_type, saved=saved)
+
+        ctx.save_for_backward(action_signal, Wa_c, Wo_c, bump_history, r0, saved)
+        ctx.J0, ctx.J1, ctx.alpha, ctx.activation_type = J0, J1, alpha, activation_type
+        return bump_history
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        action_signal, Wa, Wo, bump_history, r_init, saved = ctx.saved_tensors
+        grad_Wa = torch.zeros_like(Wa)
+        grad_Wo = torch.zeros_like(Wo)
+        bwd_cuda.bwd(grad_output=grad_output.contiguous(), A=action_signal, Wa=Wa, J0=ctx.J0, J1=ctx.J1, Wo=Wo,
+                     bump_history=bump_history, r_init=r_init, grad_Wa=grad_Wa, grad_Wo=grad_Wo,
+                     alpha=ctx.alpha, activation_type=ctx.activation_type, saved=saved)
+        return None, grad_Wa, None, None, grad_Wo, None, None, None

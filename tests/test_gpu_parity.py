@@ -1,0 +1,171 @@
+"""GPU parity: the HIP path (through the operator API and the C ABI) against the fp64 oracle on the
+same seeded inputs.  Tolerances (bf16 operands, fp32 accumulation): state trajectories and decoded
+angles within 1e-2 (max error over max magnitude); weight gradients cosine >= 0.999 and max error
+over max magnitude <= 2e-2."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import ring_oracle as O
+from tests.ring_cases import make_problem
+
+pytestmark = pytest.mark.gpu
+
+TRAJ_TOL = 1e-2
+GRAD_COS = 0.999
+GRAD_TOL = 2e-2
+ACTS = {"relu": 0, "gelu": 1, "tanh": 2, "silu": 3}
+
+CASES = [
+    # name,            B,   T,   k,  N,  act,   J0,     J1,  action
+    ("config0",        64, 120,  2, 120, "tanh", -1 / 120, 1.0, "lr"),
+    ("config0_refJ",   64, 120,  2, 120, "tanh", -0.1, 0.1, "lr"),
+    ("script_k16",    128, 100, 16, 256, "gelu", -0.1, 0.1, "lr"),
+    ("n256_gelu",     256,  40,  2, 256, "gelu", -1 / 256, 1.0, "lr"),
+    ("n256_relu",      96,  30,  2, 256, "relu", -1 / 256, 1.0, "lr"),
+    ("ragged_silu",    37,   7,  3, 100, "silu", -0.1, 0.1, "dense"),
+    ("tiny_k1",         5,   3,  1,  48, "relu", 0.02, 0.5, "dense"),
+    ("n512_tanh",      32,  16,  2, 512, "tanh", -0.1, 0.1, "dense"),
+    ("n64_one_step",   16,   1,  2,  64, "gelu", -0.1, 0.1, "dense"),
+    ("odd_shapes",     17,   9,  5, 130, "gelu", -0.05, 0.2, "spread"),
+]
+
+
+def _dev(x, device):
+    return torch.tensor(x, device=device)
+
+
+def _run_op(p, J0, J1, act, device, requires_grad=True):
+    from rnn_train_ring_attractor_amd import ring_rnn_cuda_func
+    A, r0 = _dev(p["A"], device), _dev(p["r0"], device)
+    Wa = _dev(p["Wa"], device).requires_grad_(requires_grad)
+    Wo = _dev(p["Wo"], device).requires_grad_(requires_grad)
+    hist = ring_rnn_cuda_func(action_signal=A, Wa=Wa, J0=J0, J1=J1, Wo=Wo, r_init=r0, alpha=0.15, activation=act)
+    return hist, Wa, Wo
+
+
+@pytest.mark.parametrize("case", CASES, ids=[c[0] for c in CASES])
+def test_forward_trajectory_and_decoded_angle(case, gpu_device):
+    name, B, T, k, N, act, J0, J1, action = case
+    print(f"[case] fwd {name} B={B} T={T} k={k} N={N} {act}", flush=True)
+    p = make_problem(100, B, T, k, N, action=action)
+    hist, _, _ = _run_op(p, J0, J1, act, gpu_device, requires_grad=False)
+    torch.cuda.synchronize()
+    got = hist.cpu().numpy().astype(np.float64)
+    ref, _ = O.forward_dense(p["A"], p["Wa"], J0, J1, p["Wo"], p["r0"], 0.15, act)
+    assert got.shape == (T, B, N)
+    assert np.isfinite(got).all()
+    err = O.max_rel_err(got, ref)
+    assert err <= TRAJ_TOL, f"trajectory error {err}"
+    # per-step error must not blow up along the sequence either
+    for t in (0, T // 2, T - 1):
+        assert O.max_rel_err(got[t], ref[t]) <= TRAJ_TOL
+
+
+@pytest.mark.parametrize("N,act", [(120, "tanh"), (256, "gelu"), (256, "relu")])
+def test_decoded_angles_with_bump_sustaining_weights(N, act, gpu_device):
+    """Decoded head direction is only well conditioned while a bump exists, so it is compared on the
+    reference's own sanity recipe: cos(d), cos(d +- pi/4) weights (train/train_ring_attractor.py:94-103)."""
+    from rnn_train_ring_attractor_amd import ring_rnn_cuda_func
+    B, T = 64, 120
+    print(f"[case] decode N={N} {act}", flush=True)
+    p = make_problem(500, B, T, 2, N)
+    idx = np.arange(N, dtype=np.float64)
+    d = 2 * np.pi * (idx[:, None] - idx[None, :]) / N
+    Wo = np.cos(d).astype(np.float32)
+    Wa = np.stack([np.cos(d + np.pi / 4), np.cos(d - np.pi / 4)]).astype(np.float32)
+    hist = ring_rnn_cuda_func(_dev(p["A"], gpu_device), _dev(Wa, gpu_device), -0.1, 0.1, _dev(Wo, gpu_device),
+                              _dev(p["r0"], gpu_device), 0.15, act)
+    got = hist.cpu().numpy().astype(np.float64)
+    ref, _ = O.forward_dense(p["A"], Wa, -0.1, 0.1, Wo, p["r0"], 0.15, act)
+    assert O.max_rel_err(got, ref) <= TRAJ_TOL
+    dec_got = O.decode_angle_from_population_vector(O.readout(got.transpose(1, 0, 2)))
+    dec_ref = O.decode_angle_from_population_vector(O.readout(ref.transpose(1, 0, 2)))
+    diff = np.abs(np.angle(np.exp(1j * (dec_got - dec_ref))))
+    assert diff.max() <= TRAJ_TOL * 2 * np.pi, f"decoded angle error {diff.max()} rad"
+    # and the network does integrate: the reference's own sanity bound on the loss
+    assert O.cosine_similarity_loss(O.readout(got.transpose(1, 0, 2)), p["angle"]) < 0.5
+
+
+@pytest.mark.parametrize("case", CASES, ids=[c[0] for c in CASES])
+def test_backward_weight_gradients(case, gpu_device):
+    name, B, T, k, N, act, J0, J1, action = case
+    print(f"[case] bwd {name} B={B} T={T} k={k} N={N} {act}", flush=True)
+    p = make_problem(200, B, T, k, N, action=action)
+    hist, Wa, Wo = _run_op(p, J0, J1, act, gpu_device)
+    hist.backward(_dev(p["G"], gpu_device))
+    torch.cuda.synchronize()
+    ref_hist, _ = O.forward_dense(p["A"], p["Wa"], J0, J1, p["Wo"], p["r0"], 0.15, act)
+    ref = O.backward_dense(p["G"], p["A"], p["Wa"], J0, J1, p["Wo"], ref_hist, p["r0"], 0.15, act)
+    gWo, gWa = Wo.grad.cpu().numpy(), Wa.grad.cpu().numpy()
+    assert np.isfinite(gWo).all() and np.isfinite(gWa).all()
+    assert np.abs(ref["grad_Wo"]).max() > 0, "degenerate case: the reference gradient is identically zero"
+    assert O.cosine(gWo, ref["grad_Wo"]) >= GRAD_COS
+    assert O.max_rel_err(gWo, ref["grad_Wo"]) <= GRAD_TOL
+    used = [c for c in range(k) if np.abs(p["A"][..., c]).max() > 0]
+    for c in range(k):
+        if c in used:
+            assert O.cosine(gWa[c], ref["grad_Wa"][c]) >= GRAD_COS, f"Wa[{c}]"
+            assert O.max_rel_err(gWa[c], ref["grad_Wa"][c]) <= GRAD_TOL, f"Wa[{c}]"
+        else:                       # an action channel that is identically zero has an exactly zero gradient
+            assert np.abs(gWa[c]).max() == 0.0
+
+
+@pytest.mark.parametrize("case", [CASES[0], CASES[3], CASES[5], CASES[9]], ids=lambda c: c[0])
+def test_backward_without_saved_buffer_rebuilds_it(case, gpu_device):
+    """bwd_cuda.bwd called the way the reference operator calls it (dummy re_history, reference workspaces
+    absent): F'(re) is rebuilt from bump_history and the result equals the saved-buffer path bit for bit."""
+    from rnn_train_ring_attractor_amd import bwd_cuda
+    name, B, T, k, N, act, J0, J1, action = case
+    print(f"[case] bwd-rebuild {name}", flush=True)
+    p = make_problem(200, B, T, k, N, action=action)
+    hist, Wa, Wo = _run_op(p, J0, J1, act, gpu_device)
+    G = _dev(p["G"], gpu_device)
+    hist.backward(G)
+    gWa = torch.zeros_like(Wa)
+    gWo = torch.zeros_like(Wo)
+    g0 = torch.zeros(B, N, device=gpu_device)
+    dummy = torch.empty(1, device=gpu_device, dtype=torch.bfloat16)
+    bwd_cuda.bwd(grad_output=G, A=_dev(p["A"], gpu_device), Wa=Wa.detach(), J0=J0, J1=J1, Wo=Wo.detach(),
+                 bump_history=hist.detach(), re_history=dummy, r_init=_dev(p["r0"], gpu_device),
+                 grad_Wa=gWa, grad_Wo=gWo, alpha=0.15, activation_type=ACTS[act], grad_r_init=g0)
+    torch.cuda.synchronize()
+    assert torch.equal(gWa, Wa.grad) and torch.equal(gWo, Wo.grad)
+    ref_hist, _ = O.forward_dense(p["A"], p["Wa"], J0, J1, p["Wo"], p["r0"], 0.15, act)
+    ref = O.backward_dense(p["G"], p["A"], p["Wa"], J0, J1, p["Wo"], ref_hist, p["r0"], 0.15, act)
+    assert O.cosine(g0.cpu().numpy(), ref["grad_r_init"]) >= GRAD_COS
+    assert O.max_rel_err(g0.cpu().numpy(), ref["grad_r_init"]) <= GRAD_TOL
+
+
+def test_gradients_accumulate_and_are_deterministic(gpu_device):
+    from rnn_train_ring_attractor_amd import bwd_cuda
+    B, T, k, N = 48, 20, 2, 256
+    p = make_problem(300, B, T, k, N)
+    hist, Wa, Wo = _run_op(p, -0.1, 0.1, "gelu", gpu_device)
+    G = _dev(p["G"], gpu_device)
+    hist.backward(G)
+    outs = []
+    for _ in range(2):
+        gWa = torch.ones_like(Wa)          # pre-filled: the call must ADD to it
+        gWo = torch.full_like(Wo, 2.0)
+        bwd_cuda.bwd(grad_output=G, A=_dev(p["A"], gpu_device), Wa=Wa.detach(), J0=-0.1, J1=0.1, Wo=Wo.detach(),
+                     bump_history=hist.detach(), r_init=_dev(p["r0"], gpu_device), grad_Wa=gWa, grad_Wo=gWo,
+                     alpha=0.15, activation_type=1)
+        outs.append((gWa, gWo))
+    torch.cuda.synchronize()
+    assert torch.equal(outs[0][0], outs[1][0]) and torch.equal(outs[0][1], outs[1][1])     # bitwise repeatable
+    torch.testing.assert_close(outs[0][0] - 1.0, Wa.grad, rtol=1e-4, atol=1e-5)
+    torch.testing.assert_close(outs[0][1] - 2.0, Wo.grad, rtol=1e-4, atol=1e-5)
+
+
+def test_alpha_zero_and_zero_weights_closed_forms(gpu_device):
+    from rnn_train_ring_attractor_amd import ring_rnn_cuda_func
+    B, T, k, N = 32, 6, 2, 128
+    p = make_problem(400, B, T, k, N)
+    A, r0 = _dev(p["A"], gpu_device), _dev(p["r0"], gpu_device)
+    Wa, Wo = _dev(p["Wa"], gpu_device), _dev(p["Wo"], gpu_device)
+    frozen = ring_rnn_cuda_func(A, Wa, -0.1, 0.1, Wo, r0, 0.0, "gelu")
+    assert torch.equal(frozen, r0.expand(T, B, N))
+    decay = ring_rnn_cuda_func(A, torch.zeros_like(Wa), 0.0, 1.0, torch.zeros_like(Wo), r0, 0.15, "tanh")
+    for t in range(T):
+        torch.testing.assert_close(decay[t], r0 * 0.85 ** (t + 1), rtol=1e-5, atol=1e-8)
