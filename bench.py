@@ -1,0 +1,147 @@
+"""Headline benchmark: fused forward + BPTT of the ring-attractor time loop on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu]
+
+One "step" = one forward + one backward of the operator over one synthetic batch at
+N=256, B=4096, T=120, k=2, gelu (inputs resident in HBM before the timed region).
+Prints ONE JSON line: sample-steps/s (B*T per fwd+bwd), the roofline of the slowest kernel from
+HIP events recorded on the launch stream inside the timed region, and a host-CPU baseline (torch
+port of the reference's per-sample-W_eff formulation) on a bounded sample of the same workload.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_BF16_TFLOPS = 2500.0      # MI355X dense bf16 MFMA, TFLOP/s
+PEAK_HBM_GBS = 8000.0          # MI355X HBM3E, GB/s
+
+WORKLOADS = {
+    # BASELINE config 2 (headline)
+    "train_n256_b4096_t120_gelu": dict(N=256, B=4096, T=120, k=2, act="gelu", J0=-1.0 / 256, J1=1.0),
+}
+
+
+def make_inputs(cfg, device):
+    """Seeded synthetic inputs of the named shape: weights ~ N(0,1/N), av trials (10 % leading zeros,
+    U(-0.1*pi,0.1*pi), zero ratio in {0.2,0.5,0.8}), L/R = relu(-/+av), Gaussian bump at the initial angle."""
+    import numpy as np
+    import torch
+    from tests.ring_cases import make_problem
+    p = make_problem(42, cfg["B"], cfg["T"], cfg["k"], cfg["N"])
+    t = lambda x: torch.tensor(np.ascontiguousarray(x), device=device)
+    return p, dict(A=t(p["A"]), Wa=t(p["Wa"]), Wo=t(p["Wo"]), r0=t(p["r0"]), angle=t(p["angle"]))
+
+
+def loss_head_grad(hist, angle):
+    """d(loss pair)/d(bump_history) with torch ops on the GPU, once, outside the timed region."""
+    import torch
+    from oracle import torch_port as TP
+    h = hist.detach().clone().requires_grad_(True)
+    TP.loss_pair(h, angle).backward()
+    return h.grad.contiguous()
+
+
+def cpu_baseline(cfg, sample_B, iters=3):
+    """Torch port of the reference formulation (W_eff per sample + bmm + autograd), fp32, host cores."""
+    import torch
+    from oracle import torch_port as TP
+    from tests.ring_cases import make_problem
+    threads = int(os.environ.get("OMP_NUM_THREADS", "0")) or min(16, os.cpu_count() or 1)
+    torch.set_num_threads(threads)
+    p = make_problem(42, sample_B, cfg["T"], cfg["k"], cfg["N"])
+    t = lambda x: torch.tensor(x)
+    args = (t(p["A"]), t(p["Wa"]), cfg["J0"], cfg["J1"], t(p["Wo"]), t(p["r0"]), 0.15, cfg["act"])
+    G = t(p["G"])
+    TP.fwd_bwd_autograd(*args, grad_output=G)          # warm-up
+    ts = []
+    for _ in range(iters):
+        t0 = time.perf_counter()
+        TP.fwd_bwd_autograd(*args, grad_output=G)
+        ts.append(time.perf_counter() - t0)
+    mean = sum(ts) / len(ts)
+    return {"value": sample_B * cfg["T"] / mean, "unit": "sample-steps/s", "cores": threads, "kind": "port",
+            "sample": f"N={cfg['N']} B={sample_B} T={cfg['T']} {cfg['act']} fp32, {iters} fwd+bwd iters, "
+                      f"{mean * 1e3:.0f} ms each (full B={cfg['B']} would need B*N^2*4*T bytes of saved W_eff)"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="train_n256_b4096_t120_gelu", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-cpu", action="store_true", help="skip the host-CPU baseline leg")
+    ap.add_argument("--cpu-sample-batch", type=int, default=64)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on exactly one GPU (the batch shards trivially; see DESIGN.md); use --gpus 1")
+
+    import torch
+    from rnn_train_ring_attractor_amd import _lib, ring_rnn_cuda_func
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible; the HIP path has no CPU fallback")
+    dev = torch.device("cuda:0")
+    cfg = WORKLOADS[args.workload]
+    N, B, T, k = cfg["N"], cfg["B"], cfg["T"], cfg["k"]
+    _, x = make_inputs(cfg, dev)
+    Wa = x["Wa"].requires_grad_(True)
+    Wo = x["Wo"].requires_grad_(True)
+
+    def fwd():
+        return ring_rnn_cuda_func(x["A"], Wa, cfg["J0"], cfg["J1"], Wo, x["r0"], 0.15, cfg["act"])
+
+    G = loss_head_grad(fwd(), x["angle"])
+
+    def step():
+        Wa.grad = None
+        Wo.grad = None
+        fwd().backward(G)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    _lib.profile_enable(True)
+    _lib.profile_read()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    prof = _lib.profile_read()
+    _lib.profile_enable(False)
+
+    ms_per_step = dt / args.steps * 1e3
+    value = B * T / (dt / args.steps)
+    flops_third = 6.0 * N * N * B * T                      # per kernel: fwd, bptt and dW each contract 2*3*N^2 per sample-step
+    kern = {kname: (ms / max(cnt, 1)) for kname, (ms, cnt) in prof.items() if cnt}
+    dominant = max(("fwd", "bptt", "dw"), key=lambda n_: kern.get(n_, 0.0))
+    dom_ms = kern[dominant]
+    achieved = flops_third / (dom_ms * 1e-3) / 1e12
+    bytes_per_ss = 12 * N + 8 * k                           # fp32 history write + r_prev/grad_output reads + A
+    out = {
+        "metric": "fwd+bwd sample-steps/s (B*T/s) at N=256,B=4096,T=120; % bf16 MFMA peak",
+        "value": value, "unit": "sample-steps/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": args.workload, "N": N, "B": B, "T": T, "a_dim": k, "activation": cfg["act"],
+                   "grad_output": "gradient of the cos-sim + 0.2*bump-amplitude loss pair, precomputed"},
+        "pct_bf16_mfma_peak_fwd_bwd": 100.0 * (18.0 * N * N * value) / (PEAK_BF16_TFLOPS * 1e12),
+        "algorithmic_hbm_gbs_fwd_bwd": bytes_per_ss * value / 1e9,
+        "roofline": {"bound": "mfma", "kernel": dominant, "achieved": achieved, "peak": PEAK_BF16_TFLOPS,
+                     "unit": "TFLOP/s", "frac": achieved / PEAK_BF16_TFLOPS, "traffic": None,
+                     "flops_per_launch": flops_third, "avg_launch_ms": dom_ms},
+        "kernel_ms": kern,
+    }
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline(cfg, args.cpu_sample_batch)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -84,6 +84,20 @@ RINGATTR_API int ringattr_bwd(const void* grad_output, const void* A, const void
                  const void* saved, void* grad_A, void* grad_r_init,
                  void* workspace, size_t workspace_bytes, void* stream);
 
+/* Per-kernel timing for benchmarks; no counterpart in the reference.  While enabled, every kernel
+ * launch is bracketed by two HIP events recorded on the launch stream.  ringattr_profile_read waits
+ * for the recorded events, adds their durations into ms[RINGATTR_NUM_KERNELS] and the launch counts
+ * into launches[RINGATTR_NUM_KERNELS] (both caller arrays, not cleared first) and forgets them. */
+#define RINGATTR_NUM_KERNELS 6
+#define RINGATTR_K_PACK 0
+#define RINGATTR_K_FWD 1
+#define RINGATTR_K_REBUILD 2
+#define RINGATTR_K_BPTT 3
+#define RINGATTR_K_DW 4
+#define RINGATTR_K_DW_REDUCE 5
+RINGATTR_API int ringattr_profile_enable(int on);
+RINGATTR_API int ringattr_profile_read(double* ms, long long* launches);
+
 /* Reference-signature entry points, argument for argument (cpp/fwd.cu:21-35,
  * cpp/bwd.cu:4-30).  They run on the null stream, obtain their scratch with
  * hipMalloc/hipFree around the call, ignore the reference's workspace pointers

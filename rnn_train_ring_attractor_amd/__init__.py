@@ -1,4 +1,14 @@
 """MI355X-native leaky ring-attractor RNN time loop (forward + BPTT) behind the operator API of
 chongxi/rnn_train_ring_attractor's cpp/ring_rnn_cuda.py."""
-from .ring_rnn_cuda import RingRnnCudaFunc, ring_rnn_cuda_func  # noqa: F401
-from .rnn_cuda import bwd_cuda, fwd_cuda  # noqa: F401
+
+_EXPORTS = {
+    "ring_rnn_cuda_func": "ring_rnn_cuda", "RingRnnCudaFunc": "ring_rnn_cuda",
+    "fwd_cuda": "rnn_cuda", "bwd_cuda": "rnn_cuda",
+}
+
+
+def __getattr__(name):          # resolved on first use so `python -m ...build` does not import torch
+    if name in _EXPORTS:
+        import importlib
+        return getattr(importlib.import_module(f"{__name__}.{_EXPORTS[name]}"), name)
+    raise AttributeError(name)

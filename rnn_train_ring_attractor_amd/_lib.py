@@ -32,6 +32,8 @@ PROTOTYPES = {
     "ringattr_bwd": (c_int, [c_void_p, c_void_p, c_void_p, c_float, c_float, c_void_p, c_void_p, c_void_p,
                              c_void_p, c_void_p, c_float, c_int, c_int, c_int, c_int, c_int,
                              c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
+    "ringattr_profile_enable": (c_int, [c_int]),
+    "ringattr_profile_read": (c_int, [ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_longlong)]),
     "fwd_cuda": (None, [c_void_p, c_void_p, c_float, c_float, c_void_p, c_void_p, c_void_p, c_float,
                         c_int, c_int, c_int, c_int, c_int]),
     "bwd_cuda": (None, [c_void_p, c_void_p, c_void_p, c_float, c_float, c_void_p, c_void_p, c_void_p, c_void_p,
@@ -75,3 +77,19 @@ def check(rc: int) -> None:
     if rc == 1:
         raise ValueError(msg)
     raise RuntimeError(msg)
+
+
+KERNEL_NAMES = ("pack_weights", "fwd", "rebuild_saved", "bptt", "dw", "dw_reduce")
+
+
+def profile_enable(on: bool) -> None:
+    check(load().ringattr_profile_enable(1 if on else 0))
+
+
+def profile_read():
+    """Returns {kernel name: (total ms, launches)} of the launches recorded since the last read."""
+    n = len(KERNEL_NAMES)
+    ms = (ctypes.c_double * n)()
+    cnt = (ctypes.c_longlong * n)()
+    check(load().ringattr_profile_read(ms, cnt))
+    return {KERNEL_NAMES[i]: (ms[i], cnt[i]) for i in range(n)}

@@ -408,6 +408,64 @@ __global__ __launch_bounds__(256) void ring_dw_reduce_kernel(RingDwArgs p, int N
 }
 
 // ------------------------------------------------------------------------------------------------
+// Optional per-launch HIP event bracketing (benchmarks only).
+// ------------------------------------------------------------------------------------------------
+#include <mutex>
+#include <vector>
+namespace {
+struct ProfRec { hipEvent_t a, b; int id; };
+std::mutex g_prof_mu;
+std::vector<ProfRec> g_prof;
+bool g_prof_on = false;
+
+struct ProfScope {
+  hipStream_t st;
+  ProfRec rec;
+  bool active;
+  ProfScope(int id, hipStream_t s) : st(s), active(false) {
+    if (!g_prof_on) return;
+    if (hipEventCreate(&rec.a) != hipSuccess) return;
+    if (hipEventCreate(&rec.b) != hipSuccess) { (void)hipEventDestroy(rec.a); return; }
+    rec.id = id;
+    active = true;
+    (void)hipEventRecord(rec.a, st);
+  }
+  ~ProfScope() {
+    if (!active) return;
+    (void)hipEventRecord(rec.b, st);
+    std::lock_guard<std::mutex> lk(g_prof_mu);
+    g_prof.push_back(rec);
+  }
+};
+}  // namespace
+
+void ring_profile_set(bool on) { g_prof_on = on; }
+bool ring_profile_on() { return g_prof_on; }
+
+hipError_t ring_profile_collect(double* ms, long long* launches) {
+  std::vector<ProfRec> recs;
+  {
+    std::lock_guard<std::mutex> lk(g_prof_mu);
+    recs.swap(g_prof);
+  }
+  hipError_t first = hipSuccess;
+  for (auto& r : recs) {
+    float t = 0.f;
+    hipError_t e = hipEventSynchronize(r.b);
+    if (e == hipSuccess) e = hipEventElapsedTime(&t, r.a, r.b);
+    if (e == hipSuccess) {
+      ms[r.id] += t;
+      launches[r.id] += 1;
+    } else if (first == hipSuccess) {
+      first = e;
+    }
+    (void)hipEventDestroy(r.a);
+    (void)hipEventDestroy(r.b);
+  }
+  return first;
+}
+
+// ------------------------------------------------------------------------------------------------
 // Launchers (host).  NC is chosen by the caller as the smallest of {1,2,4,8} with 64*NC >= N.
 // ------------------------------------------------------------------------------------------------
 #define RING_DISPATCH_NC(NCv, CALL)                 \
@@ -423,22 +481,26 @@ hipError_t ring_launch_pack(const float* Wo, const float* Wa, void* out, int N, 
                             hipStream_t st) {
   const size_t total = (size_t)(1 + k) * 4 * NC * 2 * NC * 64;
   const int blocks = (int)((total + 255) / 256 < 4096 ? (total + 255) / 256 : 4096);
+  ProfScope prof(0, st);
   hipLaunchKernelGGL(ring_pack_weights_kernel, dim3(blocks), dim3(256), 0, st, Wo, Wa, (bf16x8*)out, N, k, NC,
                      transposed);
   return hipGetLastError();
 }
 
 hipError_t ring_launch_fwd(const RingFwdArgs& a, int NCv, hipStream_t st) {
+  ProfScope prof(1, st);
   RING_DISPATCH_NC(NCv, hipLaunchKernelGGL(ring_fwd_kernel<NC>, dim3(a.nbt), dim3(256), 0, st, a));
   return hipGetLastError();
 }
 
 hipError_t ring_launch_rebuild(const RingFwdArgs& a, int NCv, hipStream_t st) {
+  ProfScope prof(2, st);
   RING_DISPATCH_NC(NCv, hipLaunchKernelGGL(ring_rebuild_saved_kernel<NC>, dim3(a.nbt, a.T), dim3(256), 0, st, a));
   return hipGetLastError();
 }
 
 hipError_t ring_launch_bptt(const RingBpttArgs& a, int NCv, hipStream_t st) {
+  ProfScope prof(3, st);
   RING_DISPATCH_NC(NCv, hipLaunchKernelGGL(ring_bptt_kernel<NC>, dim3(a.nbt), dim3(256), 0, st, a));
   return hipGetLastError();
 }
@@ -448,14 +510,19 @@ hipError_t ring_launch_dw(const RingDwArgs& a, int NCv, hipStream_t st) {
   const int TJ = NCv == 1 ? 4 : 8;
   const long waves = (long)(NT / 2) * (NT / TJ) * ((a.k + 3) / 3) * a.nz;
   const int blocks = (int)((waves + 3) / 4);
+  hipError_t e;
+  {
+  ProfScope prof(4, st);
   if (NCv == 1) {
     hipLaunchKernelGGL((ring_dw_kernel<1, 4>), dim3(blocks), dim3(256), 0, st, a);
   } else {
     RING_DISPATCH_NC(NCv, if constexpr (NC >= 2) hipLaunchKernelGGL((ring_dw_kernel<NC, 8>), dim3(blocks), dim3(256), 0, st, a));
   }
-  hipError_t e = hipGetLastError();
+  e = hipGetLastError();
+  }
   if (e != hipSuccess) return e;
   const size_t per_z = (size_t)(a.k + 1) * NT * NT * 64;
+  ProfScope prof(5, st);
   hipLaunchKernelGGL(ring_dw_reduce_kernel, dim3((unsigned)((per_z + 255) / 256)), dim3(256), 0, st, a, NCv);
   return hipGetLastError();
 }

@@ -44,3 +44,8 @@ hipError_t ring_launch_fwd(const RingFwdArgs& a, int NC, hipStream_t st);
 hipError_t ring_launch_rebuild(const RingFwdArgs& a, int NC, hipStream_t st);
 hipError_t ring_launch_bptt(const RingBpttArgs& a, int NC, hipStream_t st);
 hipError_t ring_launch_dw(const RingDwArgs& a, int NC, hipStream_t st);
+
+// Optional event bracketing of launches (benchmark support).
+void ring_profile_set(bool on);
+bool ring_profile_on();
+hipError_t ring_profile_collect(double* ms, long long* launches);

@@ -248,6 +248,18 @@ int ringattr_bwd(const void* grad_output, const void* A, const void* Wa, float J
   return RINGATTR_OK;
 }
 
+int ringattr_profile_enable(int on) {
+  ring_profile_set(on != 0);
+  return RINGATTR_OK;
+}
+
+int ringattr_profile_read(double* ms, long long* launches) {
+  if (!ms || !launches) return fail(RINGATTR_ERR_INVALID, "ringattr_profile_read: null output array");
+  hipError_t e = ring_profile_collect(ms, launches);
+  if (e != hipSuccess) return hip_fail(e, "profile events");
+  return RINGATTR_OK;
+}
+
 void fwd_cuda(void* A, void* Wa, float J0, float J1, void* Wo, void* r_init, void* bump_history, float alpha, int N,
               int a_dim, int seq_len, int batch_size, int activation_type) {
   const size_t need = ringattr_fwd_workspace_bytes(N, a_dim, seq_len, batch_size);
