@@ -1,0 +1,80 @@
+"""Rounding-aware restatement: the dense-form recurrence and BPTT of ring_oracle.py with the HIP
+kernels' reduced-precision points made explicit (everything else stays fp64).
+
+TEST INFRASTRUCTURE ONLY.  It answers one question the fp64 oracle cannot: is a deviation from the
+fp64 result explained by rounding the MFMA operands to bf16 (expected, bounded by the tolerances),
+or by a defect in a kernel?  A kernel is compared against this model at a tolerance ~10x tighter
+than against the fp64 oracle.
+
+Rounding points (same math as ring_oracle.forward_dense / backward_dense, which cite the reference):
+  * weights [Wo|Wa]            -> bf16   (MFMA B operand)
+  * r_prev, g as contraction operands -> bf16 (MFMA A operand); the leak term, the J0 row sums and
+    the state carried between steps stay unrounded
+  * F'(re) kept for the backward -> fp16
+  * A_c * g in the weight-gradient contraction -> bf16
+Pinned by tests/test_oracle_bf16.py: with rounding switched off it reproduces ring_oracle exactly.
+"""
+from __future__ import annotations
+
+import numpy as np
+
+from . import ring_oracle as O
+
+
+def round_bf16(x):
+    """Round-to-nearest-even to bfloat16, returned as float64."""
+    u = np.asarray(x, np.float32).view(np.uint32).astype(np.uint64)
+    u = (u + 0x7FFF + ((u >> 16) & 1)) & 0xFFFF0000
+    return u.astype(np.uint32).view(np.float32).astype(np.float64)
+
+
+def round_fp16(x):
+    return np.asarray(x, np.float64).astype(np.float16).astype(np.float64)
+
+
+def _identity(x):
+    return np.asarray(x, np.float64)
+
+
+def forward_backward(A, Wa, J0, J1, Wo, r_init, alpha, activation_name, grad_output=None, rounding=True):
+    """Returns dict(bump_history [T,B,N], and, when grad_output is given, grad_Wa, grad_Wo, grad_r_init)."""
+    rb16 = round_bf16 if rounding else _identity
+    rf16 = round_fp16 if rounding else _identity
+    A = np.asarray(A, np.float64)
+    Wa = np.asarray(Wa, np.float64)
+    Wo = np.asarray(Wo, np.float64)
+    r = np.array(r_init, np.float64)
+    B, T, k = A.shape
+    N = Wo.shape[0]
+    Wob, Wab = rb16(Wo), rb16(Wa)
+    hist = np.empty((T, B, N))
+    D = np.empty((T, B, N))
+    R = np.empty((T, B, N))
+    for t in range(T):
+        rb = rb16(r)
+        R[t] = rb
+        re = J0 * r.sum(axis=1, keepdims=True) + J1 * (rb @ Wob.T)
+        for c in range(k):
+            re = re + A[:, t, c:c + 1] * (rb @ Wab[c].T)
+        D[t] = rf16(O.activation_derivative(re, activation_name))
+        r = (1.0 - alpha) * r + alpha * O.activation(re, activation_name)
+        hist[t] = r
+    out = {"bump_history": hist}
+    if grad_output is None:
+        return out
+    G_out = np.asarray(grad_output, np.float64)
+    grad_Wo = np.zeros_like(Wo)
+    grad_Wa = np.zeros_like(Wa)
+    carry = np.zeros((B, N))
+    for t in range(T - 1, -1, -1):
+        G = G_out[t] + carry
+        g = alpha * D[t] * G
+        gb = rb16(g)
+        carry = (1.0 - alpha) * G + J0 * g.sum(axis=1, keepdims=True) + J1 * (gb @ Wob)
+        for c in range(k):
+            carry = carry + A[:, t, c:c + 1] * (gb @ Wab[c])
+        grad_Wo += J1 * (gb.T @ R[t])
+        for c in range(k):
+            grad_Wa[c] += rb16(A[:, t, c:c + 1] * gb).T @ R[t]
+    out.update(grad_Wo=grad_Wo, grad_Wa=grad_Wa, grad_r_init=carry)
+    return out

@@ -28,13 +28,25 @@ struct Tile {
   static constexpr int KG = KCH < 8 ? KCH : 8;  // chunks staged per register group
   static constexpr int NKG = KCH / KG;
   static constexpr int GW = (NC % 4 == 0) ? 4 : ((NC % 2 == 0) ? 2 : 1);  // LDS write granule
-  static constexpr int SLOTS = KCH * 64;        // 16-byte operand slots per LDS buffer
+  static constexpr int SLOTS = KCH * 4 * 17;    // 16-byte operand slots per LDS buffer (padded groups)
 };
+
+// Operand-buffer groups (one per (K chunk, q)) hold 16 row slots and are spaced 17 slots apart: the
+// 8-byte write-back of a wave then spreads over all banks (2-way, the minimum for 512 bytes) instead
+// of landing 8-way on the same ones.
+constexpr int XG = 17;
 
 // D = A(16x32 bf16) * B(32x16 bf16) + C(16x16 fp32).  Lane (q,n): A row n, B column n, both with
 // K slots 8q..8q+7; C/D rows 4q..4q+3 of column n.
 __device__ __forceinline__ f32x4 mfma16(bf16x8 a, bf16x8 b, f32x4 c) {
   return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+}
+
+// Workgroup barrier that orders LDS traffic only.  __syncthreads() also drains the vector-memory
+// counter, i.e. it would stall every time step on the HBM acknowledgement of that step's history
+// stores; the recurrence only exchanges data through LDS, so waiting for lgkmcnt is sufficient.
+__device__ __forceinline__ void lds_barrier() {
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 }
 
 // F(x) and F'(x).  gelu is the exact erf form (train/train_ring_attractor.py:16), its derivative
@@ -76,9 +88,9 @@ __device__ __forceinline__ float row16_sum(float v) {
   return v;
 }
 
-// LDS operand buffer: slot(kc,q,b) = (kc*4+q)*16 + b holds the 8 bf16 values
-// x[b][32kc+8q .. +7]; an MFMA A-operand read by lane (q,b) is slot(kc,q,b): the 64 lanes read
-// 1 KiB contiguous.  This writes the lane's [4 rows][NC neurons] fp32 values as bf16.
+// LDS operand buffer: slot(kc,q,b) = (kc*4+q)*XG + b holds the 8 bf16 values
+// x[b][32kc+8q .. +7]; an MFMA A-operand read by lane (q,b) is slot(kc,q,b): each group of 16 lanes
+// reads 256 contiguous bytes.  This writes the lane's [4 rows][NC neurons] fp32 values as bf16.
 template <int NC>
 __device__ __forceinline__ void write_operand(bf16x8* xb, const float (&v)[4][NC], int w, int q, int n) {
   constexpr int G = Tile<NC>::GW;
@@ -89,7 +101,7 @@ __device__ __forceinline__ void write_operand(bf16x8* xb, const float (&v)[4][NC
 #pragma unroll
     for (int c0 = 0; c0 < NC; c0 += G) {
       const int j = 16 * NC * w + NC * n + c0;
-      const int slot = (((j >> 5) * 4 + ((j >> 3) & 3)) * 16 + b);
+      const int slot = (((j >> 5) * 4 + ((j >> 3) & 3)) * XG + b);
       char* dst = base + slot * 16 + (j & 7) * 2;
       if constexpr (G == 4) {
         bf16x4 pk = {(__bf16)v[e][c0], (__bf16)v[e][c0 + 1], (__bf16)v[e][c0 + 2], (__bf16)v[e][c0 + 3]};

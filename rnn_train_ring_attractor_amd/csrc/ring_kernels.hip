@@ -74,7 +74,7 @@ __device__ __forceinline__ void gated_products(const bf16x8* __restrict__ xb, co
     for (int kg = 0; kg < TL::NKG; ++kg) {
       bf16x8 af[TL::KG];
 #pragma unroll
-      for (int u = 0; u < TL::KG; ++u) af[u] = xb[((kg * TL::KG + u) * 4 + q) * 16 + n];
+      for (int u = 0; u < TL::KG; ++u) af[u] = xb[((kg * TL::KG + u) * 4 + q) * XG + n];
       bf16x8 wf[2][TL::KG];
 #pragma unroll
       for (int u = 0; u < TL::KG; ++u) wf[0][u] = wm[(size_t)(0 * TL::KCH + kg * TL::KG + u) * 64];
@@ -143,7 +143,7 @@ __global__ __launch_bounds__(256) void ring_fwd_kernel(RingFwdArgs p) {
   write_operand<NC>(xbuf[0], r, w, q, n);
   publish_rowsum<NC>(psum[0], r, w, q, n);
   if (p.rfrag) side_store<NC, bf16x4, __bf16>(p.rfrag + side_offset<NC>(0, p.nbt, bt, w, lane), r);
-  __syncthreads();
+  lds_barrier();
 
   for (int t = 0; t < T; ++t) {
     const int cur = t & 1;
@@ -171,7 +171,7 @@ __global__ __launch_bounds__(256) void ring_fwd_kernel(RingFwdArgs p) {
       publish_rowsum<NC>(psum[cur ^ 1], r, w, q, n);
       if (p.rfrag) side_store<NC, bf16x4, __bf16>(p.rfrag + side_offset<NC>(t + 1, p.nbt, bt, w, lane), r);
     }
-    __syncthreads();
+    lds_barrier();
   }
 }
 
@@ -197,7 +197,7 @@ __global__ __launch_bounds__(256) void ring_rebuild_saved_kernel(RingFwdArgs p) 
   write_operand<NC>(xbuf, r, w, q, n);
   publish_rowsum<NC>(psum, r, w, q, n);
   side_store<NC, bf16x4, __bf16>(p.rfrag + side_offset<NC>(t, p.nbt, bt, w, lane), r);
-  __syncthreads();
+  lds_barrier();
 
   f32x4 acc[NC];
   gated_products<NC>(xbuf, (const bf16x8*)p.Wpack, p.A, p.k, T, B, t, b0, p.J1, w, lane, acc);
@@ -256,7 +256,7 @@ __global__ __launch_bounds__(256) void ring_bptt_kernel(RingBpttArgs p) {
     write_operand<NC>(xbuf[cur], g, w, q, n);
     publish_rowsum<NC>(psum[cur], g, w, q, n);
     side_store<NC, bf16x4, __bf16>(p.gfrag + side_offset<NC>(t, p.nbt, bt, w, lane), g);
-    __syncthreads();
+    lds_barrier();
 
     f32x4 acc[NC];
     gated_products<NC>(xbuf[cur], (const bf16x8*)p.Wpack, p.A, p.k, T, B, t, b0, p.J1, w, lane, acc);
@@ -410,6 +410,7 @@ __global__ __launch_bounds__(256) void ring_dw_reduce_kernel(RingDwArgs p, int N
 // ------------------------------------------------------------------------------------------------
 // Optional per-launch HIP event bracketing (benchmarks only).
 // ------------------------------------------------------------------------------------------------
+#include <stdlib.h>
 #include <mutex>
 #include <vector>
 namespace {
@@ -487,8 +488,16 @@ hipError_t ring_launch_pack(const float* Wo, const float* Wa, void* out, int N, 
   return hipGetLastError();
 }
 
+// RINGATTR_STREAMING=1 forces the generic weight-streaming kernels (used by tests to cross-check).
+static bool use_resident(int N, int k) {
+  if (!ring_res256_applicable(N, k)) return false;
+  const char* v = getenv("RINGATTR_STREAMING");
+  return !(v && v[0] == '1');
+}
+
 hipError_t ring_launch_fwd(const RingFwdArgs& a, int NCv, hipStream_t st) {
   ProfScope prof(1, st);
+  if (use_resident(a.N, a.k)) return ring_launch_fwd_res256(a, st);
   RING_DISPATCH_NC(NCv, hipLaunchKernelGGL(ring_fwd_kernel<NC>, dim3(a.nbt), dim3(256), 0, st, a));
   return hipGetLastError();
 }
@@ -501,6 +510,7 @@ hipError_t ring_launch_rebuild(const RingFwdArgs& a, int NCv, hipStream_t st) {
 
 hipError_t ring_launch_bptt(const RingBpttArgs& a, int NCv, hipStream_t st) {
   ProfScope prof(3, st);
+  if (use_resident(a.N, a.k)) return ring_launch_bptt_res256(a, st);
   RING_DISPATCH_NC(NCv, hipLaunchKernelGGL(ring_bptt_kernel<NC>, dim3(a.nbt), dim3(256), 0, st, a));
   return hipGetLastError();
 }
@@ -513,7 +523,9 @@ hipError_t ring_launch_dw(const RingDwArgs& a, int NCv, hipStream_t st) {
   hipError_t e;
   {
   ProfScope prof(4, st);
-  if (NCv == 1) {
+  if (ring_dw_tiled_applicable(NCv)) {
+    (void)ring_launch_dw_tiled(a, NCv, st);
+  } else if (NCv == 1) {
     hipLaunchKernelGGL((ring_dw_kernel<1, 4>), dim3(blocks), dim3(256), 0, st, a);
   } else {
     RING_DISPATCH_NC(NCv, if constexpr (NC >= 2) hipLaunchKernelGGL((ring_dw_kernel<NC, 8>), dim3(blocks), dim3(256), 0, st, a));

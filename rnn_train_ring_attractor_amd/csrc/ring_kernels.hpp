@@ -45,6 +45,16 @@ hipError_t ring_launch_rebuild(const RingFwdArgs& a, int NC, hipStream_t st);
 hipError_t ring_launch_bptt(const RingBpttArgs& a, int NC, hipStream_t st);
 hipError_t ring_launch_dw(const RingDwArgs& a, int NC, hipStream_t st);
 
+// Weight-resident variants for 128 < N <= 256, a_dim == 2 (ring_res256.hip).
+bool ring_res256_applicable(int N, int k);
+hipError_t ring_launch_fwd_res256(const RingFwdArgs& a, hipStream_t st);
+hipError_t ring_launch_bptt_res256(const RingBpttArgs& a, hipStream_t st);
+
+// LDS-tiled weight-gradient contraction for NC in {4, 8} (ring_dw.hip).
+bool ring_dw_tiled_applicable(int NC);
+int ring_dw_tiled_nz(int NC, int k, long nchunk);
+hipError_t ring_launch_dw_tiled(const RingDwArgs& a, int NC, hipStream_t st);
+
 // Optional event bracketing of launches (benchmark support).
 void ring_profile_set(bool on);
 bool ring_profile_on();

@@ -60,7 +60,7 @@ int make_geo(int N, int k, int T, int B, Geo& g) {
   if (nz > 128) nz = 128;
   if (nz > nchunk) nz = nchunk;
   if (nz < 1) nz = 1;
-  g.nz = (int)nz;
+  g.nz = ring_dw_tiled_applicable(nc) ? ring_dw_tiled_nz(nc, k, nchunk) : (int)nz;
   g.partial_bytes = align_up((size_t)g.nz * (1 + k) * g.NPAD * g.NPAD * 4);
   return RINGATTR_OK;
 }
