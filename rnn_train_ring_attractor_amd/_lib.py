@@ -43,7 +43,8 @@ PROTOTYPES = {
 
 
 def library_path() -> str:
-    return _build.LIB_PATH
+    """In-tree library, or the file named by RINGATTR_LIB (to try an experimental build)."""
+    return os.environ.get("RINGATTR_LIB") or _build.LIB_PATH
 
 
 def load():

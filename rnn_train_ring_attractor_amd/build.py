@@ -32,19 +32,19 @@ def hipcc_path() -> str:
     raise RuntimeError("hipcc not found (set HIPCC or put /opt/rocm/bin on PATH)")
 
 
-def build_library(verbose: bool = False, extra_flags=()) -> str:
+def build_library(verbose: bool = False, extra_flags=(), out_path: str = LIB_PATH) -> str:
     """Compile every HIP source into libringattr.so; raises on any compiler error."""
     cmd = [hipcc_path(), *HIPCC_FLAGS, *extra_flags, f"-I{INCLUDE}", f"-I{CSRC}",
-           *[os.path.join(CSRC, s) for s in SOURCES], "-o", LIB_PATH + ".tmp"]
+           *[os.path.join(CSRC, s) for s in SOURCES], "-o", out_path + ".tmp"]
     proc = subprocess.run(cmd, capture_output=True, text=True)
     noise = "is not a recognized feature for this target"
     log = "\n".join(l for l in (proc.stdout + proc.stderr).splitlines() if noise not in l)
     if proc.returncode != 0:
         raise RuntimeError("hipcc failed:\n" + " ".join(cmd) + "\n" + log)
-    os.replace(LIB_PATH + ".tmp", LIB_PATH)
+    os.replace(out_path + ".tmp", out_path)
     if verbose and log.strip():
         print(log)
-    return LIB_PATH
+    return out_path
 
 
 if __name__ == "__main__":

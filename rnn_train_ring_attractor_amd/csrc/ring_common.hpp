@@ -116,10 +116,9 @@ __device__ __forceinline__ void write_operand(bf16x8* xb, const float (&v)[4][NC
   }
 }
 
-// Side buffers (saved F', bf16 operand copies of r_prev and g) use the private tile order
-//   S[t][bt][w][lane][c][e],  element = X[t][16*bt + 4q + e][16*NC*w + NC*n + c]
-// so each lane moves 4*NC contiguous 2-byte values and the weight-gradient GEMM can load MFMA
-// fragments (8 samples of one neuron = rows 4q..4q+3 of two time steps) without a transpose.
+// Saved F' (fp16) uses the lane order of the recurrence kernels,
+//   S[t][bt][w][lane][c][e],  element = X[t][16*bt + 4q + e][16*NC*w + NC*n + c],
+// so the forward writes and the BPTT reads 8*NC contiguous bytes per lane.
 template <int NC>
 __device__ __forceinline__ size_t side_offset(int t, int nbt, int bt, int w, int lane) {
   return ((((size_t)t * nbt + bt) * 4 + w) * 64 + lane) * (size_t)(4 * NC);
@@ -144,6 +143,35 @@ __device__ __forceinline__ void side_load_f16(const _Float16* src, float (&v)[4]
     v[2][c] = (float)pk[2];
     v[3][c] = (float)pk[3];
   }
+}
+
+// The bf16 operand copies of r_prev and g feed the weight-gradient GEMM, whose MFMA K index runs
+// over samples.  They are stored tile-major with two time steps paired,
+//   P[t/2][bt][tile][lane][t%2][e],  tile = w*NC + c,  16 bytes per (pair, bt, tile, lane),
+// i.e. exactly one MFMA operand fragment (K slot 8q + 4*(t%2) + e) per lane: a column tile of a K
+// chunk is 1 KiB contiguous and goes global -> LDS -> MFMA without any transpose or repacking.
+template <int NC>
+__device__ __forceinline__ size_t pair_offset(int t, int nbt, int bt, int tile, int lane) {
+  return (((((size_t)(t >> 1) * nbt + bt) * (4 * NC) + tile) * 64 + lane) * 2 + (t & 1)) * 4;
+}
+
+template <int NC>
+__device__ __forceinline__ void pair_store(__bf16* base, int t, int nbt, int bt, int w, int lane, const float (&v)[4][NC]) {
+#pragma unroll
+  for (int c = 0; c < NC; ++c) {
+    bf16x4 pk = {(__bf16)v[0][c], (__bf16)v[1][c], (__bf16)v[2][c], (__bf16)v[3][c]};
+    *reinterpret_cast<bf16x4*>(base + pair_offset<NC>(t, nbt, bt, w * NC + c, lane)) = pk;
+  }
+}
+
+// With an odd sequence length the second half of the last pair has no time step; the writer of
+// the buffer zeroes it so that readers need no special case.
+template <int NC>
+__device__ __forceinline__ void pair_zero_tail(__bf16* base, int T, int nbt, int bt, int w, int lane) {
+  if ((T & 1) == 0) return;
+  const bf16x4 z = {(__bf16)0.f, (__bf16)0.f, (__bf16)0.f, (__bf16)0.f};
+#pragma unroll
+  for (int c = 0; c < NC; ++c) *reinterpret_cast<bf16x4*>(base + pair_offset<NC>(T, nbt, bt, w * NC + c, lane)) = z;
 }
 
 // Masked fp32 [rows][N] <-> lane registers.  slab points at row 0 of a [B][N] matrix.

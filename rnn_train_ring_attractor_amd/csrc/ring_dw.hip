@@ -2,86 +2,56 @@
 //
 //   dW_mm[i][j] = sum over samples (b,t) of coef_mm(b,t) * g[t,b,i] * r_prev[t,b,j]
 //
-// Work decomposition: a workgroup (4 waves) owns a 64 (i) x 128 (j) output tile of up to three
-// matrices over one K split; wave v owns row tile v of the block (16 neurons) against all eight
-// column tiles.  A K chunk is 16 batch rows x 2 time steps (32 samples, one MFMA K).  The bf16
-// operands stream from the tile-ordered side buffers through a double-buffered LDS stage laid out
-// fragment-major, so every MFMA operand is one conflict-free ds_read_b128; the action gates of the
-// chunk are staged next to them.  Two workgroups fit a CU (2 waves per SIMD) and hide each other's
-// load latency.  Partials are written once per workgroup; a fixed-order reduction follows.
+// Work decomposition: a workgroup (8 waves, 2 per SIMD) owns a 128 (i) x 128 (j) output tile of up to
+// three matrices over one K split; wave v owns row tiles 2*(v/2), 2*(v/2)+1 against column tiles
+// 4*(v%2) .. +3 (24 MFMAs per 6 operand reads: the LDS pipe, shared by the CU, stays under the MFMA
+// time).  A K chunk is 16 batch rows x 2 time steps (32 samples, one MFMA K).  The paired
+// tile-major operand buffers hold every tile of a chunk as 1 KiB of ready-made MFMA fragments, so
+// the stage is a verbatim copy: global -> registers (DW_DEPTH chunks in flight) -> double-buffered
+// LDS -> one conflict-free ds_read_b128 per operand.  The action gates of the chunk ride along.
+// Partials are written once per workgroup; a fixed-order reduction follows.
 #include "ring_common.hpp"
 #include "ring_kernels.hpp"
 
 namespace {
 
-constexpr int DW_TI = 4;   // row tiles per workgroup (64 neurons)
-constexpr int DW_TJ = 8;   // column tiles per workgroup (128 neurons)
+constexpr int DW_TI = 8;      // row tiles per workgroup (128 neurons)
+constexpr int DW_TJ = 8;      // column tiles per workgroup (128 neurons)
+constexpr int DW_DEPTH = 4;   // K chunks in flight in registers
 
-struct DwStage {           // one K chunk in flight in registers (global -> regs -> LDS)
-  f32x2 a[2];              // 2 x 8 bytes of g
-  f32x2 b[4];              // 4 x 8 bytes of r_prev
-  float cf;                // one gate value (threads 0..95)
+constexpr int DW_THREADS = 512;
+constexpr int DW_WI = 2, DW_WJ = 4;   // row / column tiles per wave
+
+struct DwStage {
+  f32x4 a;      // one 16-byte fragment of the g block (8 tiles x 64 lanes = 512 fragments)
+  f32x4 b;      // one of the r_prev block
+  float cf;     // one gate value (meaningful in threads 0..95)
 };
 
-// Unit x of an operand block: tau = time step within the chunk, then (record group, lane, c).
-template <int NC, int TT>
-__device__ __forceinline__ void unit_decode(int x, int it0, int& tau, int& tl, int& lane, int& w, int& c) {
-  constexpr int CB = NC < TT ? NC : TT;         // consecutive column tiles held in one lane record
-  tau = x / (TT * 64);
-  const int y = x % (TT * 64);
-  const int cl = y % CB;
-  lane = (y / CB) % 64;
-  const int wl = y / (CB * 64);
-  tl = wl * CB + cl;
-  const int it = it0 + tl;
-  w = it / NC;
-  c = it % NC;
-}
-
+// Branch-free on purpose: with no control flow around the loads the compiler can count the chunks in
+// flight and wait for exactly the oldest one (s_waitcnt vmcnt(n)) instead of draining all of them.
+// The chunk (bt, t0) is valid by construction of the caller's cursor; gate indices that fall outside the problem are clamped and zeroed.
 template <int NC>
-__device__ __forceinline__ void dw_fetch(const RingDwArgs& p, long ch, int it0, int jt0, int mg, int tid, DwStage& s) {
+__device__ __forceinline__ void dw_fetch(const RingDwArgs& p, int bt, int t0, int it0, int jt0, int mg, int tid, DwStage& s) {
   const int nbt = p.nbt, T = p.T;
-  const int bt = (int)(ch % nbt);
-  const int t0 = 2 * (int)(ch / nbt);
-  const f32x2 zero = {0.f, 0.f};
-#pragma unroll
-  for (int u = 0; u < 2; ++u) {
-    int tau, tl, lane, w, c;
-    unit_decode<NC, DW_TI>(tid + 256 * u, it0, tau, tl, lane, w, c);
-    const int t = t0 + tau;
-    s.a[u] = (t < T) ? *reinterpret_cast<const f32x2*>(p.gfrag + side_offset<NC>(t, nbt, bt, w, lane) + 4 * c) : zero;
-  }
-#pragma unroll
-  for (int u = 0; u < 4; ++u) {
-    int tau, tl, lane, w, c;
-    unit_decode<NC, DW_TJ>(tid + 256 * u, jt0, tau, tl, lane, w, c);
-    const int t = t0 + tau;
-    s.b[u] = (t < T) ? *reinterpret_cast<const f32x2*>(p.rfrag + side_offset<NC>(t, nbt, bt, w, lane) + 4 * c) : zero;
-  }
-  // gates: thread = (a, tau, row) for a < 3, tau < 2, row < 16
-  s.cf = 0.f;
-  if (tid < 96) {
-    const int a = tid / 32, tau = (tid / 16) & 1, row = tid & 15;
-    const int mm = 3 * mg + a, b = 16 * bt + row, t = t0 + tau;
-    if (mm >= 1 && mm <= p.k && b < p.B && t < T) s.cf = p.A[((size_t)b * T + t) * p.k + (mm - 1)];
-  }
+  const f32x4* ga = reinterpret_cast<const f32x4*>(p.gfrag + pair_offset<NC>(t0, nbt, bt, it0, 0));
+  const f32x4* rb = reinterpret_cast<const f32x4*>(p.rfrag + pair_offset<NC>(t0, nbt, bt, jt0, 0));
+  s.a = ga[tid];
+  s.b = rb[tid];
+  // gates: thread = (a, tau, row); threads past 96 load a clamped duplicate that is zeroed
+  const int a = tid >> 5, tau = (tid >> 4) & 1, row = tid & 15;
+  const int mm = 3 * mg + a, b = 16 * bt + row, t = t0 + tau;
+  const bool ok = (a < 3) && (mm >= 1) && (mm <= p.k) && (b < p.B) && (t < T);
+  const int mmc = mm < 1 ? 1 : (mm > p.k ? p.k : mm);
+  const int bc = b < p.B ? b : p.B - 1, tc = t < T ? t : T - 1;
+  const float v = p.A[((size_t)bc * T + tc) * p.k + (mmc - 1)];
+  s.cf = ok ? v : 0.f;
 }
 
-template <int NC>
-__device__ __forceinline__ void dw_publish(f32x2* la, f32x2* lb, float* lc, int tid, const DwStage& s) {
-#pragma unroll
-  for (int u = 0; u < 2; ++u) {
-    int tau, tl, lane, w, c;
-    unit_decode<NC, DW_TI>(tid + 256 * u, 0, tau, tl, lane, w, c);
-    la[(tl * 64 + lane) * 2 + tau] = s.a[u];
-  }
-#pragma unroll
-  for (int u = 0; u < 4; ++u) {
-    int tau, tl, lane, w, c;
-    unit_decode<NC, DW_TJ>(tid + 256 * u, 0, tau, tl, lane, w, c);
-    lb[(tl * 64 + lane) * 2 + tau] = s.b[u];
-  }
-  if (tid < 96) lc[tid] = s.cf;
+__device__ __forceinline__ void dw_publish(f32x4* la, f32x4* lb, float* lc, int tid, const DwStage& s) {
+  la[tid] = s.a;
+  lb[tid] = s.b;
+  lc[tid] = s.cf;
 }
 
 __device__ __forceinline__ bf16x8 gate_frag(bf16x8 x, f32x4 c0, f32x4 c1) {
@@ -96,17 +66,18 @@ __device__ __forceinline__ bf16x8 gate_frag(bf16x8 x, f32x4 c0, f32x4 c1) {
 
 }  // namespace
 
-template <int NC>
-__global__ __launch_bounds__(256, 2) void ring_dw_tiled_kernel(RingDwArgs p) {
+// NMAT = matrices of this workgroup's group (1..3); FIRST = the group starts with Wo (ungated).
+template <int NC, int NMAT, bool FIRST>
+__global__ __launch_bounds__(DW_THREADS) void ring_dw_tiled_kernel(RingDwArgs p, int mg) {
   constexpr int NT = 4 * NC;
   constexpr int NIB = NT / DW_TI, NJB = NT / DW_TJ;
-  __shared__ __attribute__((aligned(16))) f32x2 lds_a[2][DW_TI * 64 * 2];
-  __shared__ __attribute__((aligned(16))) f32x2 lds_b[2][DW_TJ * 64 * 2];
-  __shared__ __attribute__((aligned(16))) float lds_c[2][96];
+  __shared__ __attribute__((aligned(16))) f32x4 lds_a[2][DW_TI * 64];
+  __shared__ __attribute__((aligned(16))) f32x4 lds_b[2][DW_TJ * 64];
+  __shared__ __attribute__((aligned(16))) float lds_c[2][DW_THREADS];
 
   const int tid = threadIdx.x, wv = tid >> 6, lane = tid & 63, q = lane >> 4;
-  const int nmg = (p.k + 3) / 3;
-  const int tiles = NIB * NJB * nmg;
+  const int wi = wv >> 1, wj = wv & 1;
+  const int tiles = NIB * NJB;
   // keep the workgroups that share a K split on one XCD (workgroup ids are dealt round-robin to
   // the 8 XCDs) so the operand bytes they all read come out of that XCD's L2
   int z, tile;
@@ -121,60 +92,99 @@ __global__ __launch_bounds__(256, 2) void ring_dw_tiled_kernel(RingDwArgs p) {
       tile = bid % tiles;
     }
   }
-  const int ib = tile % NIB, jb = (tile / NIB) % NJB, mg = tile / (NIB * NJB);
+  const int ib = tile % NIB, jb = tile / NIB;
   const int it0 = ib * DW_TI, jt0 = jb * DW_TJ;
 
-  const long nchunk = (long)p.nbt * ((p.T + 1) / 2);
-  const long ch0 = nchunk * z / p.nz, ch1 = nchunk * (z + 1) / p.nz;
+  const int nchunk = p.nbt * ((p.T + 1) / 2);   // the host checked that this fits an int
+  const int ch0 = (int)((long)nchunk * z / p.nz), ch1 = (int)((long)nchunk * (z + 1) / p.nz);
 
-  f32x4 acc[3][DW_TJ];
+  f32x4 acc[NMAT][DW_WI][DW_WJ];
 #pragma unroll
-  for (int a = 0; a < 3; ++a)
+  for (int a = 0; a < NMAT; ++a)
 #pragma unroll
-    for (int u = 0; u < DW_TJ; ++u) acc[a][u] = f32x4{0.f, 0.f, 0.f, 0.f};
-  const int nmat = (p.k + 1 - 3 * mg) < 3 ? (p.k + 1 - 3 * mg) : 3;   // matrices of this group
+    for (int ii = 0; ii < DW_WI; ++ii)
+#pragma unroll
+      for (int u = 0; u < DW_WJ; ++u) acc[a][ii][u] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  DwStage st;
-  if (ch0 < ch1) {
-    dw_fetch<NC>(p, ch0, it0, jt0, mg, tid, st);
-    dw_publish<NC>(lds_a[0], lds_b[0], lds_c[0], tid, st);
-  }
-  __syncthreads();
-
-  for (long ch = ch0; ch < ch1; ++ch) {
-    const int cur = (int)((ch - ch0) & 1);
-    const bool more = ch + 1 < ch1;
-    if (more) dw_fetch<NC>(p, ch + 1, it0, jt0, mg, tid, st);
-
-    const bf16x8 ga = *reinterpret_cast<const bf16x8*>(&lds_a[cur][(wv * 64 + lane) * 2]);
-    bf16x8 rb[DW_TJ];
+  // Fetch cursor: chunk = (batch tile fb, time-step pair ft), batch tile fastest.  It advances one
+  // chunk per fetch with compare-and-wrap (no division in the loop) and parks on the last chunk of
+  // the split, so fetches past the end re-read valid data that is never consumed.
+  int fc = ch0, fb = ch0 % p.nbt, ft = ch0 / p.nbt;
+  auto fetch_next = [&](DwStage& s) {
+    dw_fetch<NC>(p, fb, 2 * ft, it0, jt0, mg, tid, s);
+    // branch-free advance (scalar selects): a trip of the main loop must stay one basic block so
+    // that the compiler keeps an exact count of the loads in flight
+    const int adv = (fc + 1 < ch1) ? 1 : 0;
+    fc += adv;
+    fb += adv;
+    const int wrap = (fb == p.nbt) ? 1 : 0;
+    fb = wrap ? 0 : fb;
+    ft += wrap;
+  };
+  auto compute = [&](int cur) {
+    bf16x8 ga[DW_WI], rb[DW_WJ];
 #pragma unroll
-    for (int u = 0; u < DW_TJ; ++u) rb[u] = *reinterpret_cast<const bf16x8*>(&lds_b[cur][(u * 64 + lane) * 2]);
+    for (int ii = 0; ii < DW_WI; ++ii)
+      ga[ii] = *reinterpret_cast<const bf16x8*>(&lds_a[cur][(DW_WI * wi + ii) * 64 + lane]);
+    f32x4 cf[NMAT][2];
 #pragma unroll
-    for (int a = 0; a < 3; ++a) {
-      if (a >= nmat) break;
-      bf16x8 gg = ga;
-      if (3 * mg + a != 0) {
-        const f32x4 c0 = *reinterpret_cast<const f32x4*>(&lds_c[cur][a * 32 + 4 * q]);
-        const f32x4 c1 = *reinterpret_cast<const f32x4*>(&lds_c[cur][a * 32 + 16 + 4 * q]);
-        gg = gate_frag(ga, c0, c1);
-      }
-#pragma unroll
-      for (int u = 0; u < DW_TJ; ++u) acc[a][u] = mfma16(gg, rb[u], acc[a][u]);
+    for (int a = 0; a < NMAT; ++a) {
+      cf[a][0] = *reinterpret_cast<const f32x4*>(&lds_c[cur][a * 32 + 4 * q]);
+      cf[a][1] = *reinterpret_cast<const f32x4*>(&lds_c[cur][a * 32 + 16 + 4 * q]);
     }
-    if (more) dw_publish<NC>(lds_a[cur ^ 1], lds_b[cur ^ 1], lds_c[cur ^ 1], tid, st);
+#pragma unroll
+    for (int u = 0; u < DW_WJ; ++u) rb[u] = *reinterpret_cast<const bf16x8*>(&lds_b[cur][(DW_WJ * wj + u) * 64 + lane]);
+#pragma unroll
+    for (int a = 0; a < NMAT; ++a) {
+#pragma unroll
+      for (int ii = 0; ii < DW_WI; ++ii) {
+        const bf16x8 gg = (FIRST && a == 0) ? ga[ii] : gate_frag(ga[ii], cf[a][0], cf[a][1]);
+#pragma unroll
+        for (int u = 0; u < DW_WJ; ++u) acc[a][ii][u] = mfma16(gg, rb[u], acc[a][ii][u]);
+      }
+    }
+  };
+
+  if (ch0 < ch1) {
+    DwStage st[DW_DEPTH];
+#pragma unroll
+    for (int d = 0; d < DW_DEPTH; ++d) fetch_next(st[d]);
+    dw_publish(lds_a[0], lds_b[0], lds_c[0], tid, st[0]);
     __syncthreads();
+
+    // main loop: DW_DEPTH chunks per trip, no control flow inside a trip
+    int base = ch0;
+    for (; base + DW_DEPTH <= ch1; base += DW_DEPTH) {
+#pragma unroll
+      for (int d = 0; d < DW_DEPTH; ++d) {
+        const int cur = d & 1;   // DW_DEPTH is even, so chunk parity == d parity
+        // stage d was published one step ago; refill it DW_DEPTH chunks ahead
+        fetch_next(st[d]);
+        compute(cur);
+        dw_publish(lds_a[cur ^ 1], lds_b[cur ^ 1], lds_c[cur ^ 1], tid, st[(d + 1) % DW_DEPTH]);
+        __syncthreads();
+      }
+    }
+    // tail (< DW_DEPTH chunks): stages 0.. hold chunks base.., LDS buffer 0 holds chunk `base`
+#pragma unroll
+    for (int d = 0; d < DW_DEPTH - 1; ++d) {
+      if (base + d >= ch1) break;
+      compute(d & 1);
+      dw_publish(lds_a[(d & 1) ^ 1], lds_b[(d & 1) ^ 1], lds_c[(d & 1) ^ 1], tid, st[d + 1]);
+      __syncthreads();
+    }
   }
 
 #pragma unroll
-  for (int a = 0; a < 3; ++a) {
-    if (a >= nmat) break;
+  for (int a = 0; a < NMAT; ++a) {
     const int mm = 3 * mg + a;
 #pragma unroll
-    for (int u = 0; u < DW_TJ; ++u) {
-      const int it = it0 + wv, jt = jt0 + u;
-      p.partial[((((size_t)z * (p.k + 1) + mm) * NT + it) * NT + jt) * 64 + lane] = acc[a][u];
-    }
+    for (int ii = 0; ii < DW_WI; ++ii)
+#pragma unroll
+      for (int u = 0; u < DW_WJ; ++u) {
+        const int it = it0 + DW_WI * wi + ii, jt = jt0 + DW_WJ * wj + u;
+        p.partial[((((size_t)z * (p.k + 1) + mm) * NT + it) * NT + jt) * 64 + lane] = acc[a][ii][u];
+      }
   }
 }
 
@@ -183,8 +193,9 @@ bool ring_dw_tiled_applicable(int NC) { return NC == 4 || NC == 8; }
 // K splits for the tiled kernel: about two workgroups per CU, a multiple of 8 when possible.
 int ring_dw_tiled_nz(int NC, int k, long nchunk) {
   const int NT = 4 * NC;
-  const long tiles = (long)(NT / DW_TI) * (NT / DW_TJ) * ((k + 3) / 3);
-  long nz = (512 + tiles - 1) / tiles;
+  (void)k;   // one launch per matrix group: the grid of a launch does not depend on a_dim
+  const long tiles = (long)(NT / DW_TI) * (NT / DW_TJ);
+  long nz = (256 + tiles - 1) / tiles;   // one workgroup per CU
   if (nz >= 8) nz = (nz + 7) / 8 * 8;
   if (nz > 128) nz = 128;
   if (nz > nchunk) nz = nchunk;
@@ -192,15 +203,29 @@ int ring_dw_tiled_nz(int NC, int k, long nchunk) {
   return (int)nz;
 }
 
+template <int NC>
+static hipError_t launch_group(const RingDwArgs& a, int mg, unsigned blocks, hipStream_t st) {
+  const int nmat = (a.k + 1 - 3 * mg) < 3 ? (a.k + 1 - 3 * mg) : 3;
+  if (mg == 0) {
+    if (nmat == 3) hipLaunchKernelGGL((ring_dw_tiled_kernel<NC, 3, true>), dim3(blocks), dim3(DW_THREADS), 0, st, a, mg);
+    else if (nmat == 2) hipLaunchKernelGGL((ring_dw_tiled_kernel<NC, 2, true>), dim3(blocks), dim3(DW_THREADS), 0, st, a, mg);
+    else hipLaunchKernelGGL((ring_dw_tiled_kernel<NC, 1, true>), dim3(blocks), dim3(DW_THREADS), 0, st, a, mg);
+  } else {
+    if (nmat == 3) hipLaunchKernelGGL((ring_dw_tiled_kernel<NC, 3, false>), dim3(blocks), dim3(DW_THREADS), 0, st, a, mg);
+    else if (nmat == 2) hipLaunchKernelGGL((ring_dw_tiled_kernel<NC, 2, false>), dim3(blocks), dim3(DW_THREADS), 0, st, a, mg);
+    else hipLaunchKernelGGL((ring_dw_tiled_kernel<NC, 1, false>), dim3(blocks), dim3(DW_THREADS), 0, st, a, mg);
+  }
+  return hipGetLastError();
+}
+
+// One launch per group of three matrices (a_dim = 2 needs exactly one).
 hipError_t ring_launch_dw_tiled(const RingDwArgs& a, int NC, hipStream_t st) {
   const int NT = 4 * NC;
-  const long tiles = (long)(NT / DW_TI) * (NT / DW_TJ) * ((a.k + 3) / 3);
-  const unsigned blocks = (unsigned)(tiles * a.nz);
-  if (NC == 4)
-    hipLaunchKernelGGL(ring_dw_tiled_kernel<4>, dim3(blocks), dim3(256), 0, st, a);
-  else if (NC == 8)
-    hipLaunchKernelGGL(ring_dw_tiled_kernel<8>, dim3(blocks), dim3(256), 0, st, a);
-  else
-    return hipErrorInvalidValue;
-  return hipGetLastError();
+  const unsigned blocks = (unsigned)((NT / DW_TI) * (NT / DW_TJ) * a.nz);
+  const int nmg = (a.k + 3) / 3;
+  for (int mg = 0; mg < nmg; ++mg) {
+    hipError_t e = NC == 4 ? launch_group<4>(a, mg, blocks, st) : (NC == 8 ? launch_group<8>(a, mg, blocks, st) : hipErrorInvalidValue);
+    if (e != hipSuccess) return e;
+  }
+  return hipSuccess;
 }

@@ -142,7 +142,10 @@ __global__ __launch_bounds__(256) void ring_fwd_kernel(RingFwdArgs p) {
   rows_load<NC>(p.r_init, N, B, b0, i0, r);
   write_operand<NC>(xbuf[0], r, w, q, n);
   publish_rowsum<NC>(psum[0], r, w, q, n);
-  if (p.rfrag) side_store<NC, bf16x4, __bf16>(p.rfrag + side_offset<NC>(0, p.nbt, bt, w, lane), r);
+  if (p.rfrag) {
+    pair_store<NC>(p.rfrag, 0, p.nbt, bt, w, lane, r);
+    pair_zero_tail<NC>(p.rfrag, T, p.nbt, bt, w, lane);
+  }
   lds_barrier();
 
   for (int t = 0; t < T; ++t) {
@@ -169,7 +172,7 @@ __global__ __launch_bounds__(256) void ring_fwd_kernel(RingFwdArgs p) {
     if (t + 1 < T) {
       write_operand<NC>(xbuf[cur ^ 1], r, w, q, n);
       publish_rowsum<NC>(psum[cur ^ 1], r, w, q, n);
-      if (p.rfrag) side_store<NC, bf16x4, __bf16>(p.rfrag + side_offset<NC>(t + 1, p.nbt, bt, w, lane), r);
+      if (p.rfrag) pair_store<NC>(p.rfrag, t + 1, p.nbt, bt, w, lane, r);
     }
     lds_barrier();
   }
@@ -196,7 +199,8 @@ __global__ __launch_bounds__(256) void ring_rebuild_saved_kernel(RingFwdArgs p) 
   rows_load<NC>(prev, N, B, b0, i0, r);
   write_operand<NC>(xbuf, r, w, q, n);
   publish_rowsum<NC>(psum, r, w, q, n);
-  side_store<NC, bf16x4, __bf16>(p.rfrag + side_offset<NC>(t, p.nbt, bt, w, lane), r);
+  pair_store<NC>(p.rfrag, t, p.nbt, bt, w, lane, r);
+  if (t == T - 1) pair_zero_tail<NC>(p.rfrag, T, p.nbt, bt, w, lane);
   lds_barrier();
 
   f32x4 acc[NC];
@@ -240,6 +244,7 @@ __global__ __launch_bounds__(256) void ring_bptt_kernel(RingBpttArgs p) {
   for (int e = 0; e < 4; ++e)
 #pragma unroll
     for (int c = 0; c < NC; ++c) carry[e][c] = 0.f;
+  pair_zero_tail<NC>(p.gfrag, T, p.nbt, bt, w, lane);
 
   for (int t = T - 1; t >= 0; --t) {
     const int cur = (T - 1 - t) & 1;
@@ -255,7 +260,7 @@ __global__ __launch_bounds__(256) void ring_bptt_kernel(RingBpttArgs p) {
       }
     write_operand<NC>(xbuf[cur], g, w, q, n);
     publish_rowsum<NC>(psum[cur], g, w, q, n);
-    side_store<NC, bf16x4, __bf16>(p.gfrag + side_offset<NC>(t, p.nbt, bt, w, lane), g);
+    pair_store<NC>(p.gfrag, t, p.nbt, bt, w, lane, g);
     lds_barrier();
 
     f32x4 acc[NC];
@@ -328,17 +333,13 @@ __global__ __launch_bounds__(256) void ring_dw_kernel(RingDwArgs p) {
     bf16x8 ga[2], rb[TJ];
 #pragma unroll
     for (int ii = 0; ii < 2; ++ii) {
-      const int it = 2 * ip + ii, wi = it / NC, ci = it % NC;
-      const bf16x4 lo = *reinterpret_cast<const bf16x4*>(p.gfrag + side_offset<NC>(t0, nbt, bt, wi, lane) + 4 * ci);
-      const bf16x4 hi = has1 ? *reinterpret_cast<const bf16x4*>(p.gfrag + side_offset<NC>(t1, nbt, bt, wi, lane) + 4 * ci) : zero4;
-      ga[ii] = join8(lo, hi);
+      ga[ii] = *reinterpret_cast<const bf16x8*>(p.gfrag + pair_offset<NC>(t0, nbt, bt, 2 * ip + ii, lane));
+      if (!has1) ga[ii] = join8(__builtin_shufflevector(ga[ii], ga[ii], 0, 1, 2, 3), zero4);
     }
 #pragma unroll
     for (int u = 0; u < TJ; ++u) {
-      const int jt = jo * TJ + u, wj = jt / NC, cj = jt % NC;
-      const bf16x4 lo = *reinterpret_cast<const bf16x4*>(p.rfrag + side_offset<NC>(t0, nbt, bt, wj, lane) + 4 * cj);
-      const bf16x4 hi = has1 ? *reinterpret_cast<const bf16x4*>(p.rfrag + side_offset<NC>(t1, nbt, bt, wj, lane) + 4 * cj) : zero4;
-      rb[u] = join8(lo, hi);
+      rb[u] = *reinterpret_cast<const bf16x8*>(p.rfrag + pair_offset<NC>(t0, nbt, bt, jo * TJ + u, lane));
+      if (!has1) rb[u] = join8(__builtin_shufflevector(rb[u], rb[u], 0, 1, 2, 3), zero4);
     }
 #pragma unroll
     for (int a = 0; a < 3; ++a) {

@@ -156,14 +156,17 @@ __global__ __launch_bounds__(256) void ring_fwd_res256_kernel(RingFwdArgs p) {
   }
   write_operand<R_NC>(xbuf, r, w, q, n);
   publish_rowsum4(psum, r, w, q, n);
-  if (SAVE) side_store<R_NC, bf16x4, __bf16>(p.rfrag + side_offset<R_NC>(0, p.nbt, bt, w, lane), r);
+  if (SAVE) {
+    pair_store<R_NC>(p.rfrag, 0, p.nbt, bt, w, lane, r);
+    pair_zero_tail<R_NC>(p.rfrag, T, p.nbt, bt, w, lane);
+  }
   GateStage gs;
   gates_fetch(p.A, T, B, bt, 0, +1, tid, gs);
   gates_publish(gbuf, tid, gs);
 
-  bf16x8 w0[2][R_KCH];
+  bf16x8 w0[2][R_KCH / 2];
 #pragma unroll
-  for (int kc = 0; kc < R_KCH; ++kc) w0[0][kc] = wl[kc * 64];
+  for (int u = 0; u < R_KCH / 2; ++u) w0[0][u] = wl[u * 64];
   lds_barrier();
 
   for (int t = 0; t < T; ++t) {
@@ -185,15 +188,21 @@ __global__ __launch_bounds__(256) void ring_fwd_res256_kernel(RingFwdArgs p) {
     float d[4][R_NC];
 #pragma unroll
     for (int c = 0; c < R_NC; ++c) {
-      // stage the LDS-resident fragments of the next tile (tile 0 of the next step after tile 3)
-#pragma unroll
-      for (int kc = 0; kc < R_KCH; ++kc) w0[(c + 1) & 1][kc] = wl[(((c + 1) & 3) * R_KCH + kc) * 64];
       f32x4 P0 = {0.f, 0.f, 0.f, 0.f}, P1 = P0, P2 = P0;
 #pragma unroll
-      for (int kc = 0; kc < R_KCH; ++kc) {
-        P0 = mfma16(af[kc], w0[c & 1][kc], P0);
-        P1 = mfma16(af[kc], wreg[0][c][kc], P1);
-        P2 = mfma16(af[kc], wreg[1][c][kc], P2);
+      for (int h = 0; h < 2; ++h) {
+        // stage the next half tile of the LDS-resident matrix (wraps to tile 0 of the next step)
+        constexpr int HK = R_KCH / 2;
+        const int f = 2 * c + h, fn = (f + 1) & 7;
+#pragma unroll
+        for (int u = 0; u < HK; ++u) w0[(f + 1) & 1][u] = wl[(fn * HK + u) * 64];
+#pragma unroll
+        for (int u = 0; u < HK; ++u) {
+          const int kc = h * HK + u;
+          P0 = mfma16(af[kc], w0[f & 1][u], P0);
+          P1 = mfma16(af[kc], wreg[0][c][kc], P1);
+          P2 = mfma16(af[kc], wreg[1][c][kc], P2);
+        }
       }
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
@@ -223,7 +232,7 @@ __global__ __launch_bounds__(256) void ring_fwd_res256_kernel(RingFwdArgs p) {
     if (t + 1 < T) {
       write_operand<R_NC>(xbuf + (cur ^ 1) * R_XSLOTS, r, w, q, n);
       publish_rowsum4(psum + (cur ^ 1) * 64, r, w, q, n);
-      if (SAVE) side_store<R_NC, bf16x4, __bf16>(p.rfrag + side_offset<R_NC>(t + 1, p.nbt, bt, w, lane), r);
+      if (SAVE) pair_store<R_NC>(p.rfrag, t + 1, p.nbt, bt, w, lane, r);
     }
     if (l == R_GCH - 1 && t + 1 < T) gates_publish(gbuf + ((ci + 1) & 1) * R_GCH * 16, tid, gs);
     lds_barrier();
@@ -236,29 +245,57 @@ __global__ __launch_bounds__(256) void ring_fwd_res256_kernel(RingFwdArgs p) {
 // ------------------------------------------------------------------------------------------------
 namespace {
 
+// One step's inputs in flight: grad_output rows (4 x 16 B) and the saved F' record (2 x 16 B, fp16).
 struct BpttStage {
-  float G[4][R_NC];
-  float D[4][R_NC];
+  f32x4 G[4];
+  f32x4 D[2];
 };
+
+// In the unmasked variant the six loads of a stage are issued with inline assembly and waited for
+// with an explicit vmcnt.  The compiler, seeing loads and stores share that counter, would otherwise
+// drain it completely (vmcnt(0)) before every use and expose a full HBM round trip per time step.
+// Safety of bptt_stage_wait<K>: loads return in issue order, so once at most K vector-memory
+// operations are outstanding and K later loads were issued after this stage, the stage has landed;
+// later stores can only make the wait longer.  The "+v" operands order every use after the wait.
+__device__ __forceinline__ f32x4 async_load16(const void* ptr) {
+  f32x4 v;
+  asm volatile("global_load_dwordx4 %0, %1, off" : "=&v"(v) : "v"(ptr) : "memory");
+  return v;
+}
+
+template <int K>
+__device__ __forceinline__ void bptt_stage_wait(BpttStage& s) {
+  asm volatile("s_waitcnt vmcnt(%6)"
+               : "+v"(s.G[0]), "+v"(s.G[1]), "+v"(s.G[2]), "+v"(s.G[3]), "+v"(s.D[0]), "+v"(s.D[1])
+               : "n"(K)
+               : "memory");
+}
 
 template <bool FULL>
 __device__ __forceinline__ void bptt_stage_load(const RingBpttArgs& p, int t, int bt, int w, int lane, int b0, int i0,
                                                 BpttStage& s) {
   if (t < 0) t = 0;   // redundant reload past the start of the sequence; never consumed
+  const _Float16* drec = p.dfrag + side_offset<R_NC>(t, p.nbt, bt, w, lane);
   if constexpr (FULL) {
     const float* grow = p.grad_out + ((size_t)t * p.B + b0) * p.N + i0;
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      const f32x4 v = *reinterpret_cast<const f32x4*>(grow + (size_t)e * p.N);
-      s.G[e][0] = v[0];
-      s.G[e][1] = v[1];
-      s.G[e][2] = v[2];
-      s.G[e][3] = v[3];
-    }
+    for (int e = 0; e < 4; ++e) s.G[e] = async_load16(grow + (size_t)e * p.N);
+    s.D[0] = async_load16(drec);
+    s.D[1] = async_load16(drec + 8);
   } else {
-    rows_load<R_NC>(p.grad_out + (size_t)t * p.B * p.N, p.N, p.B, b0, i0, s.G);
+    float G[4][R_NC];
+    rows_load<R_NC>(p.grad_out + (size_t)t * p.B * p.N, p.N, p.B, b0, i0, G);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) s.G[e] = f32x4{G[e][0], G[e][1], G[e][2], G[e][3]};
+    s.D[0] = *reinterpret_cast<const f32x4*>(drec);
+    s.D[1] = *reinterpret_cast<const f32x4*>(drec + 8);
   }
-  side_load_f16<R_NC>(p.dfrag + side_offset<R_NC>(t, p.nbt, bt, w, lane), s.D);
+}
+
+// F' of neuron c, rows e = 0..3: the record is [c][e] in fp16.
+__device__ __forceinline__ float stage_dact(const BpttStage& s, int e, int c) {
+  const f16x4 h = __builtin_bit_cast(f16x4, f32x2{s.D[c >> 1][2 * (c & 1)], s.D[c >> 1][2 * (c & 1) + 1]});
+  return (float)h[e];
 }
 
 }  // namespace
@@ -292,15 +329,16 @@ __global__ __launch_bounds__(256) void ring_bptt_res256_kernel(RingBpttArgs p) {
       okf[e][c] = ((b0 + e < B) && (i0 + c < N)) ? 1.f : 0.f;
     }
 
+  pair_zero_tail<R_NC>(p.gfrag, T, p.nbt, bt, w, lane);
   BpttStage st[2];
   bptt_stage_load<FULL>(p, T - 1, bt, w, lane, b0, i0, st[0]);
   bptt_stage_load<FULL>(p, T - 2, bt, w, lane, b0, i0, st[1]);
   GateStage gs;
   gates_fetch(p.A, T, B, bt, 0, -1, tid, gs);
   gates_publish(gbuf, tid, gs);
-  bf16x8 w0[2][R_KCH];
+  bf16x8 w0[2][R_KCH / 2];
 #pragma unroll
-  for (int kc = 0; kc < R_KCH; ++kc) w0[0][kc] = wl[kc * 64];
+  for (int u = 0; u < R_KCH / 2; ++u) w0[0][u] = wl[u * 64];
   // (the first lds_barrier inside the loop also publishes the gates)
 
   for (int u0 = 0; u0 < T; u0 += 2) {
@@ -312,6 +350,8 @@ __global__ __launch_bounds__(256) void ring_bptt_res256_kernel(RingBpttArgs p) {
       const int cur = u & 1, ci = u / R_GCH, l = u % R_GCH;
       if (l == 0 && (ci + 1) * R_GCH < T) gates_fetch(p.A, T, B, bt, ci + 1, -1, tid, gs);
       BpttStage& S = st[half];
+      // the other stage's six loads are the only loads issued after this stage's
+      if constexpr (FULL) bptt_stage_wait<6>(S);
 
       float G[4][R_NC], g[4][R_NC];
 #pragma unroll
@@ -319,12 +359,12 @@ __global__ __launch_bounds__(256) void ring_bptt_res256_kernel(RingBpttArgs p) {
 #pragma unroll
         for (int c = 0; c < R_NC; ++c) {
           G[e][c] = S.G[e][c] + carry[e][c];
-          g[e][c] = alpha * S.D[e][c] * G[e][c];
+          g[e][c] = alpha * stage_dact(S, e, c) * G[e][c];
         }
       bf16x8* xb = xbuf + cur * R_XSLOTS;
       write_operand<R_NC>(xb, g, w, q, n);
       publish_rowsum4(psum + cur * 64, g, w, q, n);
-      side_store<R_NC, bf16x4, __bf16>(p.gfrag + side_offset<R_NC>(t, p.nbt, bt, w, lane), g);
+      pair_store<R_NC>(p.gfrag, t, p.nbt, bt, w, lane, g);
       bptt_stage_load<FULL>(p, t - 2, bt, w, lane, b0, i0, S);
       lds_barrier();
 
@@ -340,14 +380,21 @@ __global__ __launch_bounds__(256) void ring_bptt_res256_kernel(RingBpttArgs p) {
       }
 #pragma unroll
       for (int c = 0; c < R_NC; ++c) {
-#pragma unroll
-        for (int kc = 0; kc < R_KCH; ++kc) w0[(c + 1) & 1][kc] = wl[(((c + 1) & 3) * R_KCH + kc) * 64];
         f32x4 P0 = {0.f, 0.f, 0.f, 0.f}, P1 = P0, P2 = P0;
 #pragma unroll
-        for (int kc = 0; kc < R_KCH; ++kc) {
-          P0 = mfma16(af[kc], w0[c & 1][kc], P0);
-          P1 = mfma16(af[kc], wreg[0][c][kc], P1);
-          P2 = mfma16(af[kc], wreg[1][c][kc], P2);
+        for (int h = 0; h < 2; ++h) {
+          // stage the next half tile of the LDS-resident matrix (wraps to tile 0 of the next step)
+          constexpr int HK = R_KCH / 2;
+          const int f = 2 * c + h, fn = (f + 1) & 7;
+#pragma unroll
+          for (int u = 0; u < HK; ++u) w0[(f + 1) & 1][u] = wl[(fn * HK + u) * 64];
+#pragma unroll
+          for (int u = 0; u < HK; ++u) {
+            const int kc = h * HK + u;
+            P0 = mfma16(af[kc], w0[f & 1][u], P0);
+            P1 = mfma16(af[kc], wreg[0][c][kc], P1);
+            P2 = mfma16(af[kc], wreg[1][c][kc], P2);
+          }
         }
 #pragma unroll
         for (int e = 0; e < 4; ++e) {

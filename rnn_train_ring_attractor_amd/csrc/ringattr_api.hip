@@ -28,7 +28,8 @@ size_t align_up(size_t x) { return (x + kAlign - 1) / kAlign * kAlign; }
 struct Geo {
   int N, k, T, B, NC, NPAD, nbt, nz;
   size_t wpack_bytes;    // one packed copy of [Wo|Wa] in bf16
-  size_t side_bytes;     // one tile-ordered 2-byte [T,16*nbt,NPAD] side buffer
+  size_t side_bytes;     // saved F' (fp16), [T,16*nbt,NPAD] in lane order
+  size_t pair_bytes;     // one bf16 operand copy, time steps paired: [ceil(T/2)*2,16*nbt,NPAD]
   size_t partial_bytes;  // split-K partials of the weight gradient
 };
 
@@ -53,9 +54,11 @@ int make_geo(int N, int k, int T, int B, Geo& g) {
   g.nbt = (B + 15) / 16;
   g.wpack_bytes = align_up((size_t)(1 + k) * g.NPAD * g.NPAD * 2);
   g.side_bytes = align_up((size_t)T * g.nbt * 16 * g.NPAD * 2);
+  g.pair_bytes = align_up((size_t)((T + 1) / 2) * 2 * g.nbt * 16 * g.NPAD * 2);
   const int NT = 4 * nc, TJ = nc == 1 ? 4 : 8;
   const long per_z = (long)(NT / 2) * (NT / TJ) * ((k + 3) / 3);  // wave work items per K split
   const long nchunk = (long)g.nbt * ((T + 1) / 2);
+  if (nchunk > 0x7fffffffL) return fail(RINGATTR_ERR_INVALID, "batch_size * seq_len is too large");
   long nz = (2048 + per_z - 1) / per_z;
   if (nz > 128) nz = 128;
   if (nz > nchunk) nz = nchunk;
@@ -87,7 +90,7 @@ const char* ringattr_last_error(void) { return g_err; }
 size_t ringattr_saved_bytes(int N, int a_dim, int seq_len, int batch_size) {
   Geo g;
   if (make_geo(N, a_dim, seq_len, batch_size, g) != RINGATTR_OK) return 0;
-  return 2 * g.side_bytes;
+  return g.side_bytes + g.pair_bytes;
 }
 
 size_t ringattr_fwd_workspace_bytes(int N, int a_dim, int seq_len, int batch_size) {
@@ -99,8 +102,8 @@ size_t ringattr_fwd_workspace_bytes(int N, int a_dim, int seq_len, int batch_siz
 size_t ringattr_bwd_workspace_bytes(int N, int a_dim, int seq_len, int batch_size, int have_saved) {
   Geo g;
   if (make_geo(N, a_dim, seq_len, batch_size, g) != RINGATTR_OK) return 0;
-  size_t s = g.wpack_bytes + g.side_bytes + g.partial_bytes;
-  if (!have_saved) s += g.wpack_bytes + 2 * g.side_bytes;
+  size_t s = g.wpack_bytes + g.pair_bytes + g.partial_bytes;
+  if (!have_saved) s += g.wpack_bytes + g.side_bytes + g.pair_bytes;
   return s;
 }
 
@@ -169,7 +172,7 @@ int ringattr_bwd(const void* grad_output, const void* A, const void* Wa, float J
   void* wb = ws;
   ws += g.wpack_bytes;
   __bf16* gfrag = (__bf16*)ws;
-  ws += g.side_bytes;
+  ws += g.pair_bytes;
   ring_f32x4* partial = (ring_f32x4*)ws;
   ws += g.partial_bytes;
 
