@@ -186,9 +186,13 @@ __global__ __launch_bounds__(256) void ring_fwd_res256_kernel(RingFwdArgs p) {
     }
 
     float d[4][R_NC];
-#pragma unroll
-    for (int c = 0; c < R_NC; ++c) {
-      f32x4 P0 = {0.f, 0.f, 0.f, 0.f}, P1 = P0, P2 = P0;
+    // Software pipeline over the four column tiles: the 24 MFMAs of tile c+1 are issued while the
+    // vector ALU runs the epilogue (gating, activation, leak) of tile c, so the matrix pipe works in
+    // the shadow of the epilogue instead of before it.
+    f32x4 P[2][3];
+    const f32x4 js = s * J0;
+    auto mfma_tile = [&](int c, f32x4 (&Pc)[3]) {
+      Pc[0] = Pc[1] = Pc[2] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int h = 0; h < 2; ++h) {
         // stage the next half tile of the LDS-resident matrix (wraps to tile 0 of the next step)
@@ -199,16 +203,18 @@ __global__ __launch_bounds__(256) void ring_fwd_res256_kernel(RingFwdArgs p) {
 #pragma unroll
         for (int u = 0; u < HK; ++u) {
           const int kc = h * HK + u;
-          P0 = mfma16(af[kc], w0[f & 1][u], P0);
-          P1 = mfma16(af[kc], wreg[0][c][kc], P1);
-          P2 = mfma16(af[kc], wreg[1][c][kc], P2);
+          Pc[0] = mfma16(af[kc], w0[f & 1][u], Pc[0]);
+          Pc[1] = mfma16(af[kc], wreg[0][c][kc], Pc[1]);
+          Pc[2] = mfma16(af[kc], wreg[1][c][kc], Pc[2]);
         }
       }
+    };
+    auto epilogue_tile = [&](int c, const f32x4 (&Pc)[3]) {
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        float x = fmaf(J0, s[e], J1 * P0[e]);
-        x = fmaf(gate[e][0], P1[e], x);
-        x = fmaf(gate[e][1], P2[e], x);
+        float x = fmaf(J1, Pc[0][e], js[e]);
+        x = fmaf(gate[e][0], Pc[1][e], x);
+        x = fmaf(gate[e][1], Pc[2][e], x);
         float F, D;
         act_fast<ACT>(x, F, D);
         float rn = fmaf(alpha, F, oma * r[e][c]);
@@ -219,6 +225,12 @@ __global__ __launch_bounds__(256) void ring_fwd_res256_kernel(RingFwdArgs p) {
         r[e][c] = rn;
         d[e][c] = D;
       }
+    };
+    mfma_tile(0, P[0]);
+#pragma unroll
+    for (int c = 0; c < R_NC; ++c) {
+      if (c + 1 < R_NC) mfma_tile(c + 1, P[(c + 1) & 1]);
+      epilogue_tile(c, P[c & 1]);
     }
     if constexpr (FULL) {
       float* hrow = p.hist + ((size_t)t * B + b0) * N + i0;
