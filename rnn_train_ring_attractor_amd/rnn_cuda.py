@@ -34,16 +34,21 @@ def _contig(name, t):
         raise RuntimeError(f"{name} must be contiguous")       # wording of cpp/fwd.cpp:31-35
 
 
-def _f32_cuda(name, t, shape, device):
-    _contig(name, t)
-    if t.dtype != torch.float32:
-        raise TypeError(f"{name} must be float32, got {t.dtype}")
-    if tuple(t.shape) != tuple(shape):
-        raise ValueError(f"{name} must have shape {tuple(shape)}, got {tuple(t.shape)}")
-    if not t.is_cuda:
-        raise RuntimeError(f"{name} must be a GPU tensor (device {t.device}); there is no CPU path")
-    if device is not None and t.device != device:
-        raise RuntimeError(f"{name} is on {t.device}, expected {device}")
+def _f32_cuda(specs):
+    """specs: (name, tensor, shape) triples.  Dtype and shape of every tensor are checked before any
+    device check, so malformed calls are reported the same way with or without a GPU."""
+    for name, t, shape in specs:
+        _contig(name, t)
+        if t.dtype != torch.float32:
+            raise TypeError(f"{name} must be float32, got {t.dtype}")
+        if tuple(t.shape) != tuple(shape):
+            raise ValueError(f"{name} must have shape {tuple(shape)}, got {tuple(t.shape)}")
+    device = specs[0][1].device
+    for name, t, _ in specs:
+        if not t.is_cuda:
+            raise RuntimeError(f"{name} must be a GPU tensor (device {t.device}); there is no CPU path")
+        if t.device != device:
+            raise RuntimeError(f"{name} is on {t.device}, expected {device}")
 
 
 def _scalar(name, v) -> float:
@@ -99,11 +104,8 @@ class _Fwd:
         act = _act(activation_type)
         J0, J1, alpha = _scalar("J0", J0), _scalar("J1", J1), _scalar("alpha", alpha)
         dev = A.device
-        _f32_cuda("A", A, (B, T, k), None)
-        _f32_cuda("Wa", Wa, (k, N, N), dev)
-        _f32_cuda("Wo", Wo, (N, N), dev)
-        _f32_cuda("r_init", r_init, (B, N), dev)
-        _f32_cuda("bump_history", bump_history, (T, B, N), dev)
+        _f32_cuda([("A", A, (B, T, k)), ("Wa", Wa, (k, N, N)), ("Wo", Wo, (N, N)), ("r_init", r_init, (B, N)),
+                   ("bump_history", bump_history, (T, B, N))])
         lib = _lib.load()
         if saved is not None:
             _contig("saved", saved)
@@ -144,16 +146,12 @@ class _Bwd:
         act = _act(activation_type)
         J0, J1, alpha = _scalar("J0", J0), _scalar("J1", J1), _scalar("alpha", alpha)
         dev = A.device
-        _f32_cuda("A", A, (B, T, k), None)
-        _f32_cuda("grad_output", grad_output, (T, B, N), dev)
-        _f32_cuda("Wa", Wa, (k, N, N), dev)
-        _f32_cuda("Wo", Wo, (N, N), dev)
-        _f32_cuda("bump_history", bump_history, (T, B, N), dev)
-        _f32_cuda("r_init", r_init, (B, N), dev)
-        _f32_cuda("grad_Wa", grad_Wa, (k, N, N), dev)
-        _f32_cuda("grad_Wo", grad_Wo, (N, N), dev)
+        specs = [("A", A, (B, T, k)), ("grad_output", grad_output, (T, B, N)), ("Wa", Wa, (k, N, N)),
+                 ("Wo", Wo, (N, N)), ("bump_history", bump_history, (T, B, N)), ("r_init", r_init, (B, N)),
+                 ("grad_Wa", grad_Wa, (k, N, N)), ("grad_Wo", grad_Wo, (N, N))]
         if grad_r_init is not None:
-            _f32_cuda("grad_r_init", grad_r_init, (B, N), dev)
+            specs.append(("grad_r_init", grad_r_init, (B, N)))
+        _f32_cuda(specs)
         lib = _lib.load()
         if saved is not None:
             _contig("saved", saved)

@@ -1,0 +1,110 @@
+"""Host-only checks of the drop-in boundary: the C-ABI library loads and exports every symbol the
+header declares, argument validation returns error codes / raises Python exceptions (never exits),
+and the workspace-size queries are consistent.  No kernel is launched here."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+from rnn_train_ring_attractor_amd import _lib, bwd_cuda, fwd_cuda, ring_rnn_cuda_func
+from rnn_train_ring_attractor_amd import rnn_cuda
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _header_symbols():
+    text = open(os.path.join(ROOT, "include", "ringattr.h")).read()
+    return sorted(set(re.findall(r"RINGATTR_API\s+[\w\s\*]+?\b(\w+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = _lib.load()
+    names = _header_symbols()
+    assert {"ringattr_fwd", "ringattr_bwd", "fwd_cuda", "bwd_cuda", "ringattr_saved_bytes"} <= set(names)
+    for n in names:
+        assert hasattr(lib, n), n
+    assert sorted(_lib.PROTOTYPES) == names          # the ctypes table and the header agree
+    assert lib.ringattr_version() >= 1000
+
+
+def test_size_queries():
+    lib = _lib.load()
+    N, k, T, B = 256, 2, 120, 4096
+    saved = lib.ringattr_saved_bytes(N, k, T, B)
+    assert saved == 2 * T * B * N * 2                                  # fp16 F' + bf16 r_prev, both [T,B,N]
+    assert lib.ringattr_fwd_workspace_bytes(N, k, T, B) == 3 * N * N * 2
+    with_saved = lib.ringattr_bwd_workspace_bytes(N, k, T, B, 1)
+    without = lib.ringattr_bwd_workspace_bytes(N, k, T, B, 0)
+    assert without - with_saved == saved + 3 * N * N * 2               # rebuilt buffer + forward weight pack
+    # padding: N=120 -> 128 neurons, B=64 -> 4 batch tiles; odd T rounds the paired buffer up
+    assert lib.ringattr_saved_bytes(120, 2, 7, 64) == (7 + 8) * 64 * 128 * 2
+    assert lib.ringattr_saved_bytes(0, 2, 7, 64) == 0 and "positive" in _lib.last_error()
+    assert lib.ringattr_saved_bytes(513, 2, 7, 64) == 0 and "512" in _lib.last_error()
+
+
+def test_c_abi_rejects_bad_arguments_with_codes_not_exit():
+    lib = _lib.load()
+    buf = (ctypes.c_char * 4096)()
+    p = ctypes.addressof(buf)
+    p = (p + 255) // 256 * 256
+    ok_args = [p, p, 0.0, 1.0, p, p, p, 0.15, 64, 2, 4, 16]
+    assert lib.ringattr_fwd(*ok_args, 7, None, p, 1 << 20, None) == 1 and "activation_type" in _lib.last_error()
+    assert lib.ringattr_fwd(None, *ok_args[1:], 0, None, p, 1 << 20, None) == 1 and "null" in _lib.last_error()
+    assert lib.ringattr_fwd(p + 4, *ok_args[1:], 0, None, p, 1 << 20, None) == 1 and "aligned" in _lib.last_error()
+    assert lib.ringattr_fwd(*ok_args, 0, None, p, 16, None) == 2 and "workspace" in _lib.last_error()
+    assert lib.ringattr_fwd(*ok_args, 0, None, None, 0, None) == 2
+    bad_shape = list(ok_args)
+    bad_shape[9] = 0                                                    # a_dim
+    assert lib.ringattr_fwd(*bad_shape, 0, None, p, 1 << 20, None) == 1
+    bwd_args = [p, p, p, 0.0, 1.0, p, p, p, p, p, 0.15, 64, 2, 4, 16, 0]
+    assert lib.ringattr_bwd(*bwd_args, None, None, None, p, 16, None) == 2
+    assert lib.ringattr_bwd(*bwd_args, None, p, None, p, 1 << 30, None) == 1 and "grad_A" in _lib.last_error()
+    assert lib.ringattr_profile_read(None, None) == 1
+    with pytest.raises(ValueError):
+        _lib.check(1)
+    with pytest.raises(RuntimeError):
+        _lib.check(3)
+
+
+def _cpu_problem(B=4, T=3, k=2, N=8):
+    return dict(A=torch.zeros(B, T, k), Wa=torch.zeros(k, N, N), Wo=torch.zeros(N, N), r_init=torch.zeros(B, N),
+                bump_history=torch.zeros(T, B, N))
+
+
+def test_python_binding_validation():
+    kw = _cpu_problem()
+    common = dict(J0=-0.1, J1=0.1, alpha=0.15, activation_type=0)
+    with pytest.raises(RuntimeError, match="GPU tensor"):               # there is no CPU path
+        fwd_cuda.fwd(**kw, **common)
+    bad = dict(kw, A=kw["A"].transpose(0, 1))
+    with pytest.raises(RuntimeError, match="A must be contiguous"):     # the reference's TORCH_CHECK wording
+        fwd_cuda.fwd(**bad, **common)
+    with pytest.raises(TypeError, match="float32"):
+        fwd_cuda.fwd(**dict(kw, Wo=kw["Wo"].double()), **common)
+    with pytest.raises(ValueError, match="shape"):
+        fwd_cuda.fwd(**dict(kw, r_init=torch.zeros(4, 9)), **common)
+    with pytest.raises(ValueError, match="action matrices"):
+        fwd_cuda.fwd(**dict(kw, Wa=torch.zeros(3, 8, 8)), **common)
+    with pytest.raises(ValueError, match="activation_type"):
+        fwd_cuda.fwd(**kw, J0=0.0, J1=1.0, alpha=0.15, activation_type=9)
+    with pytest.raises(TypeError, match="scalar"):
+        fwd_cuda.fwd(**kw, J0=torch.zeros(8, 8), J1=1.0, alpha=0.15, activation_type=0)
+    with pytest.raises(TypeError):
+        bwd_cuda.bwd(grad_output=kw["bump_history"], A=kw["A"], Wa=kw["Wa"], J0=0.0, J1=1.0, Wo=kw["Wo"],
+                     bump_history=kw["bump_history"], r_init=kw["r_init"], grad_Wa=kw["Wa"], grad_Wo=kw["Wo"])
+    with pytest.raises(RuntimeError, match="grad_r must be contiguous"):
+        bwd_cuda.bwd(grad_output=kw["bump_history"], A=kw["A"], Wa=kw["Wa"], J0=0.0, J1=1.0, Wo=kw["Wo"],
+                     bump_history=kw["bump_history"], r_init=kw["r_init"], grad_Wa=kw["Wa"].clone(),
+                     grad_Wo=kw["Wo"].clone(), alpha=0.15, activation_type=0, grad_r=torch.zeros(8, 4).t())
+
+
+def test_operator_rejects_unknown_activation_before_touching_the_gpu():
+    kw = _cpu_problem()
+    with pytest.raises(ValueError, match="Invalid activation 'sigmoid'"):
+        ring_rnn_cuda_func(kw["A"], kw["Wa"], -0.1, 0.1, kw["Wo"], kw["r_init"], 0.15, "sigmoid")
+
+
+def test_saved_buffer_size_helper_matches_library():
+    assert rnn_cuda.saved_nbytes(256, 2, 120, 4096) == _lib.load().ringattr_saved_bytes(256, 2, 120, 4096)

@@ -1,0 +1,91 @@
+"""Build-time checks on the compiled gfx950 ISA (hipcc cross-compiles here, no GPU needed).
+
+The BPTT kernel issues its per-step global loads with inline assembly and waits for them with an
+explicit s_waitcnt.  The compiler does not know those destination registers are still being filled,
+so this test proves on the emitted code that nothing reads or writes them between the load and the
+wait that covers it, and that the hot loops use no scratch memory."""
+import os
+import re
+import shutil
+import subprocess
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+CSRC = os.path.join(ROOT, "rnn_train_ring_attractor_amd", "csrc")
+HIPCC = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+
+pytestmark = pytest.mark.skipif(not os.path.exists(HIPCC), reason="hipcc not available")
+
+
+@pytest.fixture(scope="module")
+def res256_asm(tmp_path_factory):
+    out = tmp_path_factory.mktemp("isa") / "res256.s"
+    cmd = [HIPCC, "--offload-arch=gfx950", "-O3", "-std=c++17", "-S", "--cuda-device-only", f"-I{ROOT}/include",
+           f"-I{CSRC}", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+           "-Rpass-analysis=kernel-resource-usage", os.path.join(CSRC, "ring_res256.hip"), "-o", str(out)]
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    return out.read_text(), proc.stderr
+
+
+def _regs(tok):
+    out = set()
+    for m in re.finditer(r"\bv\[(\d+):(\d+)\]", tok):
+        out |= set(range(int(m.group(1)), int(m.group(2)) + 1))
+    for m in re.finditer(r"\bv(\d+)\b", tok):
+        out.add(int(m.group(1)))
+    return out
+
+
+def _kernel_body(asm, mangled):
+    i = asm.index(mangled + ":")
+    return asm[i:asm.index("s_endpgm", i)].split("\n")
+
+
+def test_async_loads_are_not_touched_before_their_wait(res256_asm):
+    asm, _ = res256_asm
+    body = _kernel_body(asm, "_Z23ring_bptt_res256_kernelILb1EEv12RingBpttArgs")
+    in_app, fifo, loads, waits = False, [], 0, 0
+    for ln in body + body:                      # second pass models the loop back edge
+        t = ln.strip()
+        if t.startswith(";APP"):
+            in_app = True
+            continue
+        if t.startswith(";NO_APP"):
+            in_app = False
+            continue
+        if not t or t[0] in ";.":
+            continue
+        if in_app:
+            if t.startswith("global_load"):
+                fifo.append(_regs(t.split()[1].rstrip(",")))
+                loads += 1
+            elif t.startswith("s_waitcnt") and "vmcnt" in t:
+                k = int(re.search(r"vmcnt\((\d+)\)", t).group(1))
+                del fifo[:max(0, len(fifo) - k)]
+                waits += 1
+            continue
+        if t.startswith("s_waitcnt") and "vmcnt(0)" in t:
+            fifo = []
+            continue
+        pending = set().union(*fifo) if fifo else set()
+        ops = t.split(None, 1)
+        used = _regs(ops[1]) if len(ops) > 1 else set()
+        assert not (used & pending), f"in-flight registers {sorted(used & pending)} touched by: {t}"
+    assert loads >= 12 and waits >= 2           # the pattern is present at all
+
+
+def test_hot_kernels_use_no_scratch(res256_asm):
+    _, remarks = res256_asm
+    blocks = re.split(r"remark: Function Name: ", remarks)
+    seen = 0
+    for b in blocks[1:]:
+        name = b.split()[0]
+        m = re.search(r"ScratchSize \[bytes/lane\]: (\d+)", b)
+        full_fwd = re.match(r"_Z22ring_fwd_res256_kernelILi\dELb[01]ELb1EE", name)
+        full_bptt = name.startswith("_Z23ring_bptt_res256_kernelILb1EE")
+        if full_fwd or full_bptt:
+            seen += 1
+            assert int(m.group(1)) == 0, f"{name} spills {m.group(1)} bytes per lane"
+    assert seen >= 9

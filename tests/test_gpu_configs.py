@@ -1,0 +1,154 @@
+"""GPU parity at the benchmark configurations' own shapes: full-size where the fp64 oracle finishes in
+seconds, and size-independent properties (batch-slice invariance, additivity of gradients over batch
+shards, bitwise repeatability) at the headline size."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import ring_oracle as O
+from oracle import ring_oracle_bf16 as OB
+from tests.ring_cases import make_problem
+
+pytestmark = pytest.mark.gpu
+
+TRAJ_TOL, GRAD_COS, GRAD_TOL = 1e-2, 0.999, 2e-2      # trajectories / decoded angles; gradient cosine; gradient max error
+
+
+def _t(x, dev):
+    return torch.tensor(np.ascontiguousarray(x), device=dev)
+
+
+def test_config1_inference_full_size(gpu_device):
+    """Forward only: N=256, B=1024, T=120, relu, zero ratio 0.5 (BASELINE config 1)."""
+    from rnn_train_ring_attractor_amd import ring_rnn_cuda_func
+    print("[case] config1 N=256 B=1024 T=120 relu", flush=True)
+    B, T, k, N = 1024, 120, 2, 256
+    p = make_problem(11, B, T, k, N, zero_ratios=(0.5,), weights="perfect")
+    with torch.no_grad():
+        hist = ring_rnn_cuda_func(_t(p["A"], gpu_device), _t(p["Wa"], gpu_device), -0.1, 0.1, _t(p["Wo"], gpu_device),
+                                  _t(p["r0"], gpu_device), 0.15, "gelu")
+        hist_relu = ring_rnn_cuda_func(_t(p["A"], gpu_device), _t(p["Wa"] / N, gpu_device), -1.0 / N, 1.0,
+                                       _t(p["Wo"] / N, gpu_device), _t(p["r0"], gpu_device), 0.15, "relu")
+    got = hist.cpu().numpy().astype(np.float64)
+    ref, _ = O.forward_dense(p["A"], p["Wa"], -0.1, 0.1, p["Wo"], p["r0"], 0.15, "gelu")
+    assert O.max_rel_err(got, ref) <= TRAJ_TOL
+    dg = O.decode_angle_from_population_vector(O.readout(got.transpose(1, 0, 2)))
+    dr = O.decode_angle_from_population_vector(O.readout(ref.transpose(1, 0, 2)))
+    assert np.abs(np.angle(np.exp(1j * (dg - dr)))).max() <= TRAJ_TOL * 2 * np.pi
+    # the relu variant of the same network (weights scaled to keep the bump bounded)
+    ref_relu, _ = O.forward_dense(p["A"], p["Wa"] / N, -1.0 / N, 1.0, p["Wo"] / N, p["r0"], 0.15, "relu")
+    assert O.max_rel_err(hist_relu.cpu().numpy(), ref_relu) <= TRAJ_TOL
+
+
+def test_config3_geometry_long_sequence(gpu_device):
+    """N=512, T=512, tanh (BASELINE config 3 at a batch the oracle can follow): 512 leak steps must not drift."""
+    from rnn_train_ring_attractor_amd import ring_rnn_cuda_func
+    print("[case] config3 N=512 B=32 T=512 tanh", flush=True)
+    B, T, k, N = 32, 512, 2, 512
+    p = make_problem(12, B, T, k, N, zero_ratios=(0.2,))
+    Wa = _t(p["Wa"], gpu_device).requires_grad_(True)
+    Wo = _t(p["Wo"], gpu_device).requires_grad_(True)
+    hist = ring_rnn_cuda_func(_t(p["A"], gpu_device), Wa, -0.1, 0.1, Wo, _t(p["r0"], gpu_device), 0.15, "tanh")
+    hist.backward(_t(p["G"], gpu_device))
+    ref, _ = O.forward_dense(p["A"], p["Wa"], -0.1, 0.1, p["Wo"], p["r0"], 0.15, "tanh")
+    g = O.backward_dense(p["G"], p["A"], p["Wa"], -0.1, 0.1, p["Wo"], ref, p["r0"], 0.15, "tanh")
+    got = hist.detach().cpu().numpy()
+    assert O.max_rel_err(got, ref) <= TRAJ_TOL
+    for t in (0, 255, 511):
+        assert O.max_rel_err(got[t], ref[t]) <= TRAJ_TOL
+    assert O.cosine(Wo.grad.cpu().numpy(), g["grad_Wo"]) >= GRAD_COS
+    assert O.max_rel_err(Wo.grad.cpu().numpy(), g["grad_Wo"]) <= GRAD_TOL
+    assert O.cosine(Wa.grad.cpu().numpy(), g["grad_Wa"]) >= GRAD_COS
+    assert O.max_rel_err(Wa.grad.cpu().numpy(), g["grad_Wa"]) <= GRAD_TOL
+
+
+def test_headline_size_properties(gpu_device):
+    """N=256, B=4096, T=120, gelu (BASELINE config 2).  The fp64 oracle checks a 64-row slice; the rest
+    follows from properties that do not depend on the size."""
+    from rnn_train_ring_attractor_amd import ring_rnn_cuda_func
+    print("[case] headline N=256 B=4096 T=120 gelu", flush=True)
+    B, T, k, N = 4096, 120, 2, 256
+    J0, J1 = -1.0 / N, 1.0
+    p = make_problem(42, B, T, k, N)
+    A, r0, G = _t(p["A"], gpu_device), _t(p["r0"], gpu_device), _t(p["G"], gpu_device)
+
+    def run(rows):
+        Wa = _t(p["Wa"], gpu_device).requires_grad_(True)
+        Wo = _t(p["Wo"], gpu_device).requires_grad_(True)
+        h = ring_rnn_cuda_func(A[rows].contiguous(), Wa, J0, J1, Wo, r0[rows].contiguous(), 0.15, "gelu")
+        h.backward(G[:, rows].contiguous())
+        return h.detach(), Wa.grad, Wo.grad
+
+    full = run(slice(0, B))
+    again = run(slice(0, B))
+    assert all(torch.equal(a, b) for a, b in zip(full, again))                 # bitwise repeatable
+    # samples are independent: a 64-row slice run alone reproduces its rows of the full batch bit for bit
+    part = run(slice(1024, 1088))
+    assert torch.equal(part[0], full[0][:, 1024:1088])
+    sl = slice(1024, 1088)
+    ref, _ = O.forward_dense(p["A"][sl], p["Wa"], J0, J1, p["Wo"], p["r0"][sl], 0.15, "gelu")
+    assert O.max_rel_err(part[0].cpu().numpy(), ref) <= TRAJ_TOL
+    g = O.backward_dense(p["G"][:, sl], p["A"][sl], p["Wa"], J0, J1, p["Wo"], ref, p["r0"][sl], 0.15, "gelu")
+    assert O.cosine(part[2].cpu().numpy(), g["grad_Wo"]) >= GRAD_COS
+    assert O.max_rel_err(part[2].cpu().numpy(), g["grad_Wo"]) <= GRAD_TOL
+    assert O.cosine(part[1].cpu().numpy(), g["grad_Wa"]) >= GRAD_COS
+    assert O.max_rel_err(part[1].cpu().numpy(), g["grad_Wa"]) <= GRAD_TOL
+    # gradients are sums over samples: two half-batch shards add up to the full batch (fp32 order noise)
+    lo, hi = run(slice(0, B // 2)), run(slice(B // 2, B))
+    assert O.max_rel_err((lo[1] + hi[1]).cpu().numpy(), full[1].cpu().numpy()) <= 1e-4
+    assert O.max_rel_err((lo[2] + hi[2]).cpu().numpy(), full[2].cpu().numpy()) <= 1e-4
+    assert torch.isfinite(full[0]).all()
+
+
+def test_streaming_and_resident_kernels_agree(gpu_device, monkeypatch):
+    """The generic weight-streaming kernels and the weight-resident ones evaluate the same recurrence."""
+    from rnn_train_ring_attractor_amd import ring_rnn_cuda_func
+    B, T, k, N = 80, 33, 2, 200                      # ragged: N < 256 and B not a multiple of 16
+    p = make_problem(13, B, T, k, N)
+    outs = {}
+    for mode in ("0", "1"):
+        monkeypatch.setenv("RINGATTR_STREAMING", mode)
+        Wa = _t(p["Wa"], gpu_device).requires_grad_(True)
+        Wo = _t(p["Wo"], gpu_device).requires_grad_(True)
+        h = ring_rnn_cuda_func(_t(p["A"], gpu_device), Wa, -0.1, 0.1, Wo, _t(p["r0"], gpu_device), 0.15, "silu")
+        h.backward(_t(p["G"], gpu_device))
+        outs[mode] = (h.detach().cpu().numpy(), Wa.grad.cpu().numpy(), Wo.grad.cpu().numpy())
+    for a, b in zip(outs["0"], outs["1"]):
+        assert O.max_rel_err(a, b) <= 2e-3
+    model = OB.forward_backward(p["A"], p["Wa"], -0.1, 0.1, p["Wo"], p["r0"], 0.15, "silu", p["G"])
+    assert O.max_rel_err(outs["0"][0], model["bump_history"]) <= 5e-3
+    assert O.max_rel_err(outs["0"][2], model["grad_Wo"]) <= 5e-3
+
+
+def test_training_driver_reduces_loss(gpu_device):
+    """The reference-style driver (same imports and call pattern) trains on the HIP operator."""
+    import train_general_ring_no_gain as drv
+    print("[case] training driver N=128 B=64 T=60 k=2", flush=True)
+    _, hist = drv.run_training(action_dim=2, num_neurons=128, training_steps=40, batch_size=64, seq_len=60,
+                               lr=3e-3, activation="gelu", log_every=0, seed=1)
+    assert all(np.isfinite(hist))
+    assert np.mean(hist[-5:]) < np.mean(hist[:5])
+
+
+def test_reference_signature_entry_points(gpu_device):
+    """fwd_cuda / bwd_cuda with the reference's exact C argument lists (null stream, own scratch)."""
+    import ctypes
+    from rnn_train_ring_attractor_amd import _lib
+    lib = _lib.load()
+    B, T, k, N = 32, 9, 2, 64
+    p = make_problem(14, B, T, k, N)
+    A, Wa, Wo, r0, G = (_t(p[n], gpu_device) for n in ("A", "Wa", "Wo", "r0", "G"))
+    hist = torch.empty(T, B, N, device=gpu_device)
+    torch.cuda.synchronize()
+    lib.fwd_cuda(A.data_ptr(), Wa.data_ptr(), -0.1, 0.1, Wo.data_ptr(), r0.data_ptr(), hist.data_ptr(), 0.15,
+                 N, k, T, B, 2)
+    ref, _ = O.forward_dense(p["A"], p["Wa"], -0.1, 0.1, p["Wo"], p["r0"], 0.15, "tanh")
+    assert O.max_rel_err(hist.cpu().numpy(), ref) <= TRAJ_TOL
+    gWa, gWo = torch.zeros_like(Wa), torch.zeros_like(Wo)
+    dummy = torch.empty(1, device=gpu_device, dtype=torch.bfloat16)
+    z = ctypes.c_void_p(None)
+    lib.bwd_cuda(G.data_ptr(), A.data_ptr(), Wa.data_ptr(), -0.1, 0.1, Wo.data_ptr(), hist.data_ptr(), dummy.data_ptr(),
+                 r0.data_ptr(), gWa.data_ptr(), gWo.data_ptr(), 0.15, N, k, T, B, 2, z, z, z, z, z, z, z)
+    g = O.backward_dense(p["G"], p["A"], p["Wa"], -0.1, 0.1, p["Wo"], ref, p["r0"], 0.15, "tanh")
+    assert O.cosine(gWo.cpu().numpy(), g["grad_Wo"]) >= GRAD_COS
+    assert O.max_rel_err(gWa.cpu().numpy(), g["grad_Wa"]) <= GRAD_TOL
