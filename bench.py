@@ -78,6 +78,9 @@ def main():
     ap.add_argument("--workload", default="train_n256_b4096_t120_gelu", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the host-CPU baseline leg")
     ap.add_argument("--cpu-sample-batch", type=int, default=64)
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run three 1 GiB device-to-device copies (known HBM traffic) for scaling rocprofv3's "
+                         "FETCH_SIZE / WRITE_SIZE counters")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on exactly one GPU (the batch shards trivially; see DESIGN.md); use --gpus 1")
@@ -115,6 +118,12 @@ def main():
     dt = time.perf_counter() - t0
     prof = _lib.profile_read()
     _lib.profile_enable(False)
+    if args.copy_calibration:
+        src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
 
     ms_per_step = dt / args.steps * 1e3
     value = B * T / (dt / args.steps)

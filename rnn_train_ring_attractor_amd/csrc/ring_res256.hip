@@ -271,13 +271,15 @@ struct BpttStage {
 // later stores can only make the wait longer.  The "+v" operands order every use after the wait.
 __device__ __forceinline__ f32x4 async_load16(const void* ptr) {
   f32x4 v;
-  asm volatile("global_load_dwordx4 %0, %1, off" : "=&v"(v) : "v"(ptr) : "memory");
+  // (the local labels cost nothing at run time; the build check uses them to find these loads and
+  // their waits in the emitted code)
+  asm volatile(".Lring_async_load_%=:\n\tglobal_load_dwordx4 %0, %1, off" : "=&v"(v) : "v"(ptr) : "memory");
   return v;
 }
 
 template <int K>
 __device__ __forceinline__ void bptt_stage_wait(BpttStage& s) {
-  asm volatile("s_waitcnt vmcnt(%6)"
+  asm volatile(".Lring_async_wait_%=:\n\ts_waitcnt vmcnt(%6)"
                : "+v"(s.G[0]), "+v"(s.G[1]), "+v"(s.G[2]), "+v"(s.G[3]), "+v"(s.D[0]), "+v"(s.D[1])
                : "n"(K)
                : "memory");
@@ -422,6 +424,12 @@ __global__ __launch_bounds__(256) void ring_bptt_res256_kernel(RingBpttArgs p) {
       // gate chunk; both were last read before the barrier above, so no second barrier is needed
       if (l == R_GCH - 1 && u + 1 < T) gates_publish(gbuf + ((ci + 1) & 1) * R_GCH * 16, tid, gs);
     }
+  }
+  // the last two iterations prefetched (clamped) steps that are never consumed: let those loads land
+  // while their destination registers are still reserved, before anything below reuses them
+  if constexpr (FULL) {
+    bptt_stage_wait<0>(st[0]);
+    bptt_stage_wait<0>(st[1]);
   }
   if (p.grad_r_init) rows_store<R_NC>(p.grad_r_init, N, B, b0, i0, carry);
 }

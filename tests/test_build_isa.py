@@ -46,25 +46,28 @@ def _kernel_body(asm, mangled):
 def test_async_loads_are_not_touched_before_their_wait(res256_asm):
     asm, _ = res256_asm
     body = _kernel_body(asm, "_Z23ring_bptt_res256_kernelILb1EEv12RingBpttArgs")
-    in_app, fifo, loads, waits = False, [], 0, 0
+    fifo, loads, waits, tag = [], 0, 0, None
     for ln in body + body:                      # second pass models the loop back edge
         t = ln.strip()
-        if t.startswith(";APP"):
-            in_app = True
+        if t.startswith(".Lring_async_load_"):
+            tag = "load"
             continue
-        if t.startswith(";NO_APP"):
-            in_app = False
+        if t.startswith(".Lring_async_wait_"):
+            tag = "wait"
             continue
         if not t or t[0] in ";.":
             continue
-        if in_app:
-            if t.startswith("global_load"):
-                fifo.append(_regs(t.split()[1].rstrip(",")))
-                loads += 1
-            elif t.startswith("s_waitcnt") and "vmcnt" in t:
-                k = int(re.search(r"vmcnt\((\d+)\)", t).group(1))
-                del fifo[:max(0, len(fifo) - k)]
-                waits += 1
+        if tag == "load":
+            assert t.startswith("global_load_dwordx4"), t
+            fifo.append(_regs(t.split()[1].rstrip(",")))
+            loads += 1
+            tag = None
+            continue
+        if tag == "wait":
+            k = int(re.search(r"vmcnt\((\d+)\)", t).group(1))
+            del fifo[:max(0, len(fifo) - k)]
+            waits += 1
+            tag = None
             continue
         if t.startswith("s_waitcnt") and "vmcnt(0)" in t:
             fifo = []
