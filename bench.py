@@ -21,6 +21,15 @@ if ROOT not in sys.path:
 PEAK_BF16_TFLOPS = 2500.0      # MI355X dense bf16 MFMA, TFLOP/s
 PEAK_HBM_GBS = 8000.0          # MI355X HBM3E, GB/s
 
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per dispatch, each scaled by what the
+# same counter reads for a 1 GiB device copy: x2.000 for FETCH_SIZE, x1.000 for WRITE_SIZE); the summary is
+# profiles/train_n256_b4096_t120_gelu_counters.md.  Counter runs cannot share a process with the timed region, so
+# the figures are carried here and refreshed whenever a kernel's memory behaviour changes.
+MEASURED_TRAFFIC_BYTES = {
+    "train_n256_b4096_t120_gelu": {"fwd": (6010 * 2.0 + 983284) * 1024, "bptt": (372572 * 2.0 + 249818) * 1024,
+                                   "dw": (257753 * 2.0 + 49152) * 1024},
+}
+
 WORKLOADS = {
     # BASELINE config 2 (headline)
     "train_n256_b4096_t120_gelu": dict(N=256, B=4096, T=120, k=2, act="gelu", J0=-1.0 / 256, J1=1.0),
@@ -28,22 +37,38 @@ WORKLOADS = {
 
 
 def make_inputs(cfg, device):
-    """Seeded synthetic inputs of the named shape: weights ~ N(0,1/N), av trials (10 % leading zeros,
-    U(-0.1*pi,0.1*pi), zero ratio in {0.2,0.5,0.8}), L/R = relu(-/+av), Gaussian bump at the initial angle."""
-    import numpy as np
+    """Seeded synthetic inputs of the named shape, drawn on the host with the package's own data helpers:
+    weights ~ N(0, 1/N); angular-velocity trials (10 % leading zeros, U(-0.1*pi, 0.1*pi), zero ratio in
+    {0.2, 0.5, 0.8}); L/R gates = relu(-/+av); Gaussian bump at each trial's initial angle."""
+    import math
     import torch
-    from tests.ring_cases import make_problem
-    p = make_problem(42, cfg["B"], cfg["T"], cfg["k"], cfg["N"])
-    t = lambda x: torch.tensor(np.ascontiguousarray(x), device=device)
-    return p, dict(A=t(p["A"]), Wa=t(p["Wa"]), Wo=t(p["Wo"]), r0=t(p["r0"]), angle=t(p["angle"]))
+    from rnn_train_ring_attractor_amd import host
+    torch.manual_seed(42)
+    N, B, T, k = cfg["N"], cfg["B"], cfg["T"], cfg["k"]
+    Wo = torch.randn(N, N) / math.sqrt(N)
+    Wa = torch.randn(k, N, N) / math.sqrt(N)
+    av, angle = host.generate_av_integration_data_ultra_fast(B, T)
+    A = host.av_to_action_signal(av) if k == 2 else host.av_to_action_signal_ND(av, k)
+    r0 = host.create_initial_bump(angle[:, 0], N)
+    to = lambda x: x.float().contiguous().to(device)
+    return dict(A=to(A), Wa=to(Wa), Wo=to(Wo), r0=to(r0), angle=to(angle))
 
 
 def loss_head_grad(hist, angle):
-    """d(loss pair)/d(bump_history) with torch ops on the GPU, once, outside the timed region."""
+    """d(loss)/d(bump_history) of the training script's loss pair (cosine-similarity loss of the max-normalised
+    cosine read-out + 0.2 * bump-amplitude loss; train_general_ring_no_gain.py:324-330 of the reference), computed
+    once with torch ops on the GPU, outside the timed region."""
+    import math
     import torch
-    from oracle import torch_port as TP
+    from rnn_train_ring_attractor_amd import host
+    N = hist.shape[-1]
+    idx = torch.arange(N, dtype=torch.float32, device=hist.device)
+    w_delta7 = torch.cos(2 * math.pi * (idx[:, None] - idx[None, :]) / N)
     h = hist.detach().clone().requires_grad_(True)
-    TP.loss_pair(h, angle).backward()
+    bump = h.permute(1, 0, 2)
+    proj = bump @ w_delta7
+    out = proj / proj.max(dim=2, keepdim=True)[0]
+    (host.cosine_similarity_loss(out, angle) + 0.2 * host.bump_amplitude_loss(bump)).backward()
     return h.grad.contiguous()
 
 
@@ -92,7 +117,7 @@ def main():
     dev = torch.device("cuda:0")
     cfg = WORKLOADS[args.workload]
     N, B, T, k = cfg["N"], cfg["B"], cfg["T"], cfg["k"]
-    _, x = make_inputs(cfg, dev)
+    x = make_inputs(cfg, dev)
     Wa = x["Wa"].requires_grad_(True)
     Wo = x["Wo"].requires_grad_(True)
 
@@ -143,8 +168,11 @@ def main():
         "pct_bf16_mfma_peak_fwd_bwd": 100.0 * (18.0 * N * N * value) / (PEAK_BF16_TFLOPS * 1e12),
         "algorithmic_hbm_gbs_fwd_bwd": bytes_per_ss * value / 1e9,
         "roofline": {"bound": "mfma", "kernel": dominant, "achieved": achieved, "peak": PEAK_BF16_TFLOPS,
-                     "unit": "TFLOP/s", "frac": achieved / PEAK_BF16_TFLOPS, "traffic": None,
-                     "flops_per_launch": flops_third, "avg_launch_ms": dom_ms},
+                     "unit": "TFLOP/s", "frac": achieved / PEAK_BF16_TFLOPS,
+                     "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload, {}).get(dominant),
+                     "flops_per_launch": flops_third, "avg_launch_ms": dom_ms,
+                     "algorithmic_bytes_per_launch": {"fwd": (4 * N + 4 * k) * B * T, "bptt": (4 * N + 4 * k) * B * T,
+                                                      "dw": (4 * N + 4 * k) * B * T}[dominant]},
         "kernel_ms": kern,
     }
     if not args.no_cpu:
