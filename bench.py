@@ -72,7 +72,7 @@ def loss_head_grad(hist, angle):
     return h.grad.contiguous()
 
 
-def cpu_baseline(cfg, sample_B, iters=3):
+def cpu_baseline(cfg, sample_B, iters=8):
     """Torch port of the reference formulation (W_eff per sample + bmm + autograd), fp32, host cores."""
     import torch
     from oracle import torch_port as TP
@@ -102,7 +102,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="train_n256_b4096_t120_gelu", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the host-CPU baseline leg")
-    ap.add_argument("--cpu-sample-batch", type=int, default=64)
+    ap.add_argument("--cpu-sample-batch", type=int, default=128)
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run three 1 GiB device-to-device copies (known HBM traffic) for scaling rocprofv3's "
                          "FETCH_SIZE / WRITE_SIZE counters")
