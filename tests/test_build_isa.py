@@ -13,6 +13,8 @@ import pytest
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 CSRC = os.path.join(ROOT, "rnn_train_ring_attractor_amd", "csrc")
+from rnn_train_ring_attractor_amd.build import PER_SOURCE_FLAGS  # noqa: E402
+
 HIPCC = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
 
 pytestmark = pytest.mark.skipif(not os.path.exists(HIPCC), reason="hipcc not available")
@@ -23,6 +25,7 @@ def res256_asm(tmp_path_factory):
     out = tmp_path_factory.mktemp("isa") / "res256.s"
     cmd = [HIPCC, "--offload-arch=gfx950", "-O3", "-std=c++17", "-S", "--cuda-device-only", f"-I{ROOT}/include",
            f"-I{CSRC}", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+           *PER_SOURCE_FLAGS.get("ring_res256.hip", []),
            "-Rpass-analysis=kernel-resource-usage", os.path.join(CSRC, "ring_res256.hip"), "-o", str(out)]
     proc = subprocess.run(cmd, capture_output=True, text=True)
     assert proc.returncode == 0, proc.stderr[-2000:]
