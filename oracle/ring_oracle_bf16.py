@@ -36,10 +36,23 @@ def _identity(x):
     return np.asarray(x, np.float64)
 
 
-def forward_backward(A, Wa, J0, J1, Wo, r_init, alpha, activation_name, grad_output=None, rounding=True):
-    """Returns dict(bump_history [T,B,N], and, when grad_output is given, grad_Wa, grad_Wo, grad_r_init)."""
+DACT_LO, DACT_HI = -0.25, 1.25   # range of the 8-bit F' code; covers F' of all four activations
+
+
+def round_u8_dact(x):
+    """F' stored as an 8-bit code: round((x - lo) * 255 / (hi - lo)), decoded back."""
+    scale = 255.0 / (DACT_HI - DACT_LO)
+    code = np.clip(np.rint((np.asarray(x, np.float64) - DACT_LO) * scale), 0, 255)
+    return code / scale + DACT_LO
+
+
+def forward_backward(A, Wa, J0, J1, Wo, r_init, alpha, activation_name, grad_output=None, rounding=True,
+                     rowsum_rounded=False, dact="fp16"):
+    """Returns dict(bump_history [T,B,N], and, when grad_output is given, grad_Wa, grad_Wo, grad_r_init).
+    rowsum_rounded: the J0 row sums run over the bf16 operand copy (the weight-resident kernels take them
+    from the matrix pipe) instead of the fp32 state.  dact: storage format of F', "fp16" or "u8"."""
     rb16 = round_bf16 if rounding else _identity
-    rf16 = round_fp16 if rounding else _identity
+    rf16 = (round_u8_dact if dact == "u8" else round_fp16) if rounding else _identity
     A = np.asarray(A, np.float64)
     Wa = np.asarray(Wa, np.float64)
     Wo = np.asarray(Wo, np.float64)
@@ -53,7 +66,7 @@ def forward_backward(A, Wa, J0, J1, Wo, r_init, alpha, activation_name, grad_out
     for t in range(T):
         rb = rb16(r)
         R[t] = rb
-        re = J0 * r.sum(axis=1, keepdims=True) + J1 * (rb @ Wob.T)
+        re = J0 * (rb if rowsum_rounded else r).sum(axis=1, keepdims=True) + J1 * (rb @ Wob.T)
         for c in range(k):
             re = re + A[:, t, c:c + 1] * (rb @ Wab[c].T)
         D[t] = rf16(O.activation_derivative(re, activation_name))
@@ -70,7 +83,7 @@ def forward_backward(A, Wa, J0, J1, Wo, r_init, alpha, activation_name, grad_out
         G = G_out[t] + carry
         g = alpha * D[t] * G
         gb = rb16(g)
-        carry = (1.0 - alpha) * G + J0 * g.sum(axis=1, keepdims=True) + J1 * (gb @ Wob)
+        carry = (1.0 - alpha) * G + J0 * (gb if rowsum_rounded else g).sum(axis=1, keepdims=True) + J1 * (gb @ Wob)
         for c in range(k):
             carry = carry + A[:, t, c:c + 1] * (gb @ Wab[c])
         grad_Wo += J1 * (gb.T @ R[t])

@@ -36,6 +36,14 @@ struct Tile {
 // of landing 8-way on the same ones.
 constexpr int XG = 17;
 
+// Contraction order of the pipelined NC = 4 kernels: positions 0..127 hold, wave by wave, the neurons
+// of column tiles 0,1 ("early" pair) and positions 128..255 those of tiles 2,3 ("late" pair), so a
+// wave's tile pair lands in one K chunk: position 128*h + 32*w + 2*n + cc <-> neuron 64*w + 4*n + 2*h + cc.
+__host__ __device__ __forceinline__ int split_k_neuron(int kappa) {
+  const int h = kappa >> 7, s = kappa & 127;
+  return 64 * (s >> 5) + 4 * ((s & 31) >> 1) + 2 * h + (s & 1);
+}
+
 // D = A(16x32 bf16) * B(32x16 bf16) + C(16x16 fp32).  Lane (q,n): A row n, B column n, both with
 // K slots 8q..8q+7; C/D rows 4q..4q+3 of column n.
 __device__ __forceinline__ f32x4 mfma16(bf16x8 a, bf16x8 b, f32x4 c) {

@@ -13,11 +13,13 @@
 //   out[mm][w][c][kc][lane][8]; lane (q,n) owns output column 16*NC*w + NC*n + c and the eight
 //   contraction indices 32kc+8q .. +7.  transposed = 0: value = W[col][contr] (forward, re = W r);
 //   transposed = 1: value = W[contr][col] (backward, g @ W).
+//   split_k = 1 (NC = 4 only): contraction position kappa stands for neuron split_k_neuron(kappa), the
+//   order the pipelined weight-resident kernels keep their operand tile in.
 // ------------------------------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void ring_pack_weights_kernel(const float* __restrict__ Wo,
                                                                 const float* __restrict__ Wa,
                                                                 bf16x8* __restrict__ out, int N, int k, int NC,
-                                                                int transposed) {
+                                                                int transposed, int split_k) {
   const int KCH = 2 * NC;
   const size_t total = (size_t)(1 + k) * 4 * NC * KCH * 64;
   for (size_t u = (size_t)blockIdx.x * blockDim.x + threadIdx.x; u < total; u += (size_t)gridDim.x * blockDim.x) {
@@ -36,7 +38,7 @@ __global__ __launch_bounds__(256) void ring_pack_weights_kernel(const float* __r
     bf16x8 pk;
 #pragma unroll
     for (int x = 0; x < 8; ++x) {
-      const int kk = k0 + x;
+      const int kk = split_k ? split_k_neuron(k0 + x) : k0 + x;
       float val = 0.f;
       if (col < N && kk < N) val = transposed ? W[(size_t)kk * N + col] : W[(size_t)col * N + kk];
       pk[x] = (__bf16)val;
@@ -480,17 +482,18 @@ hipError_t ring_profile_collect(double* ms, long long* launches) {
   }
 
 hipError_t ring_launch_pack(const float* Wo, const float* Wa, void* out, int N, int k, int NC, int transposed,
-                            hipStream_t st) {
+                            int split_k, hipStream_t st) {
+  if (split_k && NC != 4) return hipErrorInvalidValue;
   const size_t total = (size_t)(1 + k) * 4 * NC * 2 * NC * 64;
   const int blocks = (int)((total + 255) / 256 < 4096 ? (total + 255) / 256 : 4096);
   ProfScope prof(0, st);
   hipLaunchKernelGGL(ring_pack_weights_kernel, dim3(blocks), dim3(256), 0, st, Wo, Wa, (bf16x8*)out, N, k, NC,
-                     transposed);
+                     transposed, split_k);
   return hipGetLastError();
 }
 
 // RINGATTR_STREAMING=1 forces the generic weight-streaming kernels (used by tests to cross-check).
-static bool use_resident(int N, int k) {
+bool ring_uses_resident(int N, int k) {
   if (!ring_res256_applicable(N, k)) return false;
   const char* v = getenv("RINGATTR_STREAMING");
   return !(v && v[0] == '1');
@@ -498,7 +501,7 @@ static bool use_resident(int N, int k) {
 
 hipError_t ring_launch_fwd(const RingFwdArgs& a, int NCv, hipStream_t st) {
   ProfScope prof(1, st);
-  if (use_resident(a.N, a.k)) return ring_launch_fwd_res256(a, st);
+  if (ring_uses_resident(a.N, a.k)) return ring_launch_fwd_res256(a, st);
   RING_DISPATCH_NC(NCv, hipLaunchKernelGGL(ring_fwd_kernel<NC>, dim3(a.nbt), dim3(256), 0, st, a));
   return hipGetLastError();
 }
@@ -511,7 +514,7 @@ hipError_t ring_launch_rebuild(const RingFwdArgs& a, int NCv, hipStream_t st) {
 
 hipError_t ring_launch_bptt(const RingBpttArgs& a, int NCv, hipStream_t st) {
   ProfScope prof(3, st);
-  if (use_resident(a.N, a.k)) return ring_launch_bptt_res256(a, st);
+  if (ring_uses_resident(a.N, a.k)) return ring_launch_bptt_res256(a, st);
   RING_DISPATCH_NC(NCv, hipLaunchKernelGGL(ring_bptt_kernel<NC>, dim3(a.nbt), dim3(256), 0, st, a));
   return hipGetLastError();
 }

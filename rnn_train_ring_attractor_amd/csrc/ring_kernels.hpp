@@ -39,7 +39,7 @@ struct RingDwArgs {
 };
 
 hipError_t ring_launch_pack(const float* Wo, const float* Wa, void* out, int N, int k, int NC, int transposed,
-                            hipStream_t st);
+                            int split_k, hipStream_t st);
 hipError_t ring_launch_fwd(const RingFwdArgs& a, int NC, hipStream_t st);
 hipError_t ring_launch_rebuild(const RingFwdArgs& a, int NC, hipStream_t st);
 hipError_t ring_launch_bptt(const RingBpttArgs& a, int NC, hipStream_t st);
@@ -47,6 +47,7 @@ hipError_t ring_launch_dw(const RingDwArgs& a, int NC, hipStream_t st);
 
 // Weight-resident variants for 128 < N <= 256, a_dim == 2 (ring_res256.hip).
 bool ring_res256_applicable(int N, int k);
+bool ring_uses_resident(int N, int k);   // applicable and not disabled by RINGATTR_STREAMING=1
 hipError_t ring_launch_fwd_res256(const RingFwdArgs& a, hipStream_t st);
 hipError_t ring_launch_bptt_res256(const RingBpttArgs& a, hipStream_t st);
 

@@ -8,6 +8,8 @@
 #include "ring_common.hpp"
 #include "ring_kernels.hpp"
 
+#include <type_traits>
+
 namespace {
 
 constexpr int R_NC = 4;
@@ -15,7 +17,7 @@ constexpr int R_KCH = 8;
 constexpr int R_WLDS_SLOTS = 4 * R_NC * R_KCH * 64;   // 16-byte slots of the LDS-resident matrix
 constexpr int R_XSLOTS = R_KCH * 4 * XG;
 constexpr int R_GCH = 32;                             // time steps of action gates staged per LDS chunk
-constexpr size_t R_LDS_BYTES = (size_t)(R_WLDS_SLOTS + 2 * R_XSLOTS) * 16 + 2 * 64 * 4 + 2 * R_GCH * 16 * 8;
+constexpr size_t R_LDS_BYTES = (size_t)(R_WLDS_SLOTS + 2 * R_XSLOTS) * 16 + 2 * 64 * 4 + 2 * R_GCH * 16 * 8;   // BPTT layout (the forward uses less)
 
 // Cheap activation pairs (F, F') for the per-step critical path.
 //  gelu: Phi via the Abramowitz-Stegun 7.1.26 erfc polynomial (|err| < 1.5e-7), sharing exp(-x^2/2)
@@ -93,15 +95,17 @@ __device__ __forceinline__ void gates_fetch(const float* A, int T, int B, int bt
   const int t1 = dir > 0 ? u1 : T - 1 - u1, t2 = dir > 0 ? u2 : T - 1 - u2;
   const f32x2 va = *reinterpret_cast<const f32x2*>(A + ((size_t)bc * T + t1) * 2);
   const f32x2 vb = *reinterpret_cast<const f32x2*>(A + ((size_t)bc * T + t2) * 2);
-  const float m = b < B ? 1.f : 0.f;
-  g.a = va * m;
-  g.b = vb * m;
+  g.a = va;
+  g.b = vb;
 }
 
-__device__ __forceinline__ void gates_publish(f32x2* gb, int tid, const GateStage& g) {
+// Rows past the batch get zero gates.  The mask is applied here, not in gates_fetch, so that nothing
+// touches the loaded values (and waits for them) until the chunk is actually needed.
+__device__ __forceinline__ void gates_publish(f32x2* gb, int tid, int B, int bt, const GateStage& g) {
   const int row = tid >> 4, j = tid & 15;
-  gb[j * 16 + row] = g.a;
-  gb[(j + 16) * 16 + row] = g.b;
+  const float m = 16 * bt + row < B ? 1.f : 0.f;
+  gb[j * 16 + row] = g.a * m;
+  gb[(j + 16) * 16 + row] = g.b * m;
 }
 
 // Load this wave's resident weight slices: matrix 0 into the lane's own LDS slots, matrices 1 and 2
@@ -125,130 +129,259 @@ __device__ __forceinline__ void load_resident(const bf16x8* Wp, bf16x8* wl, bf16
 // ------------------------------------------------------------------------------------------------
 // Forward, weights resident.  Same contract as ring_fwd_kernel<4> with k == 2.
 // FULL: N == 256 and B % 16 == 0, no masking anywhere.
+//
+// One wave issues at most one instruction every four cycles and hides only about two vector-ALU
+// instructions under each MFMA, while the epilogue of a step (gating, activation, leak, conversions)
+// is several hundred of them.  So the workgroup runs EIGHT waves, two per SIMD, in two roles that
+// are half a step out of phase: while one wave of a SIMD is in its vector-ALU epilogue the other one
+// feeds the matrix pipe.  Wave (w, h), w = 0..3, h = 0/1, owns column tiles 2h and 2h+1 of neuron
+// group w (neurons 64w + 4n + 2h + {0,1}); h = 0 is the "early" role E, h = 1 the "late" role L.  The
+// contraction index is ordered so that K chunks 0..3 hold the E neurons and 4..7 the L neurons
+// (split_k_neuron), and the step t (r_t -> r_{t+1}) is
+//      barrier A_t   (r^E_t visible)
+//   E: tiles x K chunks 0..3                         L: activation of step t-1 -> r^L_t, stores of t-1
+//      barrier B_t   (r^L_t visible)
+//   E: tiles x K chunks 4..7, epilogue -> r^E_{t+1}   L: tiles x K chunks 0..7 -> pre-activations of step t
+// The E half of the operand tile is double-buffered by step parity (L still reads r^E_t while E
+// writes r^E_{t+1}); the L half is written and read in different intervals and needs one buffer.
+// Row sums for the J0 term come from the matrix pipe (r x ones).
+// Registers: 128 AGPRs hold the wave's slices of the two gated matrices, the slice of Wo sits in LDS.
 // ------------------------------------------------------------------------------------------------
+namespace {
+
+constexpr int R8_HALF_SLOTS = 4 * 4 * XG;   // 16-byte slots of one operand half (4 K chunks)
+constexpr size_t R8_LDS_BYTES = (size_t)(R_WLDS_SLOTS + 3 * R8_HALF_SLOTS) * 16 + 2 * R_GCH * 16 * 8;
+
+__device__ __forceinline__ void load_resident8(const bf16x8* Wp, bf16x8* wl, bf16x8 (&wreg)[2][2][R_KCH], int w, int h,
+                                               int lane) {
+#pragma unroll
+  for (int cc = 0; cc < 2; ++cc)
+#pragma unroll
+    for (int kc = 0; kc < R_KCH; ++kc) {
+      const int c = 2 * h + cc;
+      wl[(cc * R_KCH + kc) * 64] = Wp[((size_t)((0 * 4 + w) * R_NC + c) * R_KCH + kc) * 64 + lane];
+      wreg[0][cc][kc] = Wp[((size_t)((1 * 4 + w) * R_NC + c) * R_KCH + kc) * 64 + lane];
+      wreg[1][cc][kc] = Wp[((size_t)((2 * 4 + w) * R_NC + c) * R_KCH + kc) * 64 + lane];
+      asm volatile("" : "+a"(wreg[0][cc][kc]));
+      asm volatile("" : "+a"(wreg[1][cc][kc]));
+    }
+}
+
+// bf16 write-back of the wave's tile pair into K chunk w of one operand half.
+__device__ __forceinline__ void write_half(bf16x8* half, const float (&v)[4][2], int w, int q, int n) {
+  char* base = reinterpret_cast<char*>(half) + (size_t)((w * 4 + (n >> 2)) * XG + 4 * q) * 16 + (n & 3) * 4;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    bf16x2 pk = {(__bf16)v[e][0], (__bf16)v[e][1]};
+    *reinterpret_cast<bf16x2*>(base + e * 16) = pk;
+  }
+}
+
+}  // namespace
+
 template <int ACT, bool SAVE, bool FULL>
-__global__ __launch_bounds__(256) void ring_fwd_res256_kernel(RingFwdArgs p) {
+__global__ __launch_bounds__(512) void ring_fwd_res256_kernel(RingFwdArgs p) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
   bf16x8* wlds = reinterpret_cast<bf16x8*>(smem);
-  bf16x8* xbuf = wlds + R_WLDS_SLOTS;
-  float* psum = reinterpret_cast<float*>(xbuf + 2 * R_XSLOTS);
-  f32x2* gbuf = reinterpret_cast<f32x2*>(psum + 2 * 64);
+  bf16x8* xE = wlds + R_WLDS_SLOTS;               // two buffers, step parity
+  bf16x8* xL = xE + 2 * R8_HALF_SLOTS;
+  f32x2* gbuf = reinterpret_cast<f32x2*>(xL + R8_HALF_SLOTS);
 
-  const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, q = lane >> 4, n = lane & 15;
+  const int tid = threadIdx.x, w8 = tid >> 6, h = w8 >> 2, w = w8 & 3, lane = tid & 63, q = lane >> 4, n = lane & 15;
   const int bt = blockIdx.x;
   const int b0 = 16 * bt + 4 * q;
-  const int i0 = 16 * R_NC * w + R_NC * n;
+  const int i0 = 16 * R_NC * w + R_NC * n + 2 * h;
   const int N = p.N, B = p.B, T = p.T;
   const float oma = 1.f - p.alpha, alpha = p.alpha, J0 = p.J0, J1 = p.J1;
+  constexpr int HK = R_KCH / 2;
 
-  bf16x8 wreg[2][R_NC][R_KCH];
-  bf16x8* wl = wlds + (size_t)w * R_NC * R_KCH * 64 + lane;
-  load_resident(reinterpret_cast<const bf16x8*>(p.Wpack), wl, wreg, w, lane);
+  bf16x8 wreg[2][2][R_KCH];
+  bf16x8* wl = wlds + (size_t)(w8 * 2 * R_KCH) * 64 + lane;
+  load_resident8(reinterpret_cast<const bf16x8*>(p.Wpack), wl, wreg, w, h, lane);
+  bf16x8 ones;
+#pragma unroll
+  for (int x = 0; x < 8; ++x) ones[x] = (__bf16)1.0f;
 
-  float r[4][R_NC];
-  float okf[4][R_NC];
-  rows_load<R_NC>(p.r_init, N, B, b0, i0, r);
-  if constexpr (!FULL) {
+  float r[4][2], okf[4][2], d[4][2];
+#pragma unroll
+  for (int e = 0; e < 4; ++e)
+#pragma unroll
+    for (int cc = 0; cc < 2; ++cc) {
+      const bool ok = (b0 + e < B) && (i0 + cc < N);
+      okf[e][cc] = ok ? 1.f : 0.f;
+      r[e][cc] = ok ? p.r_init[(size_t)(b0 + e) * N + i0 + cc] : 0.f;
+    }
+  auto save_r = [&](int t) {   // bf16 copy of r_t (operand of step t) for the weight-gradient GEMM
+#pragma unroll
+    for (int cc = 0; cc < 2; ++cc) {
+      bf16x4 pk = {(__bf16)r[0][cc], (__bf16)r[1][cc], (__bf16)r[2][cc], (__bf16)r[3][cc]};
+      *reinterpret_cast<bf16x4*>(p.rfrag + pair_offset<R_NC>(t, p.nbt, bt, w * R_NC + 2 * h + cc, lane)) = pk;
+    }
+  };
+  write_half(h ? xL : xE, r, w, q, n);
+  if (SAVE) {
+    save_r(0);
+    if (T & 1) {
+      const bf16x4 z = {(__bf16)0.f, (__bf16)0.f, (__bf16)0.f, (__bf16)0.f};
+#pragma unroll
+      for (int cc = 0; cc < 2; ++cc)
+        *reinterpret_cast<bf16x4*>(p.rfrag + pair_offset<R_NC>(T, p.nbt, bt, w * R_NC + 2 * h + cc, lane)) = z;
+    }
+  }
+  GateStage gs;
+  if (h == 0) {
+    gates_fetch(p.A, T, B, bt, 0, +1, tid, gs);
+    gates_publish(gbuf, tid, B, bt, gs);
+  }
+
+  // The LDS-resident slice is consumed in units of (tile cc, four K chunks), in the order
+  // (0,K0..3) (1,K0..3) (0,K4..7) (1,K4..7); while unit f is multiplied, unit f+1 is fetched into
+  // the other register buffer.
+  bf16x8 w0[2][HK];
+  auto unit_slot = [&](int f, int u) { return (((f & 1) * R_KCH) + (f >> 1) * HK + u) * 64; };
+#pragma unroll
+  for (int u = 0; u < HK; ++u) w0[0][u] = wl[unit_slot(0, u)];
+  lds_barrier();   // A_0
+
+  // History / F' / operand-copy stores of a finished step are not issued in one burst behind its
+  // epilogue (the write path would throttle the wave for the whole burst while the matrix pipe
+  // idles) but one at a time between the MFMA groups of the following contraction.  The values stay
+  // in r[] and d[] until the next activation.  slot 0..3: history rows, 4..5: F', 6..7: operand copy.
+  auto emit_store = [&](int t, int slot) {
+    __builtin_amdgcn_sched_barrier(0);
+    if (slot < 4) {
+      const int e = slot;
+      float* dst = p.hist + ((size_t)t * B + b0 + e) * N + i0;
+      if constexpr (FULL) {
+        *reinterpret_cast<f32x2*>(dst) = f32x2{r[e][0], r[e][1]};
+      } else {
+        if (okf[e][0] != 0.f) dst[0] = r[e][0];
+        if (okf[e][1] != 0.f) dst[1] = r[e][1];
+      }
+    } else if (slot < 6) {
+      if (SAVE) {
+        const int cc = slot - 4;
+        _Float16* drec = p.dfrag + side_offset<R_NC>(t, p.nbt, bt, w, lane) + 8 * h + 4 * cc;
+        const f16x4 pk = {(_Float16)d[0][cc], (_Float16)d[1][cc], (_Float16)d[2][cc], (_Float16)d[3][cc]};
+        *reinterpret_cast<f16x4*>(drec) = pk;
+      }
+    } else if (SAVE) {
+      const int cc = slot - 6;   // r after step t is the operand of step t+1
+      bf16x4 pk = {(__bf16)r[0][cc], (__bf16)r[1][cc], (__bf16)r[2][cc], (__bf16)r[3][cc]};
+      *reinterpret_cast<bf16x4*>(p.rfrag + pair_offset<R_NC>(t + 1, p.nbt, bt, w * R_NC + 2 * h + cc, lane)) = pk;
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  };
+
+  f32x4 P[2][3], S;
+  auto mfma_unit = [&](int f, const bf16x8 (&af)[HK], int ts, int slot, auto emit) {
+    const int cc = f & 1, ph = f >> 1, fn = (f + 1) & 3;
+#pragma unroll
+    for (int u = 0; u < HK; ++u) w0[(f + 1) & 1][u] = wl[unit_slot(fn, u)];
+#pragma unroll
+    for (int u = 0; u < HK; ++u) {
+      const int kc = ph * HK + u;
+      if constexpr (decltype(emit)::value) {
+        if (u == HK / 2) emit_store(ts, slot);
+      }
+      P[cc][0] = mfma16(af[u], w0[f & 1][u], P[cc][0]);
+      P[cc][1] = mfma16(af[u], wreg[0][cc][kc], P[cc][1]);
+      P[cc][2] = mfma16(af[u], wreg[1][cc][kc], P[cc][2]);
+    }
+  };
+  // K chunks 0..3 (ph = 0, from the E buffer of this step's parity) or 4..7 (ph = 1, from the L half);
+  // with emit, four of the eight pending stores of step ts go out between the MFMA groups.
+  auto contract_half = [&](int ph, const bf16x8* half, int ts, auto emit) {
+    bf16x8 af[HK];
+    const bf16x8* xrow = half + q * XG + n;
+#pragma unroll
+    for (int u = 0; u < HK; ++u) af[u] = xrow[u * 4 * XG];
+    if (ph == 0) {
+      const f32x4 z = {0.f, 0.f, 0.f, 0.f};
+      S = z;
+#pragma unroll
+      for (int cc = 0; cc < 2; ++cc) P[cc][0] = P[cc][1] = P[cc][2] = z;
+    }
+#pragma unroll
+    for (int u = 0; u < HK; ++u) S = mfma16(af[u], ones, S);
+    if constexpr (decltype(emit)::value) emit_store(ts, 4 * ph + 0);
+    mfma_unit(2 * ph, af, ts, 4 * ph + 1, emit);
+    if constexpr (decltype(emit)::value) emit_store(ts, 4 * ph + 2);
+    mfma_unit(2 * ph + 1, af, ts, 4 * ph + 3, emit);
+  };
+  // x[e][cc] = J0*rowsum + J1*P0 + a0*P1 + a1*P2 with the gates of step t
+  auto preactivation = [&](int t, float (&x)[4][2]) {
+    const f32x2* gb = gbuf + (((t / R_GCH) & 1) * R_GCH + t % R_GCH) * 16 + 4 * q;
+    const f32x4 js = S * J0;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const f32x2 gate = gb[e];
+#pragma unroll
+      for (int cc = 0; cc < 2; ++cc) {
+        float v = fmaf(J1, P[cc][0][e], js[e]);
+        v = fmaf(gate[0], P[cc][1][e], v);
+        x[e][cc] = fmaf(gate[1], P[cc][2][e], v);
+      }
+    }
+  };
+  auto activate = [&](const float (&x)[4][2]) {
 #pragma unroll
     for (int e = 0; e < 4; ++e)
 #pragma unroll
-      for (int c = 0; c < R_NC; ++c) okf[e][c] = ((b0 + e < B) && (i0 + c < N)) ? 1.f : 0.f;
-  }
-  write_operand<R_NC>(xbuf, r, w, q, n);
-  publish_rowsum4(psum, r, w, q, n);
-  if (SAVE) {
-    pair_store<R_NC>(p.rfrag, 0, p.nbt, bt, w, lane, r);
-    pair_zero_tail<R_NC>(p.rfrag, T, p.nbt, bt, w, lane);
-  }
-  GateStage gs;
-  gates_fetch(p.A, T, B, bt, 0, +1, tid, gs);
-  gates_publish(gbuf, tid, gs);
-
-  bf16x8 w0[2][R_KCH / 2];
-#pragma unroll
-  for (int u = 0; u < R_KCH / 2; ++u) w0[0][u] = wl[u * 64];
-  lds_barrier();
-
-  for (int t = 0; t < T; ++t) {
-    const int cur = t & 1, ci = t / R_GCH, l = t % R_GCH;
-    if (l == 0 && (ci + 1) * R_GCH < T) gates_fetch(p.A, T, B, bt, ci + 1, +1, tid, gs);
-
-    const bf16x8* xb = xbuf + cur * R_XSLOTS;
-    bf16x8 af[R_KCH];
-#pragma unroll
-    for (int kc = 0; kc < R_KCH; ++kc) af[kc] = xb[(kc * 4 + q) * XG + n];
-    const f32x4 s = read_rowsum4(psum + cur * 64, q);
-    f32x2 gate[4];
-    {
-      const f32x2* gb = gbuf + ((ci & 1) * R_GCH + l) * 16 + 4 * q;
-#pragma unroll
-      for (int e = 0; e < 4; ++e) gate[e] = gb[e];
-    }
-
-    float d[4][R_NC];
-    // Software pipeline over the four column tiles: the 24 MFMAs of tile c+1 are issued while the
-    // vector ALU runs the epilogue (gating, activation, leak) of tile c, so the matrix pipe works in
-    // the shadow of the epilogue instead of before it.
-    f32x4 P[2][3];
-    const f32x4 js = s * J0;
-    auto mfma_tile = [&](int c, f32x4 (&Pc)[3]) {
-      Pc[0] = Pc[1] = Pc[2] = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int h = 0; h < 2; ++h) {
-        // stage the next half tile of the LDS-resident matrix (wraps to tile 0 of the next step)
-        constexpr int HK = R_KCH / 2;
-        const int f = 2 * c + h, fn = (f + 1) & 7;
-#pragma unroll
-        for (int u = 0; u < HK; ++u) w0[(f + 1) & 1][u] = wl[(fn * HK + u) * 64];
-#pragma unroll
-        for (int u = 0; u < HK; ++u) {
-          const int kc = h * HK + u;
-          Pc[0] = mfma16(af[kc], w0[f & 1][u], Pc[0]);
-          Pc[1] = mfma16(af[kc], wreg[0][c][kc], Pc[1]);
-          Pc[2] = mfma16(af[kc], wreg[1][c][kc], Pc[2]);
-        }
-      }
-    };
-    auto epilogue_tile = [&](int c, const f32x4 (&Pc)[3]) {
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        float x = fmaf(J1, Pc[0][e], js[e]);
-        x = fmaf(gate[e][0], Pc[1][e], x);
-        x = fmaf(gate[e][1], Pc[2][e], x);
+      for (int cc = 0; cc < 2; ++cc) {
         float F, D;
-        act_fast<ACT>(x, F, D);
-        float rn = fmaf(alpha, F, oma * r[e][c]);
+        act_fast<ACT>(x[e][cc], F, D);
+        float rn = fmaf(alpha, F, oma * r[e][cc]);
         if constexpr (!FULL) {
-          rn *= okf[e][c];
-          D *= okf[e][c];
+          rn *= okf[e][cc];
+          D *= okf[e][cc];
         }
-        r[e][c] = rn;
-        d[e][c] = D;
+        r[e][cc] = rn;
+        d[e][cc] = D;
       }
+  };
+  constexpr std::true_type with_stores{};
+  constexpr std::false_type no_stores{};
+  if (h == 0) {
+    // ---------------- role E ----------------
+    auto e_step = [&](int t, auto emit) {
+      const int ci = t / R_GCH, l = t % R_GCH;
+      if (l == 0 && (ci + 1) * R_GCH < T) gates_fetch(p.A, T, B, bt, ci + 1, +1, tid, gs);
+      contract_half(0, xE + (t & 1) * R8_HALF_SLOTS, t - 1, emit);
+      lds_barrier();   // B_t
+      contract_half(1, xL, t - 1, emit);
+      float x[4][2];
+      preactivation(t, x);
+      activate(x);
+      if (t + 1 < T) write_half(xE + ((t + 1) & 1) * R8_HALF_SLOTS, r, w, q, n);
+      // the next chunk's gates are first read after barrier B of its first step
+      if (l == R_GCH - 1 && t + 1 < T) gates_publish(gbuf + ((ci + 1) & 1) * R_GCH * 16, tid, B, bt, gs);
+      lds_barrier();   // A_{t+1}
     };
-    mfma_tile(0, P[0]);
-#pragma unroll
-    for (int c = 0; c < R_NC; ++c) {
-      if (c + 1 < R_NC) mfma_tile(c + 1, P[(c + 1) & 1]);
-      epilogue_tile(c, P[c & 1]);
+    e_step(0, no_stores);
+    for (int t = 1; t < T; ++t) e_step(t, with_stores);
+  } else {
+    // ---------------- role L ----------------
+    float x[4][2];
+    lds_barrier();   // B_0 (r^L_0 was written before A_0)
+    contract_half(0, xE, -1, no_stores);
+    contract_half(1, xL, -1, no_stores);
+    preactivation(0, x);
+    lds_barrier();   // A_1
+    for (int t = 1; t < T; ++t) {
+      activate(x);   // step t-1 -> r^L_t
+      write_half(xL, r, w, q, n);
+      lds_barrier();   // B_t
+      contract_half(0, xE + (t & 1) * R8_HALF_SLOTS, t - 1, with_stores);
+      contract_half(1, xL, t - 1, with_stores);
+      preactivation(t, x);
+      lds_barrier();   // A_{t+1}
     }
-    if constexpr (FULL) {
-      float* hrow = p.hist + ((size_t)t * B + b0) * N + i0;
-#pragma unroll
-      for (int e = 0; e < 4; ++e)
-        *reinterpret_cast<f32x4*>(hrow + (size_t)e * N) = f32x4{r[e][0], r[e][1], r[e][2], r[e][3]};
-    } else {
-      rows_store<R_NC>(p.hist + (size_t)t * B * N, N, B, b0, i0, r);
-    }
-    if (SAVE) side_store<R_NC, f16x4, _Float16>(p.dfrag + side_offset<R_NC>(t, p.nbt, bt, w, lane), d);
-    if (t + 1 < T) {
-      write_operand<R_NC>(xbuf + (cur ^ 1) * R_XSLOTS, r, w, q, n);
-      publish_rowsum4(psum + (cur ^ 1) * 64, r, w, q, n);
-      if (SAVE) pair_store<R_NC>(p.rfrag, t + 1, p.nbt, bt, w, lane, r);
-    }
-    if (l == R_GCH - 1 && t + 1 < T) gates_publish(gbuf + ((ci + 1) & 1) * R_GCH * 16, tid, gs);
-    lds_barrier();
+    activate(x);
   }
+  // stores of the last step (its state is not an operand of any further step)
+#pragma unroll
+  for (int slot = 0; slot < 6; ++slot) emit_store(T - 1, slot);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -349,7 +482,7 @@ __global__ __launch_bounds__(256) void ring_bptt_res256_kernel(RingBpttArgs p) {
   bptt_stage_load<FULL>(p, T - 2, bt, w, lane, b0, i0, st[1]);
   GateStage gs;
   gates_fetch(p.A, T, B, bt, 0, -1, tid, gs);
-  gates_publish(gbuf, tid, gs);
+  gates_publish(gbuf, tid, B, bt, gs);
   bf16x8 w0[2][R_KCH / 2];
 #pragma unroll
   for (int u = 0; u < R_KCH / 2; ++u) w0[0][u] = wl[u * 64];
@@ -422,7 +555,7 @@ __global__ __launch_bounds__(256) void ring_bptt_res256_kernel(RingBpttArgs p) {
       }
       // the next iteration overwrites the other operand buffer and, every R_GCH steps, the other
       // gate chunk; both were last read before the barrier above, so no second barrier is needed
-      if (l == R_GCH - 1 && u + 1 < T) gates_publish(gbuf + ((ci + 1) & 1) * R_GCH * 16, tid, gs);
+      if (l == R_GCH - 1 && u + 1 < T) gates_publish(gbuf + ((ci + 1) & 1) * R_GCH * 16, tid, B, bt, gs);
     }
   }
   // the last two iterations prefetched (clamped) steps that are never consumed: let those loads land
@@ -443,9 +576,9 @@ template <int ACT, bool SAVE, bool FULL>
 static hipError_t launch_fwd_variant(const RingFwdArgs& a, hipStream_t st) {
   auto kern = ring_fwd_res256_kernel<ACT, SAVE, FULL>;
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                     (int)R_LDS_BYTES);
+                                     (int)R8_LDS_BYTES);
   if (e != hipSuccess) return e;
-  hipLaunchKernelGGL(kern, dim3(a.nbt), dim3(256), R_LDS_BYTES, st, a);
+  hipLaunchKernelGGL(kern, dim3(a.nbt), dim3(512), R8_LDS_BYTES, st, a);
   return hipGetLastError();
 }
 

@@ -123,7 +123,7 @@ int ringattr_fwd(const void* A, const void* Wa, float J0, float J1, const void* 
                 workspace ? workspace_bytes : (size_t)0);
   hipStream_t st = static_cast<hipStream_t>(stream);
 
-  hipError_t e = ring_launch_pack((const float*)Wo, (const float*)Wa, workspace, N, a_dim, g.NC, 0, st);
+  hipError_t e = ring_launch_pack((const float*)Wo, (const float*)Wa, workspace, N, a_dim, g.NC, 0, ring_uses_resident(N, a_dim) ? 1 : 0, st);
   if (e != hipSuccess) return hip_fail(e, "pack weights");
 
   RingFwdArgs a;
@@ -187,7 +187,7 @@ int ringattr_bwd(const void* grad_output, const void* A, const void* Wa, float J
     _Float16* d = (_Float16*)ws;
     ws += g.side_bytes;
     __bf16* r = (__bf16*)ws;
-    hipError_t e = ring_launch_pack((const float*)Wo, (const float*)Wa, wf, N, a_dim, g.NC, 0, st);
+    hipError_t e = ring_launch_pack((const float*)Wo, (const float*)Wa, wf, N, a_dim, g.NC, 0, 0, st);
     if (e != hipSuccess) return hip_fail(e, "pack weights");
     RingFwdArgs f;
     f.A = (const float*)A;
@@ -211,7 +211,7 @@ int ringattr_bwd(const void* grad_output, const void* A, const void* Wa, float J
     rfrag = r;
   }
 
-  hipError_t e = ring_launch_pack((const float*)Wo, (const float*)Wa, wb, N, a_dim, g.NC, 1, st);
+  hipError_t e = ring_launch_pack((const float*)Wo, (const float*)Wa, wb, N, a_dim, g.NC, 1, 0, st);
   if (e != hipSuccess) return hip_fail(e, "pack transposed weights");
 
   RingBpttArgs b;

@@ -114,7 +114,7 @@ def test_streaming_and_resident_kernels_agree(gpu_device, monkeypatch):
         h.backward(_t(p["G"], gpu_device))
         outs[mode] = (h.detach().cpu().numpy(), Wa.grad.cpu().numpy(), Wo.grad.cpu().numpy())
     for a, b in zip(outs["0"], outs["1"]):
-        assert O.max_rel_err(a, b) <= 2e-3
+        assert O.max_rel_err(a, b) <= 5e-3          # both round the same operands; only the J0 row sums differ
     model = OB.forward_backward(p["A"], p["Wa"], -0.1, 0.1, p["Wo"], p["r0"], 0.15, "silu", p["G"])
     assert O.max_rel_err(outs["0"][0], model["bump_history"]) <= 5e-3
     assert O.max_rel_err(outs["0"][2], model["grad_Wo"]) <= 5e-3

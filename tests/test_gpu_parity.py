@@ -23,6 +23,13 @@ GRAD_TOL = 2e-2
 MODEL_TOL = 5e-3        # HIP vs the rounding-aware CPU model (same operand rounding, fp64 accumulation)
 ACTS = {"relu": 0, "gelu": 1, "tanh": 2, "silu": 3}
 
+
+def _rowsum_rounded(N, k):
+    """The weight-resident kernels (a_dim == 2, 128 < N <= 256) take the J0 row sums over the bf16 operand copy
+    of the state, the generic ones over the fp32 state; the rounding model follows the kernel under test."""
+    return k == 2 and 128 < N <= 256
+
+
 CASES = [
     # name,            B,   T,   k,  N,  act,   J0,     J1,  action
     ("config0",        64, 120,  2, 120, "tanh", -1 / 120, 1.0, "lr"),
@@ -69,7 +76,8 @@ def test_forward_trajectory_and_decoded_angle(case, gpu_device):
     assert np.isfinite(got).all()
     err = O.max_rel_err(got, ref)
     assert err <= TRAJ_TOL, f"trajectory error {err}"
-    model = OB.forward_backward(p["A"], p["Wa"], J0, J1, p["Wo"], p["r0"], 0.15, act)["bump_history"]
+    model = OB.forward_backward(p["A"], p["Wa"], J0, J1, p["Wo"], p["r0"], 0.15, act,
+                                rowsum_rounded=_rowsum_rounded(N, k))["bump_history"]
     assert O.max_rel_err(got, model) <= MODEL_TOL
     # per-step error must not blow up along the sequence either
     for t in (0, T // 2, T - 1):
@@ -111,7 +119,8 @@ def test_backward_weight_gradients(case, gpu_device):
     torch.cuda.synchronize()
     ref_hist, _ = O.forward_dense(p["A"], p["Wa"], J0, J1, p["Wo"], p["r0"], 0.15, act)
     ref = O.backward_dense(p["G"], p["A"], p["Wa"], J0, J1, p["Wo"], ref_hist, p["r0"], 0.15, act)
-    model = OB.forward_backward(p["A"], p["Wa"], J0, J1, p["Wo"], p["r0"], 0.15, act, p["G"])
+    model = OB.forward_backward(p["A"], p["Wa"], J0, J1, p["Wo"], p["r0"], 0.15, act, p["G"],
+                                rowsum_rounded=_rowsum_rounded(N, k))
     gWo, gWa = Wo.grad.cpu().numpy(), Wa.grad.cpu().numpy()
     assert np.isfinite(gWo).all() and np.isfinite(gWa).all()
     assert np.abs(ref["grad_Wo"]).max() > 0, "degenerate case: the reference gradient is identically zero"
@@ -177,9 +186,10 @@ def test_gradients_accumulate_and_are_deterministic(gpu_device):
         outs.append((gWa, gWo))
     torch.cuda.synchronize()
     assert torch.equal(outs[0][0], outs[1][0]) and torch.equal(outs[0][1], outs[1][1])     # bitwise repeatable
-    # accumulation: result = prefill + gradient (the rebuild path differs from the saved path by fp32 noise)
-    assert O.max_rel_err((outs[0][0] - 1.0).cpu().numpy(), Wa.grad.cpu().numpy()) <= 1e-3
-    assert O.max_rel_err((outs[0][1] - 2.0).cpu().numpy(), Wo.grad.cpu().numpy()) <= 1e-3
+    # accumulation: result = prefill + gradient.  The rebuild path recomputes F' with fp32 row sums of the stored
+    # history, the saved path took them over the bf16 operand copy: a difference at operand-rounding level.
+    assert O.max_rel_err((outs[0][0] - 1.0).cpu().numpy(), Wa.grad.cpu().numpy()) <= MODEL_TOL
+    assert O.max_rel_err((outs[0][1] - 2.0).cpu().numpy(), Wo.grad.cpu().numpy()) <= MODEL_TOL
 
 
 def test_alpha_zero_and_zero_weights_closed_forms(gpu_device):
