@@ -234,13 +234,14 @@ __global__ __launch_bounds__(512) void ring_fwd_res256_kernel(RingFwdArgs p) {
     gates_publish(gbuf, tid, B, bt, gs);
   }
 
-  // The LDS-resident slice is consumed in units of (tile cc, four K chunks), in the order
-  // (0,K0..3) (1,K0..3) (0,K4..7) (1,K4..7); while unit f is multiplied, unit f+1 is fetched into
-  // the other register buffer.
-  bf16x8 w0[2][HK];
-  auto unit_slot = [&](int f, int u) { return (((f & 1) * R_KCH) + (f >> 1) * HK + u) * 64; };
+  // The LDS-resident slice is consumed in units of (tile cc, two K chunks), eight per step in the
+  // order f = 4*ph + 2*cc + j -> chunks 4*ph + 2*j + {0,1}; while unit f is multiplied, unit f+1 is
+  // fetched into the other register buffer.
+  constexpr int UF = 2;
+  bf16x8 w0[2][UF];
+  auto unit_slot = [&](int f, int u) { return ((((f >> 1) & 1) * R_KCH) + (f >> 2) * HK + (f & 1) * UF + u) * 64; };
 #pragma unroll
-  for (int u = 0; u < HK; ++u) w0[0][u] = wl[unit_slot(0, u)];
+  for (int u = 0; u < UF; ++u) w0[0][u] = wl[unit_slot(0, u)];
   lds_barrier();   // A_0
 
   // History / F' / operand-copy stores of a finished step are not issued in one burst behind its
@@ -274,19 +275,16 @@ __global__ __launch_bounds__(512) void ring_fwd_res256_kernel(RingFwdArgs p) {
   };
 
   f32x4 P[2][3], S;
-  auto mfma_unit = [&](int f, const bf16x8 (&af)[HK], int ts, int slot, auto emit) {
-    const int cc = f & 1, ph = f >> 1, fn = (f + 1) & 3;
+  auto mfma_unit = [&](int f, const bf16x8 (&af)[HK]) {
+    const int cc = (f >> 1) & 1, ph = f >> 2, j = f & 1, fn = (f + 1) & 7;
 #pragma unroll
-    for (int u = 0; u < HK; ++u) w0[(f + 1) & 1][u] = wl[unit_slot(fn, u)];
+    for (int u = 0; u < UF; ++u) w0[(f + 1) & 1][u] = wl[unit_slot(fn, u)];
 #pragma unroll
-    for (int u = 0; u < HK; ++u) {
-      const int kc = ph * HK + u;
-      if constexpr (decltype(emit)::value) {
-        if (u == HK / 2) emit_store(ts, slot);
-      }
-      P[cc][0] = mfma16(af[u], w0[f & 1][u], P[cc][0]);
-      P[cc][1] = mfma16(af[u], wreg[0][cc][kc], P[cc][1]);
-      P[cc][2] = mfma16(af[u], wreg[1][cc][kc], P[cc][2]);
+    for (int u = 0; u < UF; ++u) {
+      const int kl = j * UF + u, kc = ph * HK + kl;
+      P[cc][0] = mfma16(af[kl], w0[f & 1][u], P[cc][0]);
+      P[cc][1] = mfma16(af[kl], wreg[0][cc][kc], P[cc][1]);
+      P[cc][2] = mfma16(af[kl], wreg[1][cc][kc], P[cc][2]);
     }
   };
   // K chunks 0..3 (ph = 0, from the E buffer of this step's parity) or 4..7 (ph = 1, from the L half);
@@ -304,10 +302,11 @@ __global__ __launch_bounds__(512) void ring_fwd_res256_kernel(RingFwdArgs p) {
     }
 #pragma unroll
     for (int u = 0; u < HK; ++u) S = mfma16(af[u], ones, S);
-    if constexpr (decltype(emit)::value) emit_store(ts, 4 * ph + 0);
-    mfma_unit(2 * ph, af, ts, 4 * ph + 1, emit);
-    if constexpr (decltype(emit)::value) emit_store(ts, 4 * ph + 2);
-    mfma_unit(2 * ph + 1, af, ts, 4 * ph + 3, emit);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      if constexpr (decltype(emit)::value) emit_store(ts, 4 * ph + j);
+      mfma_unit(4 * ph + j, af);
+    }
   };
   // x[e][cc] = J0*rowsum + J1*P0 + a0*P1 + a1*P2 with the gates of step t
   auto preactivation = [&](int t, float (&x)[4][2]) {
