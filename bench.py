@@ -2,6 +2,9 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu]
 
+Defaults: K = 1000 timed steps after W = 200 warm-up steps (about one second of GPU time): the chip's clocks
+take some tens of milliseconds of sustained load to settle, and a step is well under a millisecond.
+
 One "step" = one forward + one backward of the operator over one synthetic batch at
 N=256, B=4096, T=120, k=2, gelu (inputs resident in HBM before the timed region).
 Prints ONE JSON line: sample-steps/s (B*T per fwd+bwd), the roofline of the slowest kernel from
@@ -98,8 +101,8 @@ def cpu_baseline(cfg, sample_B, iters=8):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=1000)
+    ap.add_argument("--warmup", type=int, default=200)
     ap.add_argument("--workload", default="train_n256_b4096_t120_gelu", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the host-CPU baseline leg")
     ap.add_argument("--cpu-sample-batch", type=int, default=128)
