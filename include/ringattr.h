@@ -75,8 +75,10 @@ RINGATTR_API int ringattr_fwd(const void* A, const void* Wa, float J0, float J1,
 /* Reverse-time BPTT + weight gradients.
  * Replaces bwd_cuda (cpp/bwd.cu:4-52) and cpp/bwd.cpp:34-99.
  * `saved` may be NULL: F'(re) is then recomputed from bump_history.
- * grad_A [B,T,k] and grad_r_init [B,N] are optional outputs (NULL = skip); the
- * reference returns None for both (cpp/ring_rnn_cuda.py:144). */
+ * grad_A [B,T,k] and grad_r_init [B,N] are optional outputs (NULL = skip), written
+ * rather than accumulated; the reference returns None for both
+ * (cpp/ring_rnn_cuda.py:144).  Asking for grad_A (a_dim <= 48) adds one read of
+ * bump_history and runs the BPTT on the weight-streaming kernel for every N. */
 RINGATTR_API int ringattr_bwd(const void* grad_output, const void* A, const void* Wa, float J0, float J1,
                  const void* Wo, const void* bump_history, const void* r_init,
                  void* grad_Wa, void* grad_Wo, float alpha,

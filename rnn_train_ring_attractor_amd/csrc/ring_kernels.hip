@@ -52,10 +52,13 @@ __global__ __launch_bounds__(256) void ring_pack_weights_kernel(const float* __r
 // X is read as MFMA A-operand fragments from the LDS operand buffer, W_mm streams from the packed
 // global copy (L2 resident).  coef_0 = J1, coef_{1+j}[e] = A[b_e, t, j].
 // ------------------------------------------------------------------------------------------------
-template <int NC>
+// With GA, rp holds r_prev[row 4q+e][neuron tile c] and ga_part (k x 4 waves x 16 rows) receives, per action
+// matrix and batch row, this wave's share of  sum_j (X @ W_mm)[row][j] * r_prev[row][j]  (= dL/dA[b,t,mm-1]).
+template <int NC, bool GA = false>
 __device__ __forceinline__ void gated_products(const bf16x8* __restrict__ xb, const bf16x8* __restrict__ Wp,
                                                const float* __restrict__ A, int k, int T, int B, int t, int b0,
-                                               float J1, int w, int lane, f32x4 (&acc)[NC]) {
+                                               float J1, int w, int lane, f32x4 (&acc)[NC],
+                                               const float (*rp)[NC] = nullptr, float* ga_part = nullptr) {
   using TL = Tile<NC>;
   const int q = lane >> 4, n = lane & 15;
 #pragma unroll
@@ -95,6 +98,18 @@ __device__ __forceinline__ void gated_products(const bf16x8* __restrict__ xb, co
     for (int c = 0; c < NC; ++c)
 #pragma unroll
       for (int e = 0; e < 4; ++e) acc[c][e] += coef[e] * p[c][e];
+    if constexpr (GA) {
+      if (mm > 0) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          float d = 0.f;
+#pragma unroll
+          for (int c = 0; c < NC; ++c) d = fmaf(p[c][e], rp[e][c], d);
+          d = row16_sum(d);
+          if (n == 0) ga_part[((mm - 1) * 4 + w) * 16 + 4 * q + e] = d;
+        }
+      }
+    }
   }
 }
 
@@ -228,11 +243,24 @@ __global__ __launch_bounds__(256) void ring_rebuild_saved_kernel(RingFwdArgs p) 
 //   carry' = (1-alpha) G + J0 * sum_i g + J1 (g @ Wo) + sum_j A_j (g @ Wa_j)
 // legacy/bwd_fp32.py:86-109.  One barrier per step.
 // ------------------------------------------------------------------------------------------------
-template <int NC>
+// Sum the four waves' shares of one step in wave order and write grad_A[b, t, c] for the tile's 16 rows.
+__device__ __forceinline__ void bptt_flush_grad_A(const RingBpttArgs& p, const float* part, int t, int bt, int tid) {
+  for (int idx = tid; idx < 16 * p.k; idx += 256) {
+    const int c = idx >> 4, row = idx & 15, b = 16 * bt + row;
+    const float* s = part + c * 64 + row;
+    if (b < p.B) p.grad_A[((size_t)b * p.T + t) * p.k + c] = ((s[0] + s[16]) + s[32]) + s[48];
+  }
+}
+
+// GA: also produce grad_A[b,t,c] = sum_j (g Wa[c])[j] * r_prev[j].  The per-wave shares of a step go to
+// a double-buffered LDS array (dynamic shared memory, 2*k*64 floats) and are summed in wave order and
+// written out after the next step's barrier.
+template <int NC, bool GA>
 __global__ __launch_bounds__(256) void ring_bptt_kernel(RingBpttArgs p) {
   using TL = Tile<NC>;
   __shared__ bf16x8 xbuf[2][TL::SLOTS];
   __shared__ float psum[2][64];
+  extern __shared__ float ga_buf[];   // [2][k][4 waves][16 rows] when GA
 
   const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, q = lane >> 4, n = lane & 15;
   const int bt = blockIdx.x;
@@ -266,7 +294,16 @@ __global__ __launch_bounds__(256) void ring_bptt_kernel(RingBpttArgs p) {
     lds_barrier();
 
     f32x4 acc[NC];
-    gated_products<NC>(xbuf[cur], (const bf16x8*)p.Wpack, p.A, p.k, T, B, t, b0, p.J1, w, lane, acc);
+    if constexpr (GA) {
+      // the shares of step t+1 are complete (every wave passed the barrier above after writing them)
+      if (t + 1 < T) bptt_flush_grad_A(p, ga_buf + (cur ^ 1) * p.k * 64, t + 1, bt, tid);
+      float rp[4][NC];
+      rows_load<NC>(t == 0 ? p.r_init : p.hist + (size_t)(t - 1) * B * N, N, B, b0, i0, rp);
+      gated_products<NC, true>(xbuf[cur], (const bf16x8*)p.Wpack, p.A, p.k, T, B, t, b0, p.J1, w, lane, acc, rp,
+                               ga_buf + cur * p.k * 64);
+    } else {
+      gated_products<NC>(xbuf[cur], (const bf16x8*)p.Wpack, p.A, p.k, T, B, t, b0, p.J1, w, lane, acc);
+    }
     float s[4];
     read_rowsum(psum[cur], q, s);
 #pragma unroll
@@ -276,6 +313,10 @@ __global__ __launch_bounds__(256) void ring_bptt_kernel(RingBpttArgs p) {
         const bool ok = (b0 + e < B) && (i0 + c < N);
         carry[e][c] = ok ? (oma * G[e][c] + p.J0 * s[e] + acc[c][e]) : 0.f;
       }
+  }
+  if constexpr (GA) {
+    lds_barrier();
+    bptt_flush_grad_A(p, ga_buf + ((T - 1) & 1) * p.k * 64, 0, bt, tid);
   }
   if (p.grad_r_init) rows_store<NC>(p.grad_r_init, N, B, b0, i0, carry);
 }
@@ -514,8 +555,13 @@ hipError_t ring_launch_rebuild(const RingFwdArgs& a, int NCv, hipStream_t st) {
 
 hipError_t ring_launch_bptt(const RingBpttArgs& a, int NCv, hipStream_t st) {
   ProfScope prof(3, st);
+  if (a.grad_A) {   // the generic kernel is the one that also produces dL/dA
+    const size_t dyn = (size_t)2 * a.k * 64 * sizeof(float);
+    RING_DISPATCH_NC(NCv, hipLaunchKernelGGL((ring_bptt_kernel<NC, true>), dim3(a.nbt), dim3(256), dyn, st, a));
+    return hipGetLastError();
+  }
   if (ring_uses_resident(a.N, a.k)) return ring_launch_bptt_res256(a, st);
-  RING_DISPATCH_NC(NCv, hipLaunchKernelGGL(ring_bptt_kernel<NC>, dim3(a.nbt), dim3(256), 0, st, a));
+  RING_DISPATCH_NC(NCv, hipLaunchKernelGGL((ring_bptt_kernel<NC, false>), dim3(a.nbt), dim3(256), 0, st, a));
   return hipGetLastError();
 }
 

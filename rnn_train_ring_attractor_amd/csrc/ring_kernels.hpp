@@ -23,6 +23,9 @@ struct RingBpttArgs {
   const _Float16* dfrag;
   __bf16* gfrag;         // bf16 g in tile order (output)
   float* grad_r_init;    // [B,N] or null
+  float* grad_A;         // [B,T,k] or null (written, not accumulated); needs hist and r_init
+  const float* hist;     // [T,B,N] state history (r_prev of step t is hist[t-1]); only read for grad_A
+  const float* r_init;   // [B,N]
   float J0, J1, alpha;
   int N, k, T, B, nbt;
 };

@@ -157,10 +157,11 @@ int ringattr_bwd(const void* grad_output, const void* A, const void* Wa, float J
   if ((rc = check_act(activation_type))) return rc;
   if (!grad_output || !A || !Wa || !Wo || !bump_history || !r_init || !grad_Wa || !grad_Wo)
     return fail(RINGATTR_ERR_INVALID, "ringattr_bwd: null tensor pointer");
-  if (grad_A) return fail(RINGATTR_ERR_INVALID, "ringattr_bwd: grad_A output is not implemented yet; pass NULL");
+  if (grad_A && (size_t)2 * a_dim * 64 * sizeof(float) > 24 * 1024)
+    return fail(RINGATTR_ERR_INVALID, "ringattr_bwd: grad_A is supported for a_dim <= 48 (got %d)", a_dim);
   if (!aligned16(grad_output) || !aligned16(A) || !aligned16(Wa) || !aligned16(Wo) || !aligned16(bump_history) ||
       !aligned16(r_init) || !aligned16(grad_Wa) || !aligned16(grad_Wo) || !aligned16(saved) ||
-      !aligned16(grad_r_init) || !aligned16(workspace))
+      !aligned16(grad_r_init) || !aligned16(grad_A) || !aligned16(workspace))
     return fail(RINGATTR_ERR_INVALID, "ringattr_bwd: every pointer must be 16-byte aligned");
   const size_t need = ringattr_bwd_workspace_bytes(N, a_dim, seq_len, batch_size, saved != nullptr);
   if (!workspace || workspace_bytes < need)
@@ -221,6 +222,9 @@ int ringattr_bwd(const void* grad_output, const void* A, const void* Wa, float J
   b.dfrag = dfrag;
   b.gfrag = gfrag;
   b.grad_r_init = (float*)grad_r_init;
+  b.grad_A = (float*)grad_A;
+  b.hist = (const float*)bump_history;
+  b.r_init = (const float*)r_init;
   b.J0 = J0;
   b.J1 = J1;
   b.alpha = alpha;

@@ -39,7 +39,7 @@ class RingRnnCudaFunc(Function):
         bump_history = torch.empty(seq_len, batch_size, N, device=action_signal.device, dtype=action_signal.dtype)
 
         # F'(re) and the bf16 operand copy of r_prev are only worth writing when a backward will follow
-        needs_grad = ctx.needs_input_grad[1] or ctx.needs_input_grad[4]
+        needs_grad = any(ctx.needs_input_grad[i] for i in (0, 1, 4, 5))
         saved = None
         if needs_grad:
             saved = torch.empty(saved_nbytes(N, a_dim, seq_len, batch_size), dtype=torch.uint8,
@@ -56,7 +56,12 @@ class RingRnnCudaFunc(Function):
         action_signal, Wa, Wo, bump_history, r_init, saved = ctx.saved_tensors
         grad_Wa = torch.zeros_like(Wa)
         grad_Wo = torch.zeros_like(Wo)
+        # The reference returns None for action_signal and r_init (cpp/ring_rnn_cuda.py:144); here they get their
+        # gradients when the caller asked for them (gain networks in front of the op need dL/d action_signal).
+        grad_A = torch.empty_like(action_signal) if ctx.needs_input_grad[0] else None
+        grad_r0 = torch.empty_like(r_init) if ctx.needs_input_grad[5] else None
         bwd_cuda.bwd(grad_output=grad_output.contiguous(), A=action_signal, Wa=Wa, J0=ctx.J0, J1=ctx.J1, Wo=Wo,
                      bump_history=bump_history, r_init=r_init, grad_Wa=grad_Wa, grad_Wo=grad_Wo,
-                     alpha=ctx.alpha, activation_type=ctx.activation_type, saved=saved)
-        return None, grad_Wa, None, None, grad_Wo, None, None, None
+                     alpha=ctx.alpha, activation_type=ctx.activation_type, saved=saved, grad_A=grad_A,
+                     grad_r_init=grad_r0)
+        return grad_A, grad_Wa, None, None, grad_Wo, grad_r0, None, None

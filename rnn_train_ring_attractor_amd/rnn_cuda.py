@@ -14,7 +14,7 @@ Differences from the reference, all at the edges:
   * the reference's workspace tensors and cublas_handle are accepted and ignored -- the scratch
     this implementation needs is sized by the library and taken from torch's caching allocator;
   * optional keywords `saved=` (forward: buffer to fill; backward: buffer to consume),
-    `grad_r_init=` and `stream=`;
+    `grad_r_init=` [B,N] and `grad_A=` [B,T,a_dim] (both overwritten, not accumulated) and `stream=`;
   * work goes to torch's CURRENT stream, not the legacy default stream;
   * importing this module needs no GPU; calling it does (RuntimeError otherwise).
 """
@@ -130,7 +130,7 @@ class _Bwd:
     def bwd(grad_output, A, Wa, J0, J1, Wo, bump_history, re_history=None, r_init=None, grad_Wa=None, grad_Wo=None,
             alpha=None, activation_type=None, grad_r=None, W_eff_temp=None, grad_re_temp=None,
             grad_W_eff_temp_bf16=None, A_t_temp_bf16=None, grad_re_temp_T=None, cublas_handle=None,
-            saved=None, grad_r_init=None, stream=None):
+            saved=None, grad_r_init=None, grad_A=None, stream=None):
         for name, t in (("grad_output", grad_output), ("A", A), ("Wa", Wa), ("Wo", Wo),
                         ("bump_history", bump_history), ("r_init", r_init), ("grad_Wa", grad_Wa), ("grad_Wo", grad_Wo)):
             _contig(name, t)
@@ -151,6 +151,8 @@ class _Bwd:
                  ("grad_Wa", grad_Wa, (k, N, N)), ("grad_Wo", grad_Wo, (N, N))]
         if grad_r_init is not None:
             specs.append(("grad_r_init", grad_r_init, (B, N)))
+        if grad_A is not None:
+            specs.append(("grad_A", grad_A, (B, T, k)))
         _f32_cuda(specs)
         lib = _lib.load()
         if saved is not None:
@@ -165,7 +167,8 @@ class _Bwd:
             ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
             rc = lib.ringattr_bwd(_ptr(grad_output), _ptr(A), _ptr(Wa), J0, J1, _ptr(Wo), _ptr(bump_history),
                                   _ptr(r_init), _ptr(grad_Wa), _ptr(grad_Wo), alpha, N, k, T, B, act,
-                                  _ptr(saved), None, _ptr(grad_r_init), _ptr(ws), ws_bytes, _stream_ptr(stream, dev))
+                                  _ptr(saved), _ptr(grad_A), _ptr(grad_r_init), _ptr(ws), ws_bytes,
+                                  _stream_ptr(stream, dev))
         _lib.check(rc)
         return None
 

@@ -60,7 +60,10 @@ def test_c_abi_rejects_bad_arguments_with_codes_not_exit():
     assert lib.ringattr_fwd(*bad_shape, 0, None, p, 1 << 20, None) == 1
     bwd_args = [p, p, p, 0.0, 1.0, p, p, p, p, p, 0.15, 64, 2, 4, 16, 0]
     assert lib.ringattr_bwd(*bwd_args, None, None, None, p, 16, None) == 2
-    assert lib.ringattr_bwd(*bwd_args, None, p, None, p, 1 << 30, None) == 1 and "grad_A" in _lib.last_error()
+    wide = list(bwd_args)
+    wide[12] = 64                                                       # a_dim beyond what the grad_A path stages in LDS
+    assert lib.ringattr_bwd(*wide, None, p, None, p, 1 << 30, None) == 1 and "grad_A" in _lib.last_error()
+    assert lib.ringattr_bwd(*bwd_args, None, p + 4, None, p, 1 << 30, None) == 1 and "aligned" in _lib.last_error()
     assert lib.ringattr_profile_read(None, None) == 1
     with pytest.raises(ValueError):
         _lib.check(1)

@@ -169,6 +169,33 @@ def test_backward_without_saved_buffer_rebuilds_it(case, gpu_device):
     assert O.max_rel_err(g0.cpu().numpy(), ref["grad_r_init"]) <= GRAD_TOL
 
 
+@pytest.mark.parametrize("B,T,k,N,act,action", [(40, 24, 2, 120, "tanh", "lr"), (48, 20, 2, 256, "gelu", "lr"),
+                                                (21, 9, 3, 200, "silu", "dense"), (32, 12, 16, 64, "tanh", "spread")],
+                         ids=["n120", "n256", "ragged_k3", "k16"])
+def test_gradients_of_action_signal_and_initial_state(B, T, k, N, act, action, gpu_device):
+    """dL/d action_signal and dL/d r_init, which the reference operator does not return (cpp/ring_rnn_cuda.py:144);
+    pinned by the fp64 oracle, whose grad_A / grad_r_init are themselves checked by finite differences."""
+    from rnn_train_ring_attractor_amd import ring_rnn_cuda_func
+    print(f"[case] grad_A B={B} T={T} k={k} N={N} {act}", flush=True)
+    p = _problem(400, B, T, k, N, action)
+    J0, J1 = -0.05, 0.4
+    A = _dev(p["A"], gpu_device).requires_grad_(True)
+    r0 = _dev(p["r0"], gpu_device).requires_grad_(True)
+    Wa = _dev(p["Wa"], gpu_device).requires_grad_(True)
+    Wo = _dev(p["Wo"], gpu_device).requires_grad_(True)
+    hist = ring_rnn_cuda_func(A, Wa, J0, J1, Wo, r0, 0.15, act)
+    hist.backward(_dev(p["G"], gpu_device))
+    torch.cuda.synchronize()
+    ref_hist, _ = O.forward_dense(p["A"], p["Wa"], J0, J1, p["Wo"], p["r0"], 0.15, act)
+    ref = O.backward_dense(p["G"], p["A"], p["Wa"], J0, J1, p["Wo"], ref_hist, p["r0"], 0.15, act)
+    for name, got, want in (("grad_A", A.grad, ref["grad_A"]), ("grad_r_init", r0.grad, ref["grad_r_init"]),
+                            ("grad_Wo", Wo.grad, ref["grad_Wo"]), ("grad_Wa", Wa.grad, ref["grad_Wa"])):
+        got = got.cpu().numpy()
+        assert got.shape == want.shape and np.isfinite(got).all(), name
+        assert O.cosine(got, want) >= GRAD_COS, name
+        assert O.max_rel_err(got, want) <= GRAD_TOL, name
+
+
 def test_gradients_accumulate_and_are_deterministic(gpu_device):
     from rnn_train_ring_attractor_amd import bwd_cuda
     B, T, k, N = 48, 20, 2, 256
