@@ -179,3 +179,59 @@ class GeneralizedRingAttractorNoGain(nn.Module):
                                   r_init=r_init, alpha=0.15, activation=self.activation_name).permute(1, 0, 2)
         proj = bump @ self.W_delta7
         return (proj / proj.max(dim=2, keepdim=True)[0]).clone(), bump.clone()
+
+
+class LeakyRingAttractor(nn.Module):
+    """The two-channel model with learned input gains (reference: train/train_ring_attractor.py:55-187):
+    L = gain_l(relu(-av)) * relu(-av), R = gain_r(relu(av)) * relu(av), each gain a 1 -> h -> 1 MLP (GELU hidden,
+    softplus output) applied per sample and step, then the leaky recurrence with [Wl, Wr] through the HIP operator.
+    The operator returns dL/d action_signal, so the gain networks train through it.  Parameter names follow the
+    reference (Wo, Wl, Wr, gain_r_net, gain_l_net); 'debug_perfect' fixes the weights and bypasses the gains."""
+
+    def __init__(self, num_neurons, tau=10.0, dt=1.0, activation="tanh", initialization="random", hidden_gain_neurons=16):
+        super().__init__()
+        self.num_neurons, self.tau, self.dt = num_neurons, tau, dt
+        self.activation_name, self.initialization = activation, initialization
+
+        def gain_net():
+            return nn.Sequential(nn.Linear(1, hidden_gain_neurons), nn.GELU(), nn.Linear(hidden_gain_neurons, 1),
+                                 nn.Softplus())
+
+        self.gain_r_net, self.gain_l_net = gain_net(), gain_net()
+        idx = torch.arange(num_neurons, dtype=torch.float32)
+        diff = 2 * math.pi * (idx[:, None] - idx[None, :]) / num_neurons
+        self.register_buffer("W_delta7", torch.cos(diff))
+        self.J0, self.J1 = -0.1, 0.1
+        if initialization == "random":
+            scale = 1.0 / math.sqrt(num_neurons)
+            self.Wo = nn.Parameter(torch.randn(num_neurons, num_neurons) * scale)
+            self.Wl = nn.Parameter(torch.randn(num_neurons, num_neurons) * scale)
+            self.Wr = nn.Parameter(torch.randn(num_neurons, num_neurons) * scale)
+        elif initialization in ("perfect", "debug_perfect"):
+            learn = initialization == "perfect"
+            if not learn:
+                self.gain_r_net = self.gain_l_net = None
+            self.Wo = nn.Parameter(torch.cos(diff), requires_grad=learn)
+            self.Wl = nn.Parameter(torch.cos(diff + math.pi / 4), requires_grad=learn)
+            self.Wr = nn.Parameter(torch.cos(diff - math.pi / 4), requires_grad=learn)
+        else:
+            raise ValueError(f"Unknown initialization type: {initialization}")
+
+    def action_signal(self, av_signal):
+        """[B,T] angular velocity -> [B,T,2] gated (L, R) channels."""
+        left, right = torch.relu(-av_signal).unsqueeze(2), torch.relu(av_signal).unsqueeze(2)
+        if self.gain_l_net is not None:
+            left, right = self.gain_l_net(left) * left, self.gain_r_net(right) * right
+        return torch.cat([left, right], dim=2)
+
+    def forward(self, av_signal, r_init=None):
+        from .ring_rnn_cuda import ring_rnn_cuda_func
+        batch_size = av_signal.shape[0]
+        if r_init is None:
+            angle = torch.full((batch_size,), math.pi, device=self.Wo.device)
+            r_init = create_initial_bump(angle, self.num_neurons, device=self.Wo.device)
+        bump = ring_rnn_cuda_func(action_signal=self.action_signal(av_signal), Wa=torch.stack([self.Wl, self.Wr]),
+                                  J0=self.J0, J1=self.J1, Wo=self.Wo, r_init=r_init, alpha=0.15,
+                                  activation=self.activation_name).permute(1, 0, 2)
+        proj = bump @ self.W_delta7
+        return proj / proj.max(dim=2, keepdim=True)[0], bump

@@ -120,6 +120,45 @@ def test_streaming_and_resident_kernels_agree(gpu_device, monkeypatch):
     assert O.max_rel_err(outs["0"][2], model["grad_Wo"]) <= 5e-3
 
 
+def test_gain_network_model_trains_through_the_operator(gpu_device):
+    """The general ring with gain networks (reduced size; tanh, because relu with the model's fixed J0 = -0.1 and
+    random weights silences every neuron and all gradients vanish): gain-MLP gradients reach the parameters through
+    dL/d action_signal.  Checked against CPU autograd of the torch port with the same parameters."""
+    from oracle import torch_port as TP
+    from rnn_train_ring_attractor_amd import host
+    print("[case] gain-network model N=256 B=64 T=40 tanh", flush=True)
+    torch.manual_seed(5)
+    N, B, T = 256, 64, 40
+    model = host.LeakyRingAttractor(N, activation="tanh", initialization="random")
+    av, angle = host.generate_av_integration_data_ultra_fast(B, T)
+    r0 = host.create_initial_bump(angle[:, 0], N)
+
+    def loss_of(r_hist, bump):
+        return host.cosine_similarity_loss(r_hist, angle.to(r_hist.device)) + 0.2 * host.bump_amplitude_loss(bump)
+
+    # CPU reference: same module parameters, recurrence by the torch port, autograd end to end
+    A_cpu = model.action_signal(av)
+    bump_cpu = TP.ring_forward(A_cpu, torch.stack([model.Wl, model.Wr]), model.J0, model.J1, model.Wo, r0, 0.15,
+                               "tanh").permute(1, 0, 2)
+    proj = bump_cpu @ model.W_delta7
+    loss_cpu = loss_of(proj / proj.max(dim=2, keepdim=True)[0], bump_cpu)
+    loss_cpu.backward()
+    want = {n: p.grad.clone() for n, p in model.named_parameters()}
+    model.zero_grad()
+
+    model.to(gpu_device)
+    r_hist, bump = model(av.to(gpu_device), r0.to(gpu_device))
+    loss = loss_of(r_hist, bump)
+    loss.backward()
+    torch.cuda.synchronize()
+    assert abs(float(loss) - float(loss_cpu)) <= 1e-2 * abs(float(loss_cpu))
+    for n, p in model.named_parameters():
+        got, ref = p.grad.cpu().numpy(), want[n].numpy()
+        assert np.isfinite(got).all(), n
+        assert O.cosine(got, ref) >= 0.999, n
+        assert O.max_rel_err(got, ref) <= 2e-2, n
+
+
 def test_training_driver_reduces_loss(gpu_device):
     """The reference-style driver (same imports and call pattern) trains on the HIP operator."""
     import train_general_ring_no_gain as drv
