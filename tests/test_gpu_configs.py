@@ -120,6 +120,28 @@ def test_streaming_and_resident_kernels_agree(gpu_device, monkeypatch):
     assert O.max_rel_err(outs["0"][2], model["grad_Wo"]) <= 5e-3
 
 
+@pytest.mark.parametrize("T", [1, 2, 3, 32, 33, 64, 65])
+def test_sequence_length_edges_of_the_resident_kernels(T, gpu_device):
+    """Sequence lengths around the kernels' internal boundaries (first/last step peeling, paired time steps,
+    gate chunks of 32 steps) with a ragged batch, forward and backward."""
+    from rnn_train_ring_attractor_amd import ring_rnn_cuda_func
+    B, k, N = 17, 2, 256
+    print(f"[case] sequence edge T={T}", flush=True)
+    p = make_problem(50 + T, B, T, k, N)
+    Wa = _t(p["Wa"], gpu_device).requires_grad_(True)
+    Wo = _t(p["Wo"], gpu_device).requires_grad_(True)
+    r0 = _t(p["r0"], gpu_device).requires_grad_(True)
+    h = ring_rnn_cuda_func(_t(p["A"], gpu_device), Wa, -0.1, 0.4, Wo, r0, 0.15, "gelu")
+    h.backward(_t(p["G"], gpu_device))
+    torch.cuda.synchronize()
+    ref_hist, _ = O.forward_dense(p["A"], p["Wa"], -0.1, 0.4, p["Wo"], p["r0"], 0.15, "gelu")
+    ref = O.backward_dense(p["G"], p["A"], p["Wa"], -0.1, 0.4, p["Wo"], ref_hist, p["r0"], 0.15, "gelu")
+    assert O.max_rel_err(h.detach().cpu().numpy(), ref_hist) <= TRAJ_TOL
+    for key, got in (("grad_Wo", Wo.grad), ("grad_Wa", Wa.grad), ("grad_r_init", r0.grad)):
+        assert O.cosine(got.cpu().numpy(), ref[key]) >= 0.999, key
+        assert O.max_rel_err(got.cpu().numpy(), ref[key]) <= 2e-2, key
+
+
 def test_gain_network_model_trains_through_the_operator(gpu_device):
     """The general ring with gain networks (reduced size; tanh, because relu with the model's fixed J0 = -0.1 and
     random weights silences every neuron and all gradients vanish): gain-MLP gradients reach the parameters through
