@@ -10,7 +10,7 @@ Rounding points (same math as ring_oracle.forward_dense / backward_dense, which 
   * weights [Wo|Wa]            -> bf16   (MFMA B operand)
   * r_prev, g as contraction operands -> bf16 (MFMA A operand); the leak term, the J0 row sums and
     the state carried between steps stay unrounded
-  * F'(re) kept for the backward -> fp16
+  * alpha * F'(re) kept for the backward -> fp16
   * A_c * g in the weight-gradient contraction -> bf16
 Pinned by tests/test_oracle_bf16.py: with rounding switched off it reproduces ring_oracle exactly.
 """
@@ -69,7 +69,7 @@ def forward_backward(A, Wa, J0, J1, Wo, r_init, alpha, activation_name, grad_out
         re = J0 * (rb if rowsum_rounded else r).sum(axis=1, keepdims=True) + J1 * (rb @ Wob.T)
         for c in range(k):
             re = re + A[:, t, c:c + 1] * (rb @ Wab[c].T)
-        D[t] = rf16(O.activation_derivative(re, activation_name))
+        D[t] = rf16(alpha * O.activation_derivative(re, activation_name))   # the kernels save alpha * F'
         r = (1.0 - alpha) * r + alpha * O.activation(re, activation_name)
         hist[t] = r
     out = {"bump_history": hist}
@@ -81,7 +81,7 @@ def forward_backward(A, Wa, J0, J1, Wo, r_init, alpha, activation_name, grad_out
     carry = np.zeros((B, N))
     for t in range(T - 1, -1, -1):
         G = G_out[t] + carry
-        g = alpha * D[t] * G
+        g = D[t] * G
         gb = rb16(g)
         carry = (1.0 - alpha) * G + J0 * (gb if rowsum_rounded else g).sum(axis=1, keepdims=True) + J1 * (gb @ Wob)
         for c in range(k):

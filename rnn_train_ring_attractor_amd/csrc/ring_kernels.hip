@@ -13,13 +13,14 @@
 //   out[mm][w][c][kc][lane][8]; lane (q,n) owns output column 16*NC*w + NC*n + c and the eight
 //   contraction indices 32kc+8q .. +7.  transposed = 0: value = W[col][contr] (forward, re = W r);
 //   transposed = 1: value = W[contr][col] (backward, g @ W).
+//   scale0 multiplies matrix 0 (Wo) before rounding: kernels that fold J1 into the weights pass J1.
 //   split_k = 1 (NC = 4 only): contraction position kappa stands for neuron split_k_neuron(kappa), the
 //   order the pipelined weight-resident kernels keep their operand tile in.
 // ------------------------------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void ring_pack_weights_kernel(const float* __restrict__ Wo,
                                                                 const float* __restrict__ Wa,
                                                                 bf16x8* __restrict__ out, int N, int k, int NC,
-                                                                int transposed, int split_k) {
+                                                                int transposed, int split_k, float scale0) {
   const int KCH = 2 * NC;
   const size_t total = (size_t)(1 + k) * 4 * NC * KCH * 64;
   for (size_t u = (size_t)blockIdx.x * blockDim.x + threadIdx.x; u < total; u += (size_t)gridDim.x * blockDim.x) {
@@ -41,7 +42,7 @@ __global__ __launch_bounds__(256) void ring_pack_weights_kernel(const float* __r
       const int kk = split_k ? split_k_neuron(k0 + x) : k0 + x;
       float val = 0.f;
       if (col < N && kk < N) val = transposed ? W[(size_t)kk * N + col] : W[(size_t)col * N + kk];
-      pk[x] = (__bf16)val;
+      pk[x] = (__bf16)(mm == 0 ? val * scale0 : val);
     }
     out[u] = pk;
   }
@@ -181,7 +182,7 @@ __global__ __launch_bounds__(256) void ring_fwd_kernel(RingFwdArgs p) {
         act_eval(p.act, x, F, D);
         const bool ok = (b0 + e < B) && (i0 + c < N);
         r[e][c] = ok ? (oma * r[e][c] + p.alpha * F) : 0.f;
-        d[e][c] = ok ? D : 0.f;
+        d[e][c] = ok ? p.alpha * D : 0.f;   // the saved record is alpha * F'(re)
       }
     }
     rows_store<NC>(p.hist + (size_t)t * B * N, N, B, b0, i0, r);
@@ -231,7 +232,7 @@ __global__ __launch_bounds__(256) void ring_rebuild_saved_kernel(RingFwdArgs p) 
     for (int c = 0; c < NC; ++c) {
       float F, D;
       act_eval(p.act, acc[c][e] + p.J0 * s[e], F, D);
-      d[e][c] = ((b0 + e < B) && (i0 + c < N)) ? D : 0.f;
+      d[e][c] = ((b0 + e < B) && (i0 + c < N)) ? p.alpha * D : 0.f;
     }
   }
   side_store<NC, f16x4, _Float16>(p.dfrag + side_offset<NC>(t, p.nbt, bt, w, lane), d);
@@ -239,7 +240,7 @@ __global__ __launch_bounds__(256) void ring_rebuild_saved_kernel(RingFwdArgs p) 
 
 // ------------------------------------------------------------------------------------------------
 // BPTT recurrence, reverse time.  carry = dL/dr_t flowing in from later steps (fp32 registers).
-//   G = carry + grad_output[t];  g = alpha * F'(re_t) * G  (bf16 copy -> LDS operand + gfrag)
+//   G = carry + grad_output[t];  g = (alpha * F'(re_t)) * G  (saved record; bf16 copy -> LDS operand + gfrag)
 //   carry' = (1-alpha) G + J0 * sum_i g + J1 (g @ Wo) + sum_j A_j (g @ Wa_j)
 // legacy/bwd_fp32.py:86-109.  One barrier per step.
 // ------------------------------------------------------------------------------------------------
@@ -286,7 +287,7 @@ __global__ __launch_bounds__(256) void ring_bptt_kernel(RingBpttArgs p) {
 #pragma unroll
       for (int c = 0; c < NC; ++c) {
         G[e][c] += carry[e][c];
-        g[e][c] = p.alpha * g[e][c] * G[e][c];
+        g[e][c] = g[e][c] * G[e][c];   // the saved record already carries alpha
       }
     write_operand<NC>(xbuf[cur], g, w, q, n);
     publish_rowsum<NC>(psum[cur], g, w, q, n);
@@ -523,13 +524,13 @@ hipError_t ring_profile_collect(double* ms, long long* launches) {
   }
 
 hipError_t ring_launch_pack(const float* Wo, const float* Wa, void* out, int N, int k, int NC, int transposed,
-                            int split_k, hipStream_t st) {
+                            int split_k, float scale0, hipStream_t st) {
   if (split_k && NC != 4) return hipErrorInvalidValue;
   const size_t total = (size_t)(1 + k) * 4 * NC * 2 * NC * 64;
   const int blocks = (int)((total + 255) / 256 < 4096 ? (total + 255) / 256 : 4096);
   ProfScope prof(0, st);
   hipLaunchKernelGGL(ring_pack_weights_kernel, dim3(blocks), dim3(256), 0, st, Wo, Wa, (bf16x8*)out, N, k, NC,
-                     transposed, split_k);
+                     transposed, split_k, scale0);
   return hipGetLastError();
 }
 

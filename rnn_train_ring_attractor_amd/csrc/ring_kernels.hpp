@@ -42,7 +42,7 @@ struct RingDwArgs {
 };
 
 hipError_t ring_launch_pack(const float* Wo, const float* Wa, void* out, int N, int k, int NC, int transposed,
-                            int split_k, hipStream_t st);
+                            int split_k, float scale0, hipStream_t st);
 hipError_t ring_launch_fwd(const RingFwdArgs& a, int NC, hipStream_t st);
 hipError_t ring_launch_rebuild(const RingFwdArgs& a, int NC, hipStream_t st);
 hipError_t ring_launch_bptt(const RingBpttArgs& a, int NC, hipStream_t st);

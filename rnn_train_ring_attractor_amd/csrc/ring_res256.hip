@@ -17,7 +17,7 @@ constexpr int R_KCH = 8;
 constexpr int R_WLDS_SLOTS = 4 * R_NC * R_KCH * 64;   // 16-byte slots of the LDS-resident matrix
 constexpr int R_XSLOTS = R_KCH * 4 * XG;
 constexpr int R_GCH = 32;                             // time steps of action gates staged per LDS chunk
-constexpr size_t R_LDS_BYTES = (size_t)(R_WLDS_SLOTS + 2 * R_XSLOTS) * 16 + 2 * 64 * 4 + 2 * R_GCH * 16 * 8;   // BPTT layout (the forward uses less)
+constexpr size_t R_LDS_BYTES = (size_t)(R_WLDS_SLOTS + 2 * R_XSLOTS) * 16 + 2 * R_GCH * 16 * 8;   // BPTT layout
 
 // Cheap activation pairs (F, F') for the per-step critical path.
 //  gelu: Phi via the Abramowitz-Stegun 7.1.26 erfc polynomial (|err| < 1.5e-7), sharing exp(-x^2/2)
@@ -51,30 +51,6 @@ __device__ __forceinline__ void act_fast(float x, float& F, float& D) {
     F = x * s;
     D = s * fmaf(x, 1.f - s, 1.f);
   }
-}
-
-__device__ __forceinline__ float dpp_row_sum(float v) {
-  // butterfly over the 16 lanes of a DPP row: quad_perm [1,0,3,2], [2,3,0,1], row_half_mirror, row_mirror
-  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, false));
-  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, false));
-  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xF, 0xF, false));
-  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x140, 0xF, 0xF, false));
-  return v;
-}
-
-__device__ __forceinline__ void publish_rowsum4(float* psum, const float (&v)[4][R_NC], int w, int q, int n) {
-  f32x4 s;
-#pragma unroll
-  for (int e = 0; e < 4; ++e) s[e] = dpp_row_sum((v[e][0] + v[e][1]) + (v[e][2] + v[e][3]));
-  if (n == 0) *reinterpret_cast<f32x4*>(psum + w * 16 + 4 * q) = s;
-}
-
-__device__ __forceinline__ f32x4 read_rowsum4(const float* psum, int q) {
-  const f32x4 a = *reinterpret_cast<const f32x4*>(psum + 0 * 16 + 4 * q);
-  const f32x4 b = *reinterpret_cast<const f32x4*>(psum + 1 * 16 + 4 * q);
-  const f32x4 c = *reinterpret_cast<const f32x4*>(psum + 2 * 16 + 4 * q);
-  const f32x4 d = *reinterpret_cast<const f32x4*>(psum + 3 * 16 + 4 * q);
-  return ((a + b) + c) + d;
 }
 
 // Action gates (A[b,t,0], A[b,t,1]) reach the lanes through LDS in chunks of R_GCH steps, so the
@@ -336,7 +312,7 @@ __global__ __launch_bounds__(512) void ring_fwd_res256_kernel(RingFwdArgs p) {
           D *= okf[e][cc];
         }
         r[e][cc] = rn;
-        d[e][cc] = D;
+        d[e][cc] = alpha * D;   // the saved record is alpha * F'(re)
       }
   };
   constexpr std::true_type with_stores{};
@@ -451,19 +427,21 @@ __global__ __launch_bounds__(256) void ring_bptt_res256_kernel(RingBpttArgs p) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
   bf16x8* wlds = reinterpret_cast<bf16x8*>(smem);
   bf16x8* xbuf = wlds + R_WLDS_SLOTS;
-  float* psum = reinterpret_cast<float*>(xbuf + 2 * R_XSLOTS);
-  f32x2* gbuf = reinterpret_cast<f32x2*>(psum + 2 * 64);
+  f32x2* gbuf = reinterpret_cast<f32x2*>(xbuf + 2 * R_XSLOTS);
 
   const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, q = lane >> 4, n = lane & 15;
   const int bt = blockIdx.x;
   const int b0 = 16 * bt + 4 * q;
   const int i0 = 16 * R_NC * w + R_NC * n;
   const int N = p.N, B = p.B, T = p.T;
-  const float oma = 1.f - p.alpha, alpha = p.alpha, J0 = p.J0, J1 = p.J1;
+  const float oma = 1.f - p.alpha, J0 = p.J0;   // alpha rides in the saved F' record, J1 in the packed Wo fragments
 
   bf16x8 wreg[2][R_NC][R_KCH];
   bf16x8* wl = wlds + (size_t)w * R_NC * R_KCH * 64 + lane;
   load_resident(reinterpret_cast<const bf16x8*>(p.Wpack), wl, wreg, w, lane);
+  bf16x8 ones;
+#pragma unroll
+  for (int x = 0; x < 8; ++x) ones[x] = (__bf16)1.0f;
 
   float carry[4][R_NC];
   float okf[4][R_NC];
@@ -505,11 +483,10 @@ __global__ __launch_bounds__(256) void ring_bptt_res256_kernel(RingBpttArgs p) {
 #pragma unroll
         for (int c = 0; c < R_NC; ++c) {
           G[e][c] = S.G[e][c] + carry[e][c];
-          g[e][c] = alpha * stage_dact(S, e, c) * G[e][c];
+          g[e][c] = stage_dact(S, e, c) * G[e][c];
         }
       bf16x8* xb = xbuf + cur * R_XSLOTS;
       write_operand<R_NC>(xb, g, w, q, n);
-      publish_rowsum4(psum + cur * 64, g, w, q, n);
       pair_store<R_NC>(p.gfrag, t, p.nbt, bt, w, lane, g);
       bptt_stage_load<FULL>(p, t - 2, bt, w, lane, b0, i0, S);
       lds_barrier();
@@ -517,7 +494,11 @@ __global__ __launch_bounds__(256) void ring_bptt_res256_kernel(RingBpttArgs p) {
       bf16x8 af[R_KCH];
 #pragma unroll
       for (int kc = 0; kc < R_KCH; ++kc) af[kc] = xb[(kc * 4 + q) * XG + n];
-      const f32x4 s = read_rowsum4(psum + cur * 64, q);
+      // J0 * (row sums of g) from the matrix pipe: g x ones puts every row's sum in all 16 columns
+      f32x4 js = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int kc = 0; kc < R_KCH; ++kc) js = mfma16(af[kc], ones, js);
+      js *= J0;
       f32x2 gate[4];
       {
         const f32x2* gb = gbuf + ((ci & 1) * R_GCH + l) * 16 + 4 * q;
@@ -526,7 +507,9 @@ __global__ __launch_bounds__(256) void ring_bptt_res256_kernel(RingBpttArgs p) {
       }
 #pragma unroll
       for (int c = 0; c < R_NC; ++c) {
-        f32x4 P0 = {0.f, 0.f, 0.f, 0.f}, P1 = P0, P2 = P0;
+        // the ungated chain starts from the terms that need no product: (1 - alpha) * G + J0 * sum(g)
+        f32x4 P0 = {fmaf(oma, G[0][c], js[0]), fmaf(oma, G[1][c], js[1]), fmaf(oma, G[2][c], js[2]), fmaf(oma, G[3][c], js[3])};
+        f32x4 P1 = {0.f, 0.f, 0.f, 0.f}, P2 = P1;
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
           // stage the next half tile of the LDS-resident matrix (wraps to tile 0 of the next step)
@@ -544,9 +527,7 @@ __global__ __launch_bounds__(256) void ring_bptt_res256_kernel(RingBpttArgs p) {
         }
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-          float x = fmaf(oma, G[e][c], J0 * s[e]);
-          x = fmaf(J1, P0[e], x);
-          x = fmaf(gate[e][0], P1[e], x);
+          float x = fmaf(gate[e][0], P1[e], P0[e]);
           x = fmaf(gate[e][1], P2[e], x);
           if constexpr (!FULL) x *= okf[e][c];
           carry[e][c] = x;

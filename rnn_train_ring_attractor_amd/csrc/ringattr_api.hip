@@ -123,7 +123,7 @@ int ringattr_fwd(const void* A, const void* Wa, float J0, float J1, const void* 
                 workspace ? workspace_bytes : (size_t)0);
   hipStream_t st = static_cast<hipStream_t>(stream);
 
-  hipError_t e = ring_launch_pack((const float*)Wo, (const float*)Wa, workspace, N, a_dim, g.NC, 0, ring_uses_resident(N, a_dim) ? 1 : 0, st);
+  hipError_t e = ring_launch_pack((const float*)Wo, (const float*)Wa, workspace, N, a_dim, g.NC, 0, ring_uses_resident(N, a_dim) ? 1 : 0, 1.f, st);
   if (e != hipSuccess) return hip_fail(e, "pack weights");
 
   RingFwdArgs a;
@@ -188,7 +188,7 @@ int ringattr_bwd(const void* grad_output, const void* A, const void* Wa, float J
     _Float16* d = (_Float16*)ws;
     ws += g.side_bytes;
     __bf16* r = (__bf16*)ws;
-    hipError_t e = ring_launch_pack((const float*)Wo, (const float*)Wa, wf, N, a_dim, g.NC, 0, 0, st);
+    hipError_t e = ring_launch_pack((const float*)Wo, (const float*)Wa, wf, N, a_dim, g.NC, 0, 0, 1.f, st);
     if (e != hipSuccess) return hip_fail(e, "pack weights");
     RingFwdArgs f;
     f.A = (const float*)A;
@@ -212,7 +212,9 @@ int ringattr_bwd(const void* grad_output, const void* A, const void* Wa, float J
     rfrag = r;
   }
 
-  hipError_t e = ring_launch_pack((const float*)Wo, (const float*)Wa, wb, N, a_dim, g.NC, 1, 0, st);
+  // the weight-resident BPTT kernel takes J1 folded into the transposed Wo fragments
+  const bool bptt_resident = ring_uses_resident(N, a_dim) && !grad_A;
+  hipError_t e = ring_launch_pack((const float*)Wo, (const float*)Wa, wb, N, a_dim, g.NC, 1, 0, bptt_resident ? J1 : 1.f, st);
   if (e != hipSuccess) return hip_fail(e, "pack transposed weights");
 
   RingBpttArgs b;
