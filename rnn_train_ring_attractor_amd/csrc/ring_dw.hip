@@ -7,7 +7,10 @@
 // accumulators (192 accumulation VGPRs).  A K chunk is 16 batch rows x 2 time steps (32 samples, one
 // MFMA K).  The paired tile-major operand buffers hold every tile of a chunk as 1 KiB of ready-made
 // MFMA fragments, so nothing is ever transposed or repacked:
-//   * the wave's own two g fragments and its action gates load straight into registers;
+//   * the wave's own two g fragments load straight into registers;
+//   * the action gates of a chunk (16 rows x 2 steps x up to 3 matrices) are fetched one value per
+//     thread and handed round through a small LDS stage next to the r_prev one: per-lane gate loads
+//     (eight scattered 4-byte loads per wave and chunk) cost more than the whole gating arithmetic;
 //   * the eight r_prev fragments every wave needs are copied verbatim into a double-buffered LDS
 //     stage once per workgroup (8 KiB per chunk) and read back with conflict-free ds_read_b128 --
 //     L2 -> CU traffic stays at 16 KiB per chunk and the LDS pipe at 40 KiB, both under the MFMA time.
@@ -27,7 +30,7 @@ template <int NG>
 struct DwStage {
   bf16x8 a[DW_WI];                    // g fragments of the wave's row tiles
   f32x4 bpart[2];                     // this thread's two fragments of the chunk's r_prev block (LDS stage)
-  f32x2 gate[NG > 0 ? NG : 1][4];     // per gated matrix and batch row 4q+e: (value at t0, at t0+1)
+  float gate;                         // one action gate of the chunk: matrix tid/32 % 4, row (tid/2) % 16, step tid % 2
 };
 
 // NMAT matrices in this launch's group, the first of them ungated (Wo) when FIRST.
@@ -36,36 +39,32 @@ struct DwStage {
 // batch tile fastest), 4*NC KiB apart.
 template <int NC, int NMAT, bool FIRST>
 __device__ __forceinline__ void dw_fetch(const RingDwArgs& p, const bf16x8* ga, const f32x4* rb, int bt, int t0, int mg,
-                                         int lane, DwStage<NMAT - (FIRST ? 1 : 0)>& s) {
+                                         int tid, DwStage<NMAT - (FIRST ? 1 : 0)>& s) {
   const int T = p.T, k = p.k;
 #pragma unroll
   for (int u = 0; u < DW_WI; ++u) s.a[u] = ga[u * 64];
   s.bpart[0] = rb[0];
   s.bpart[1] = rb[256];
-  // gates: addresses are clamped into the problem and the values used as loaded.  No masking is
-  // needed (and none may touch the values here, or the fetch would wait for its own loads): batch
-  // rows past B and the missing second step of an odd-length sequence carry zero fragments.
-  const int q = lane >> 4;
-  const int t1 = t0 + 1 < T ? t0 + 1 : t0;
-#pragma unroll
-  for (int a = FIRST ? 1 : 0; a < NMAT; ++a) {
-    const int ch = 3 * mg + a - 1;   // action channel of this matrix
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      const int b = 16 * bt + 4 * q + e;
-      const int bc = b < p.B ? b : p.B - 1;
-      const float* row = p.A + ((size_t)bc * T) * k + ch;
-      s.gate[a - (FIRST ? 1 : 0)][e] = f32x2{row[(size_t)t0 * k], row[(size_t)t1 * k]};
-    }
+  // gate of (gated matrix ga, sample row, step t0 + tt) for thread tid = 32*ga + 2*row + tt (mod 128).
+  // The address is clamped into the tensor and the value used as loaded: rows past B and the missing
+  // second step of an odd-length sequence meet zero g fragments.
+  {
+    const int gi = tid & 127, gm = gi >> 5, row = (gi >> 1) & 15, tt = gi & 1;
+    constexpr int NG = NMAT - (FIRST ? 1 : 0);
+    const int ch = 3 * mg + (gm < NG ? gm : 0) - (FIRST ? 0 : 1);   // matrix 3*mg + a gates with channel 3*mg + a - 1
+    const int b = 16 * bt + row, bc = b < p.B ? b : p.B - 1;
+    const int tg = t0 + tt < T ? t0 + tt : t0;
+    s.gate = p.A[((size_t)bc * T + tg) * k + ch];
   }
 }
 
-__device__ __forceinline__ bf16x8 gate_frag(bf16x8 x, const f32x2 (&g)[4]) {
+// g8 = gates of rows 4q..4q+3 as (t0, t0+1) pairs: K slot e of the fragment is row e at t0, slot 4+e row e at t0+1
+__device__ __forceinline__ bf16x8 gate_frag(bf16x8 x, const f32x4 (&g8)[2]) {
   bf16x8 o;
 #pragma unroll
   for (int e = 0; e < 4; ++e) {
-    o[e] = (__bf16)((float)x[e] * g[e][0]);
-    o[4 + e] = (__bf16)((float)x[4 + e] * g[e][1]);
+    o[e] = (__bf16)((float)x[e] * g8[e >> 1][2 * (e & 1)]);
+    o[4 + e] = (__bf16)((float)x[4 + e] * g8[e >> 1][2 * (e & 1) + 1]);
   }
   return o;
 }
@@ -78,6 +77,7 @@ __global__ __launch_bounds__(256) void ring_dw_direct_kernel(RingDwArgs p, int m
   constexpr int NB = NT / 8;             // 128-neuron blocks per side
   constexpr int NG = NMAT - (FIRST ? 1 : 0);
   __shared__ __attribute__((aligned(16))) f32x4 lds_b[2][DW_WJ * 64];
+  __shared__ __attribute__((aligned(16))) float lds_g[2][4][16][2];   // [buffer][gated matrix][row][step]
   const int tid = threadIdx.x, wv = tid >> 6, lane = tid & 63;
   const int tiles = NB * NB;
   // keep the workgroups that share a K split on one XCD (workgroup ids are dealt round-robin to
@@ -121,7 +121,7 @@ __global__ __launch_bounds__(256) void ring_dw_direct_kernel(RingDwArgs p, int m
   const bf16x8* ga = reinterpret_cast<const bf16x8*>(p.gfrag) + (size_t)ch0 * CHUNK_FRAGS + (size_t)it0 * 64 + lane;
   const f32x4* rb = reinterpret_cast<const f32x4*>(p.rfrag) + (size_t)ch0 * CHUNK_FRAGS + (size_t)jt0 * 64 + tid;
   auto fetch_next = [&](DwStage<NG>& s) {
-    dw_fetch<NC, NMAT, FIRST>(p, ga, rb, fb, 2 * ft, mg, lane, s);
+    dw_fetch<NC, NMAT, FIRST>(p, ga, rb, fb, 2 * ft, mg, tid, s);
     const int adv = (fc + 1 < ch1) ? 1 : 0;
     ga += adv * CHUNK_FRAGS;
     rb += adv * CHUNK_FRAGS;
@@ -135,11 +135,18 @@ __global__ __launch_bounds__(256) void ring_dw_direct_kernel(RingDwArgs p, int m
     bf16x8 b[DW_WJ];
 #pragma unroll
     for (int u = 0; u < DW_WJ; ++u) b[u] = *reinterpret_cast<const bf16x8*>(&lds_b[cur][u * 64 + lane]);
+    f32x4 g8[NG > 0 ? NG : 1][2];
+#pragma unroll
+    for (int a = 0; a < NG; ++a) {
+      const f32x4* gp = reinterpret_cast<const f32x4*>(&lds_g[cur][a][4 * (lane >> 4)][0]);
+      g8[a][0] = gp[0];
+      g8[a][1] = gp[1];
+    }
 #pragma unroll
     for (int a = 0; a < NMAT; ++a) {
 #pragma unroll
       for (int ii = 0; ii < DW_WI; ++ii) {
-        const bf16x8 gg = (FIRST && a == 0) ? s.a[ii] : gate_frag(s.a[ii], s.gate[a - (FIRST ? 1 : 0)]);
+        const bf16x8 gg = (FIRST && a == 0) ? s.a[ii] : gate_frag(s.a[ii], g8[a - (FIRST ? 1 : 0)]);
 #pragma unroll
         for (int u = 0; u < DW_WJ; ++u) acc[a][ii][u] = mfma16(gg, b[u], acc[a][ii][u]);
       }
@@ -148,6 +155,7 @@ __global__ __launch_bounds__(256) void ring_dw_direct_kernel(RingDwArgs p, int m
   auto publish = [&](const DwStage<NG>& s, int buf) {
     lds_b[buf][tid] = s.bpart[0];
     lds_b[buf][tid + 256] = s.bpart[1];
+    if (tid < 128) (&lds_g[buf][0][0][0])[tid] = s.gate;
   };
 
   if (ch0 < ch1) {
