@@ -171,16 +171,6 @@ __global__ __launch_bounds__(256) void ring_dw_direct_kernel(RingDwArgs p, int m
         compute(st[d], d & 1);                      // DW_DEPTH is even: chunk parity == d parity
         fetch_next(st[d]);                          // refill DW_DEPTH chunks ahead
         publish(st[(d + 1) % DW_DEPTH], (d & 1) ^ 1);
-        // issue order for this step: LDS reads first, then every MFMA followed by a few of the
-        // gating / addressing VALU ops and one of the refill loads, so the vector ALU works in the
-        // shadow of the matrix pipe instead of ahead of it
-        __builtin_amdgcn_sched_group_barrier(0x100, DW_WJ, 0);
-#pragma unroll
-        for (int m = 0; m < NMAT * DW_WI * DW_WJ; ++m) {
-          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-          __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);
-          if (m % 4 == 3) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
-        }
         lds_barrier();
         // keep the refill of stage d where it is: the scheduler would otherwise sink all refills of
         // a trip to its end and drain the whole queue once per trip
