@@ -432,8 +432,17 @@ __global__ __launch_bounds__(256) void ring_dw_reduce_kernel(RingDwArgs p, int N
   const size_t per_z = (size_t)(p.k + 1) * NT * NT * 64;
   const size_t u = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (u >= per_z) return;
+  // fixed summation order z = 0, 1, 2, ...; the loads of sixteen slices are issued together
   f32x4 s = {0.f, 0.f, 0.f, 0.f};
-  for (int z = 0; z < p.nz; ++z) s += p.partial[(size_t)z * per_z + u];
+  int z = 0;
+  for (; z + 16 <= p.nz; z += 16) {
+    f32x4 v[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) v[i] = __builtin_nontemporal_load(&p.partial[(size_t)(z + i) * per_z + u]);
+#pragma unroll
+    for (int i = 0; i < 16; ++i) s += v[i];
+  }
+  for (; z < p.nz; ++z) s += p.partial[(size_t)z * per_z + u];
   const int lane = (int)(u & 63);
   size_t v = u >> 6;
   const int jt = (int)(v % NT);
