@@ -51,9 +51,11 @@ RINGATTR_API int ringattr_version(void);
 RINGATTR_API const char* ringattr_last_error(void);
 
 /* Bytes of the "saved activations" buffer the forward pass fills for training:
- * F'(re) as fp16 and the bf16 operand copy of r_prev, both in the kernels'
- * private tile order.  Opaque to the caller: allocate, pass to ringattr_fwd,
- * keep until ringattr_bwd.  Replaces the reference's re_history slot
+ * alpha*F'(re) as fp16 and the bf16 operand copy of r_prev, both in the kernels'
+ * private tile order, and the transposed bf16 weight fragments the backward
+ * multiplies with (so a backward that is handed `saved` differentiates at the
+ * weights its forward saw and needs no packing launch of its own).  Opaque to
+ * the caller: allocate, pass to ringattr_fwd, keep until ringattr_bwd.  Replaces the reference's re_history slot
  * (cpp/ring_rnn_cuda.py:106, cpp/bwd.cu:12). */
 RINGATTR_API size_t ringattr_saved_bytes(int N, int a_dim, int seq_len, int batch_size);
 

@@ -17,34 +17,44 @@
 //   split_k = 1 (NC = 4 only): contraction position kappa stands for neuron split_k_neuron(kappa), the
 //   order the pipelined weight-resident kernels keep their operand tile in.
 // ------------------------------------------------------------------------------------------------
+__device__ __forceinline__ bf16x8 pack_fragment(const float* __restrict__ Wo, const float* __restrict__ Wa, size_t u,
+                                                int N, int NC, int transposed, int split_k, float scale0) {
+  const int KCH = 2 * NC;
+  const int lane = (int)(u & 63);
+  size_t v = u >> 6;
+  const int kc = (int)(v % KCH);
+  v /= KCH;
+  const int c = (int)(v % NC);
+  v /= NC;
+  const int w = (int)(v & 3);
+  const int mm = (int)(v >> 2);
+  const int q = lane >> 4, n = lane & 15;
+  const int col = 16 * NC * w + NC * n + c;
+  const int k0 = 32 * kc + 8 * q;
+  const float* W = (mm == 0) ? Wo : Wa + (size_t)(mm - 1) * N * N;
+  bf16x8 pk;
+#pragma unroll
+  for (int x = 0; x < 8; ++x) {
+    const int kk = split_k ? split_k_neuron(k0 + x) : k0 + x;
+    float val = 0.f;
+    if (col < N && kk < N) val = transposed ? W[(size_t)kk * N + col] : W[(size_t)col * N + kk];
+    pk[x] = (__bf16)(mm == 0 ? val * scale0 : val);
+  }
+  return pk;
+}
+
+// One launch can write two packed copies (the forward's own and the transposed one its backward will
+// need): fragments [0, total) go to out, [total, 2*total) to out2 when out2 is not null.
 __global__ __launch_bounds__(256) void ring_pack_weights_kernel(const float* __restrict__ Wo,
                                                                 const float* __restrict__ Wa,
-                                                                bf16x8* __restrict__ out, int N, int k, int NC,
-                                                                int transposed, int split_k, float scale0) {
-  const int KCH = 2 * NC;
-  const size_t total = (size_t)(1 + k) * 4 * NC * KCH * 64;
-  for (size_t u = (size_t)blockIdx.x * blockDim.x + threadIdx.x; u < total; u += (size_t)gridDim.x * blockDim.x) {
-    const int lane = (int)(u & 63);
-    size_t v = u >> 6;
-    const int kc = (int)(v % KCH);
-    v /= KCH;
-    const int c = (int)(v % NC);
-    v /= NC;
-    const int w = (int)(v & 3);
-    const int mm = (int)(v >> 2);
-    const int q = lane >> 4, n = lane & 15;
-    const int col = 16 * NC * w + NC * n + c;
-    const int k0 = 32 * kc + 8 * q;
-    const float* W = (mm == 0) ? Wo : Wa + (size_t)(mm - 1) * N * N;
-    bf16x8 pk;
-#pragma unroll
-    for (int x = 0; x < 8; ++x) {
-      const int kk = split_k ? split_k_neuron(k0 + x) : k0 + x;
-      float val = 0.f;
-      if (col < N && kk < N) val = transposed ? W[(size_t)kk * N + col] : W[(size_t)col * N + kk];
-      pk[x] = (__bf16)(mm == 0 ? val * scale0 : val);
-    }
-    out[u] = pk;
+                                                                bf16x8* __restrict__ out, bf16x8* __restrict__ out2, int N,
+                                                                int k, int NC, int transposed, int split_k, float scale0,
+                                                                int transposed2, int split_k2, float scale2) {
+  const size_t total = (size_t)(1 + k) * 4 * NC * 2 * NC * 64;
+  const size_t all = out2 ? 2 * total : total;
+  for (size_t u = (size_t)blockIdx.x * blockDim.x + threadIdx.x; u < all; u += (size_t)gridDim.x * blockDim.x) {
+    if (u < total) out[u] = pack_fragment(Wo, Wa, u, N, NC, transposed, split_k, scale0);
+    else out2[u - total] = pack_fragment(Wo, Wa, u - total, N, NC, transposed2, split_k2, scale2);
   }
 }
 
@@ -532,15 +542,21 @@ hipError_t ring_profile_collect(double* ms, long long* launches) {
     default: return hipErrorInvalidValue;           \
   }
 
-hipError_t ring_launch_pack(const float* Wo, const float* Wa, void* out, int N, int k, int NC, int transposed,
-                            int split_k, float scale0, hipStream_t st) {
-  if (split_k && NC != 4) return hipErrorInvalidValue;
-  const size_t total = (size_t)(1 + k) * 4 * NC * 2 * NC * 64;
+hipError_t ring_launch_pack2(const float* Wo, const float* Wa, int N, int k, int NC, void* out, int transposed,
+                             int split_k, float scale0, void* out2, int transposed2, int split_k2, float scale2,
+                             hipStream_t st) {
+  if ((split_k || (out2 && split_k2)) && NC != 4) return hipErrorInvalidValue;
+  const size_t total = (size_t)(1 + k) * 4 * NC * 2 * NC * 64 * (out2 ? 2 : 1);
   const int blocks = (int)((total + 255) / 256 < 4096 ? (total + 255) / 256 : 4096);
   ProfScope prof(0, st);
-  hipLaunchKernelGGL(ring_pack_weights_kernel, dim3(blocks), dim3(256), 0, st, Wo, Wa, (bf16x8*)out, N, k, NC,
-                     transposed, split_k, scale0);
+  hipLaunchKernelGGL(ring_pack_weights_kernel, dim3(blocks), dim3(256), 0, st, Wo, Wa, (bf16x8*)out, (bf16x8*)out2, N, k,
+                     NC, transposed, split_k, scale0, transposed2, split_k2, scale2);
   return hipGetLastError();
+}
+
+hipError_t ring_launch_pack(const float* Wo, const float* Wa, void* out, int N, int k, int NC, int transposed,
+                            int split_k, float scale0, hipStream_t st) {
+  return ring_launch_pack2(Wo, Wa, N, k, NC, out, transposed, split_k, scale0, nullptr, 0, 0, 1.f, st);
 }
 
 // RINGATTR_STREAMING=1 forces the generic weight-streaming kernels (used by tests to cross-check).

@@ -90,7 +90,7 @@ const char* ringattr_last_error(void) { return g_err; }
 size_t ringattr_saved_bytes(int N, int a_dim, int seq_len, int batch_size) {
   Geo g;
   if (make_geo(N, a_dim, seq_len, batch_size, g) != RINGATTR_OK) return 0;
-  return g.side_bytes + g.pair_bytes;
+  return g.side_bytes + g.pair_bytes + g.wpack_bytes;
 }
 
 size_t ringattr_fwd_workspace_bytes(int N, int a_dim, int seq_len, int batch_size) {
@@ -123,7 +123,12 @@ int ringattr_fwd(const void* A, const void* Wa, float J0, float J1, const void* 
                 workspace ? workspace_bytes : (size_t)0);
   hipStream_t st = static_cast<hipStream_t>(stream);
 
-  hipError_t e = ring_launch_pack((const float*)Wo, (const float*)Wa, workspace, N, a_dim, g.NC, 0, ring_uses_resident(N, a_dim) ? 1 : 0, 1.f, st);
+  // With a saved buffer the same launch also writes the transposed copy the backward will need (J1
+  // folded into Wo for the weight-resident BPTT kernel) behind the saved activations.
+  const int resident = ring_uses_resident(N, a_dim) ? 1 : 0;
+  void* wpack_t = saved ? (char*)saved + g.side_bytes + g.pair_bytes : nullptr;
+  hipError_t e = ring_launch_pack2((const float*)Wo, (const float*)Wa, N, a_dim, g.NC, workspace, 0, resident, 1.f,
+                                   wpack_t, 1, 0, resident ? J1 : 1.f, st);
   if (e != hipSuccess) return hip_fail(e, "pack weights");
 
   RingFwdArgs a;
@@ -213,9 +218,16 @@ int ringattr_bwd(const void* grad_output, const void* A, const void* Wa, float J
   }
 
   // the weight-resident BPTT kernel takes J1 folded into the transposed Wo fragments
-  const bool bptt_resident = ring_uses_resident(N, a_dim) && !grad_A;
-  hipError_t e = ring_launch_pack((const float*)Wo, (const float*)Wa, wb, N, a_dim, g.NC, 1, 0, bptt_resident ? J1 : 1.f, st);
-  if (e != hipSuccess) return hip_fail(e, "pack transposed weights");
+  const bool resident = ring_uses_resident(N, a_dim);
+  const bool bptt_resident = resident && !grad_A;
+  hipError_t e = hipSuccess;
+  if (saved && bptt_resident == resident) {
+    // the forward left the transposed copy (with the scale this BPTT kernel expects) behind the saved activations
+    wb = (char*)const_cast<void*>(saved) + g.side_bytes + g.pair_bytes;
+  } else {
+    e = ring_launch_pack((const float*)Wo, (const float*)Wa, wb, N, a_dim, g.NC, 1, 0, bptt_resident ? J1 : 1.f, st);
+    if (e != hipSuccess) return hip_fail(e, "pack transposed weights");
+  }
 
   RingBpttArgs b;
   b.A = (const float*)A;

@@ -33,13 +33,14 @@ def test_size_queries():
     lib = _lib.load()
     N, k, T, B = 256, 2, 120, 4096
     saved = lib.ringattr_saved_bytes(N, k, T, B)
-    assert saved == 2 * T * B * N * 2                                  # fp16 F' + bf16 r_prev, both [T,B,N]
+    wpack = 3 * N * N * 2                                              # one bf16 copy of [Wo|Wa0|Wa1]
+    assert saved == 2 * T * B * N * 2 + wpack                          # fp16 F' + bf16 r_prev [T,B,N] + transposed weights
     assert lib.ringattr_fwd_workspace_bytes(N, k, T, B) == 3 * N * N * 2
     with_saved = lib.ringattr_bwd_workspace_bytes(N, k, T, B, 1)
     without = lib.ringattr_bwd_workspace_bytes(N, k, T, B, 0)
-    assert without - with_saved == saved + 3 * N * N * 2               # rebuilt buffer + forward weight pack
+    assert without - with_saved == saved                               # rebuilt F' and r_prev copy + forward weight pack
     # padding: N=120 -> 128 neurons, B=64 -> 4 batch tiles; odd T rounds the paired buffer up
-    assert lib.ringattr_saved_bytes(120, 2, 7, 64) == (7 + 8) * 64 * 128 * 2
+    assert lib.ringattr_saved_bytes(120, 2, 7, 64) == (7 + 8) * 64 * 128 * 2 + 3 * 128 * 128 * 2
     assert lib.ringattr_saved_bytes(0, 2, 7, 64) == 0 and "positive" in _lib.last_error()
     assert lib.ringattr_saved_bytes(513, 2, 7, 64) == 0 and "512" in _lib.last_error()
 
