@@ -34,8 +34,12 @@ MEASURED_TRAFFIC_BYTES = {
 }
 
 WORKLOADS = {
-    # BASELINE config 2 (headline)
-    "train_n256_b4096_t120_gelu": dict(N=256, B=4096, T=120, k=2, act="gelu", J0=-1.0 / 256, J1=1.0),
+    # BASELINE config 2 (headline; the default and the only workload the metric is quoted on)
+    "train_n256_b4096_t120_gelu": dict(N=256, B=4096, T=120, k=2, act="gelu", J0=-1.0 / 256, J1=1.0, mode="train"),
+    # the other BASELINE shapes, for reference figures (run with --workload; pick --steps to taste)
+    "train_n120_b64_t120_tanh": dict(N=120, B=64, T=120, k=2, act="tanh", J0=-1.0 / 120, J1=1.0, mode="train"),
+    "infer_n256_b1024_t120_relu": dict(N=256, B=1024, T=120, k=2, act="relu", J0=-1.0 / 256, J1=1.0, mode="infer"),
+    "train_n512_b8192_t512_tanh": dict(N=512, B=8192, T=512, k=2, act="tanh", J0=-1.0 / 512, J1=1.0, mode="train"),
 }
 
 
@@ -127,12 +131,18 @@ def main():
     def fwd():
         return ring_rnn_cuda_func(x["A"], Wa, cfg["J0"], cfg["J1"], Wo, x["r0"], 0.15, cfg["act"])
 
-    G = loss_head_grad(fwd(), x["angle"])
+    train = cfg["mode"] == "train"
+    if train:
+        G = loss_head_grad(fwd(), x["angle"])
 
-    def step():
-        Wa.grad = None
-        Wo.grad = None
-        fwd().backward(G)
+        def step():
+            Wa.grad = None
+            Wo.grad = None
+            fwd().backward(G)
+    else:
+        def step():
+            with torch.no_grad():
+                fwd()
 
     for _ in range(args.warmup):
         step()
@@ -157,19 +167,22 @@ def main():
     value = B * T / (dt / args.steps)
     flops_third = 6.0 * N * N * B * T                      # per kernel: fwd, bptt and dW each contract 2*3*N^2 per sample-step
     kern = {kname: (ms / max(cnt, 1)) for kname, (ms, cnt) in prof.items() if cnt}
-    dominant = max(("fwd", "bptt", "dw"), key=lambda n_: kern.get(n_, 0.0))
+    dominant = max(("fwd", "bptt", "dw") if train else ("fwd",), key=lambda n_: kern.get(n_, 0.0))
     dom_ms = kern[dominant]
     achieved = flops_third / (dom_ms * 1e-3) / 1e12
     bytes_per_ss = 12 * N + 8 * k                           # fp32 history write + r_prev/grad_output reads + A
     out = {
-        "metric": "fwd+bwd sample-steps/s (B*T/s) at N=256,B=4096,T=120; % bf16 MFMA peak",
+        "metric": ("fwd+bwd sample-steps/s (B*T/s) at N=256,B=4096,T=120; % bf16 MFMA peak"
+                   if args.workload == "train_n256_b4096_t120_gelu" else
+                   f"{'fwd+bwd' if train else 'fwd'} sample-steps/s (B*T/s) at N={N},B={B},T={T}"),
         "value": value, "unit": "sample-steps/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
         "config": {"workload": args.workload, "N": N, "B": B, "T": T, "a_dim": k, "activation": cfg["act"],
-                   "grad_output": "gradient of the cos-sim + 0.2*bump-amplitude loss pair, precomputed"},
-        "pct_bf16_mfma_peak_fwd_bwd": 100.0 * (18.0 * N * N * value) / (PEAK_BF16_TFLOPS * 1e12),
-        "algorithmic_hbm_gbs_fwd_bwd": bytes_per_ss * value / 1e9,
+                   "mode": "forward + backward" if train else "forward only (no saved activations)",
+                   "grad_output": "gradient of the cos-sim + 0.2*bump-amplitude loss pair, precomputed" if train else None},
+        "pct_bf16_mfma_peak": 100.0 * ((18.0 if train else 6.0) * N * N * value) / (PEAK_BF16_TFLOPS * 1e12),
+        "algorithmic_hbm_gbs": (bytes_per_ss if train else 4 * N + 4 * k) * value / 1e9,
         "roofline": {"bound": "mfma", "kernel": dominant, "achieved": achieved, "peak": PEAK_BF16_TFLOPS,
                      "unit": "TFLOP/s", "frac": achieved / PEAK_BF16_TFLOPS,
                      "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload, {}).get(dominant),
@@ -179,7 +192,7 @@ def main():
         "kernel_ms": kern,
     }
     if not args.no_cpu:
-        out["cpu_baseline"] = cpu_baseline(cfg, args.cpu_sample_batch)
+        out["cpu_baseline"] = cpu_baseline(cfg, min(args.cpu_sample_batch, B))
     print(json.dumps(out))
 
 
