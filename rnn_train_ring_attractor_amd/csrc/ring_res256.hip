@@ -374,9 +374,8 @@ struct BpttStage {
 // In the unmasked variant the six loads of a stage are issued with inline assembly and waited for
 // with an explicit vmcnt.  The compiler, seeing loads and stores share that counter, would otherwise
 // drain it completely (vmcnt(0)) before every use and expose a full HBM round trip per time step.
-// Safety of bptt_stage_wait<K>: loads return in issue order, so once at most K vector-memory
-// operations are outstanding and K later loads were issued after this stage, the stage has landed;
-// later stores can only make the wait longer.  The "+v" operands order every use after the wait.
+// Safety of bptt_stage_wait<K>: vector-memory operations leave the counter in issue order, so once at
+// most K are outstanding and at least K were issued after this stage's loads, the stage has landed.  The "+v" operands order every use after the wait.
 __device__ __forceinline__ f32x4 async_load16(const void* ptr) {
   f32x4 v;
   // (the local labels cost nothing at run time; the build check uses them to find these loads and
@@ -474,8 +473,10 @@ __global__ __launch_bounds__(256) void ring_bptt_res256_kernel(RingBpttArgs p) {
       const int cur = u & 1, ci = u / R_GCH, l = u % R_GCH;
       if (l == 0 && (ci + 1) * R_GCH < T) gates_fetch(p.A, T, B, bt, ci + 1, -1, tid, gs);
       BpttStage& S = st[half];
-      // the other stage's six loads are the only loads issued after this stage's
-      if constexpr (FULL) bptt_stage_wait<6>(S);
+      // issued after this stage's six loads: the previous step's four operand-copy stores and the other
+      // stage's six loads.  The counter is in order, so "at most ten outstanding" means this stage landed;
+      // a smaller number would also wait for those stores to be acknowledged by memory.
+      if constexpr (FULL) bptt_stage_wait<10>(S);
 
       float G[4][R_NC], g[4][R_NC];
 #pragma unroll

@@ -1,7 +1,8 @@
 """Build-time checks on the compiled gfx950 ISA (hipcc cross-compiles here, no GPU needed).
 
 The BPTT kernel issues its per-step global loads with inline assembly and waits for them with an
-explicit s_waitcnt.  The compiler does not know those destination registers are still being filled,
+explicit s_waitcnt vmcnt(N), where N counts the vector-memory instructions (loads and stores alike:
+one in-order counter on this target) issued after the loads being waited for.  The compiler does not know those destination registers are still being filled,
 so this test proves on the emitted code that nothing reads or writes them between the load and the
 wait that covers it, and that the hot loops use no scratch memory."""
 import os
@@ -74,6 +75,11 @@ def test_async_loads_are_not_touched_before_their_wait(res256_asm):
             continue
         if t.startswith("s_waitcnt") and "vmcnt(0)" in t:
             fifo = []
+            continue
+        # every other vector-memory instruction occupies a slot of the same in-order counter: stores define no
+        # register, compiler-issued loads are waited for by the compiler itself
+        if t.startswith(("global_store", "global_load", "buffer_store", "buffer_load", "scratch_")):
+            fifo.append(set())
             continue
         pending = set().union(*fifo) if fifo else set()
         ops = t.split(None, 1)
