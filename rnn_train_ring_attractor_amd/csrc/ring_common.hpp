@@ -57,33 +57,39 @@ __device__ __forceinline__ void lds_barrier() {
   asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 }
 
-// F(x) and F'(x).  gelu is the exact erf form (train/train_ring_attractor.py:16), its derivative
+// F(x) and F'(x).  gelu is the exact erf form (train/train_ring_attractor.py:16) and its derivative
 // uses the normal density 1/sqrt(2*pi) as the torch path does (legacy/bwd_fp32.py:455-457).
-__device__ __forceinline__ void act_eval(int act, float x, float& F, float& D) {
-  switch (act) {
-    case ACT_RELU:
-      F = fmaxf(x, 0.f);
-      D = x > 0.f ? 1.f : 0.f;
-      break;
-    case ACT_GELU: {
-      float cdf = 0.5f * erfcf(-x * 0.70710678118654752f);
-      float pdf = 0.39894228040143268f * __expf(-0.5f * x * x);
-      F = x * cdf;
-      D = cdf + x * pdf;
-      break;
-    }
-    case ACT_TANH: {
-      float th = tanhf(x);
-      F = th;
-      D = 1.f - th * th;
-      break;
-    }
-    default: {  // ACT_SILU
-      float s = 1.f / (1.f + __expf(-x));
-      F = x * s;
-      D = s * (1.f + x * (1.f - s));
-      break;
-    }
+// Branch-free activation pairs (F, F') for the per-step critical path of every recurrence kernel.
+//  gelu: Phi via the Abramowitz-Stegun 7.1.26 erfc polynomial (|err| < 1.5e-7), sharing exp(-x^2/2)
+//  with the density term of F'.   tanh/silu: one v_exp + one v_rcp.
+template <int ACT>
+__device__ __forceinline__ void act_fast(float x, float& F, float& D) {
+  if constexpr (ACT == ACT_RELU) {
+    F = fmaxf(x, 0.f);
+    D = x > 0.f ? 1.f : 0.f;
+  } else if constexpr (ACT == ACT_GELU) {
+    const float ax = fabsf(x);
+    const float t = __builtin_amdgcn_rcpf(fmaf(ax, 0.3275911f * 0.70710678f, 1.f));
+    const float e = __builtin_amdgcn_exp2f(x * x * -0.72134752f);   // exp(-x^2/2)
+    float poly = fmaf(t, 0.5f * 1.061405429f, 0.5f * -1.453152027f);
+    poly = fmaf(t, poly, 0.5f * 1.421413741f);
+    poly = fmaf(t, poly, 0.5f * -0.284496736f);
+    poly = fmaf(t, poly, 0.5f * 0.254829592f);
+    const float h = poly * t * e;                 // 0.5*erfc(|x|/sqrt2) = Phi(-|x|)
+    const float cdf = x >= 0.f ? 1.f - h : h;
+    F = x * cdf;
+    D = fmaf(x * e, 0.39894228f, cdf);
+  } else if constexpr (ACT == ACT_TANH) {
+    const float xc = fminf(fmaxf(x, -15.f), 15.f);
+    const float e2 = __builtin_amdgcn_exp2f(xc * 2.88539008f);      // exp(2x)
+    const float th = 1.f - 2.f * __builtin_amdgcn_rcpf(e2 + 1.f);
+    F = th;
+    D = 1.f - th * th;
+  } else {
+    const float xc = fmaxf(x, -87.f);
+    const float s = __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(xc * -1.44269504f));
+    F = x * s;
+    D = s * fmaf(x, 1.f - s, 1.f);
   }
 }
 

@@ -71,9 +71,29 @@ __device__ __forceinline__ void gated_products(const bf16x8* __restrict__ xb, co
                                                float J1, int w, int lane, f32x4 (&acc)[NC],
                                                const float (*rp)[NC] = nullptr, float* ga_part = nullptr) {
   using TL = Tile<NC>;
+  constexpr int KG = TL::KG, NKG = TL::NKG;
+  constexpr int UPM = NKG * NC;                 // weight units (one column tile x KG chunks) per matrix
+  constexpr int PD = UPM >= 4 ? 4 : UPM;        // register buffers: PD - 1 units are in flight ahead of the MFMAs
   const int q = lane >> 4, n = lane & 15;
 #pragma unroll
   for (int c = 0; c < NC; ++c) acc[c] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  // The weights of a step stream from L2 as one linear sequence of units, matrix after matrix; what
+  // bounds the step is how many bytes are in flight, so the prefetch runs PD - 1 units ahead and
+  // straight across matrix boundaries (past the last matrix it re-reads the last unit, unused).
+  const int units = (k + 1) * UPM;
+  auto unit_ptr = [&](int u) {
+    u = u < units ? u : units - 1;
+    const int mm = u / UPM, rem = u % UPM, kg = rem / NC, c = rem % NC;
+    return Wp + ((size_t)((mm * 4 + w) * NC + c) * TL::KCH + kg * KG) * 64 + lane;
+  };
+  bf16x8 wf[PD][KG];
+#pragma unroll
+  for (int d = 0; d < PD - 1; ++d) {
+    const bf16x8* src = unit_ptr(d);
+#pragma unroll
+    for (int u = 0; u < KG; ++u) wf[d][u] = src[(size_t)u * 64];
+  }
 
   for (int mm = 0; mm <= k; ++mm) {
     float coef[4];
@@ -85,24 +105,23 @@ __device__ __forceinline__ void gated_products(const bf16x8* __restrict__ xb, co
     f32x4 p[NC];
 #pragma unroll
     for (int c = 0; c < NC; ++c) p[c] = f32x4{0.f, 0.f, 0.f, 0.f};
-    const bf16x8* wm = Wp + ((size_t)(mm * 4 + w) * NC) * TL::KCH * 64 + lane;
 #pragma unroll
-    for (int kg = 0; kg < TL::NKG; ++kg) {
-      bf16x8 af[TL::KG];
+    for (int kg = 0; kg < NKG; ++kg) {
+      bf16x8 af[KG];
 #pragma unroll
-      for (int u = 0; u < TL::KG; ++u) af[u] = xb[((kg * TL::KG + u) * 4 + q) * XG + n];
-      bf16x8 wf[2][TL::KG];
-#pragma unroll
-      for (int u = 0; u < TL::KG; ++u) wf[0][u] = wm[(size_t)(0 * TL::KCH + kg * TL::KG + u) * 64];
+      for (int u = 0; u < KG; ++u) af[u] = xb[((kg * KG + u) * 4 + q) * XG + n];
 #pragma unroll
       for (int c = 0; c < NC; ++c) {
-        if (c + 1 < NC) {
+        constexpr int dummy = 0;
+        (void)dummy;
+        const int ul = kg * NC + c;             // unit within the matrix; UPM % PD == 0 keeps buffer indices static
+        {
+          const bf16x8* src = unit_ptr(mm * UPM + ul + PD - 1);
 #pragma unroll
-          for (int u = 0; u < TL::KG; ++u)
-            wf[(c + 1) & 1][u] = wm[(size_t)((c + 1) * TL::KCH + kg * TL::KG + u) * 64];
+          for (int u = 0; u < KG; ++u) wf[(ul + PD - 1) % PD][u] = src[(size_t)u * 64];
         }
 #pragma unroll
-        for (int u = 0; u < TL::KG; ++u) p[c] = mfma16(af[u], wf[c & 1][u], p[c]);
+        for (int u = 0; u < KG; ++u) p[c] = mfma16(af[u], wf[ul % PD][u], p[c]);
       }
     }
 #pragma unroll
@@ -153,7 +172,7 @@ __device__ __forceinline__ void read_rowsum(const float* psum, int q, float (&s)
 // per step).  Writes bump_history [T,B,N] fp32 and, when training, F'(re) (fp16) and the bf16
 // operand copy of r_prev in tile order.
 // ------------------------------------------------------------------------------------------------
-template <int NC>
+template <int NC, int ACT>
 __global__ __launch_bounds__(256) void ring_fwd_kernel(RingFwdArgs p) {
   using TL = Tile<NC>;
   __shared__ bf16x8 xbuf[2][TL::SLOTS];
@@ -189,7 +208,7 @@ __global__ __launch_bounds__(256) void ring_fwd_kernel(RingFwdArgs p) {
       for (int c = 0; c < NC; ++c) {
         const float x = acc[c][e] + p.J0 * s[e];
         float F, D;
-        act_eval(p.act, x, F, D);
+        act_fast<ACT>(x, F, D);
         const bool ok = (b0 + e < B) && (i0 + c < N);
         r[e][c] = ok ? (oma * r[e][c] + p.alpha * F) : 0.f;
         d[e][c] = ok ? p.alpha * D : 0.f;   // the saved record is alpha * F'(re)
@@ -210,7 +229,7 @@ __global__ __launch_bounds__(256) void ring_fwd_kernel(RingFwdArgs p) {
 // Rebuild of the saved activations from the state history (used when the forward's buffer was not
 // kept): one workgroup per (batch tile, step); no recurrence.
 // ------------------------------------------------------------------------------------------------
-template <int NC>
+template <int NC, int ACT>
 __global__ __launch_bounds__(256) void ring_rebuild_saved_kernel(RingFwdArgs p) {
   using TL = Tile<NC>;
   __shared__ bf16x8 xbuf[TL::SLOTS];
@@ -241,7 +260,7 @@ __global__ __launch_bounds__(256) void ring_rebuild_saved_kernel(RingFwdArgs p) 
 #pragma unroll
     for (int c = 0; c < NC; ++c) {
       float F, D;
-      act_eval(p.act, acc[c][e] + p.J0 * s[e], F, D);
+      act_fast<ACT>(acc[c][e] + p.J0 * s[e], F, D);
       d[e][c] = ((b0 + e < B) && (i0 + c < N)) ? p.alpha * D : 0.f;
     }
   }
@@ -533,6 +552,15 @@ hipError_t ring_profile_collect(double* ms, long long* launches) {
 // ------------------------------------------------------------------------------------------------
 // Launchers (host).  NC is chosen by the caller as the smallest of {1,2,4,8} with 64*NC >= N.
 // ------------------------------------------------------------------------------------------------
+#define RING_DISPATCH_ACT(ACTv, CALL)                          \
+  switch (ACTv) {                                              \
+    case ACT_RELU: { constexpr int ACT = ACT_RELU; CALL; } break; \
+    case ACT_GELU: { constexpr int ACT = ACT_GELU; CALL; } break; \
+    case ACT_TANH: { constexpr int ACT = ACT_TANH; CALL; } break; \
+    case ACT_SILU: { constexpr int ACT = ACT_SILU; CALL; } break; \
+    default: return hipErrorInvalidValue;                      \
+  }
+
 #define RING_DISPATCH_NC(NCv, CALL)                 \
   switch (NCv) {                                    \
     case 1: { constexpr int NC = 1; CALL; } break;  \
@@ -569,13 +597,13 @@ bool ring_uses_resident(int N, int k) {
 hipError_t ring_launch_fwd(const RingFwdArgs& a, int NCv, hipStream_t st) {
   ProfScope prof(1, st);
   if (ring_uses_resident(a.N, a.k)) return ring_launch_fwd_res256(a, st);
-  RING_DISPATCH_NC(NCv, hipLaunchKernelGGL(ring_fwd_kernel<NC>, dim3(a.nbt), dim3(256), 0, st, a));
+  RING_DISPATCH_NC(NCv, RING_DISPATCH_ACT(a.act, hipLaunchKernelGGL((ring_fwd_kernel<NC, ACT>), dim3(a.nbt), dim3(256), 0, st, a)));
   return hipGetLastError();
 }
 
 hipError_t ring_launch_rebuild(const RingFwdArgs& a, int NCv, hipStream_t st) {
   ProfScope prof(2, st);
-  RING_DISPATCH_NC(NCv, hipLaunchKernelGGL(ring_rebuild_saved_kernel<NC>, dim3(a.nbt, a.T), dim3(256), 0, st, a));
+  RING_DISPATCH_NC(NCv, RING_DISPATCH_ACT(a.act, hipLaunchKernelGGL((ring_rebuild_saved_kernel<NC, ACT>), dim3(a.nbt, a.T), dim3(256), 0, st, a)));
   return hipGetLastError();
 }
 

@@ -19,40 +19,6 @@ constexpr int R_XSLOTS = R_KCH * 4 * XG;
 constexpr int R_GCH = 32;                             // time steps of action gates staged per LDS chunk
 constexpr size_t R_LDS_BYTES = (size_t)(R_WLDS_SLOTS + 2 * R_XSLOTS) * 16 + 2 * R_GCH * 16 * 8;   // BPTT layout
 
-// Cheap activation pairs (F, F') for the per-step critical path.
-//  gelu: Phi via the Abramowitz-Stegun 7.1.26 erfc polynomial (|err| < 1.5e-7), sharing exp(-x^2/2)
-//  with the density term of F'.   tanh/silu: one v_exp + one v_rcp.
-template <int ACT>
-__device__ __forceinline__ void act_fast(float x, float& F, float& D) {
-  if constexpr (ACT == ACT_RELU) {
-    F = fmaxf(x, 0.f);
-    D = x > 0.f ? 1.f : 0.f;
-  } else if constexpr (ACT == ACT_GELU) {
-    const float ax = fabsf(x);
-    const float t = __builtin_amdgcn_rcpf(fmaf(ax, 0.3275911f * 0.70710678f, 1.f));
-    const float e = __builtin_amdgcn_exp2f(x * x * -0.72134752f);   // exp(-x^2/2)
-    float poly = fmaf(t, 0.5f * 1.061405429f, 0.5f * -1.453152027f);
-    poly = fmaf(t, poly, 0.5f * 1.421413741f);
-    poly = fmaf(t, poly, 0.5f * -0.284496736f);
-    poly = fmaf(t, poly, 0.5f * 0.254829592f);
-    const float h = poly * t * e;                 // 0.5*erfc(|x|/sqrt2) = Phi(-|x|)
-    const float cdf = x >= 0.f ? 1.f - h : h;
-    F = x * cdf;
-    D = fmaf(x * e, 0.39894228f, cdf);
-  } else if constexpr (ACT == ACT_TANH) {
-    const float xc = fminf(fmaxf(x, -15.f), 15.f);
-    const float e2 = __builtin_amdgcn_exp2f(xc * 2.88539008f);      // exp(2x)
-    const float th = 1.f - 2.f * __builtin_amdgcn_rcpf(e2 + 1.f);
-    F = th;
-    D = 1.f - th * th;
-  } else {
-    const float xc = fmaxf(x, -87.f);
-    const float s = __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(xc * -1.44269504f));
-    F = x * s;
-    D = s * fmaf(x, 1.f - s, 1.f);
-  }
-}
-
 // Action gates (A[b,t,0], A[b,t,1]) reach the lanes through LDS in chunks of R_GCH steps, so the
 // time loop issues no vector-memory load whose wait would also drain the history stores.
 // Chunk ci holds loop iterations u = ci*R_GCH + l; iteration u is time step u (dir > 0, forward)
