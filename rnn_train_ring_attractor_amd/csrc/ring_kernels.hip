@@ -63,13 +63,46 @@ __global__ __launch_bounds__(256) void ring_pack_weights_kernel(const float* __r
 // X is read as MFMA A-operand fragments from the LDS operand buffer, W_mm streams from the packed
 // global copy (L2 resident).  coef_0 = J1, coef_{1+j}[e] = A[b_e, t, j].
 // ------------------------------------------------------------------------------------------------
+// Action gates of one step for the workgroup's 16 rows, staged through LDS one step ahead (a_dim <= GATE_KMAX):
+// a coalesced tile load instead of scattered per-lane loads, and the place where all-zero channels are
+// found.  A channel whose gate is zero for all 16 rows at this step contributes nothing to the
+// pre-activation (forward) or to the carried gradient (BPTT), so its matrix is neither fetched nor
+// multiplied: zero-padded action signals (16 channels of which two are driven) cost what two cost.
+constexpr int GATE_KMAX = 64;
+
+__device__ __forceinline__ void gates_stage(float* gl, const float* __restrict__ A, int k, int T, int B, int t, int bt,
+                                            int tid) {
+  for (int idx = tid; idx < 16 * k; idx += 256) {
+    const int row = idx / k, c = idx - row * k, b = 16 * bt + row;
+    gl[row * GATE_KMAX + c] = b < B ? A[((size_t)b * T + t) * k + c] : 0.f;
+  }
+}
+
+// bit c set <=> channel c has a non-zero gate in some row; every wave computes the same mask
+__device__ __forceinline__ unsigned long long gates_active(const float* gl, int k, int lane) {
+  unsigned long long m = 0;
+  for (int c0 = 0; c0 < k; c0 += 4) {
+    const int c = c0 + (lane >> 4);
+    const float v = c < k ? gl[(lane & 15) * GATE_KMAX + c] : 0.f;
+    const unsigned long long bal = __ballot(v != 0.f);
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      if ((bal >> (16 * j)) & 0xffffull) m |= 1ull << (c0 + j);
+  }
+  // the mask is the same in every lane; say so, so that the matrix loop it drives is scalar control flow
+  const unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)m), hi = __builtin_amdgcn_readfirstlane((unsigned)(m >> 32));
+  return ((unsigned long long)hi << 32) | lo;
+}
+
 // With GA, rp holds r_prev[row 4q+e][neuron tile c] and ga_part (k x 4 waves x 16 rows) receives, per action
 // matrix and batch row, this wave's share of  sum_j (X @ W_mm)[row][j] * r_prev[row][j]  (= dL/dA[b,t,mm-1]).
+// gl: this step's staged gates (null: read A from global); active: channels worth multiplying.
 template <int NC, bool GA = false>
 __device__ __forceinline__ void gated_products(const bf16x8* __restrict__ xb, const bf16x8* __restrict__ Wp,
-                                               const float* __restrict__ A, int k, int T, int B, int t, int b0,
-                                               float J1, int w, int lane, f32x4 (&acc)[NC],
-                                               const float (*rp)[NC] = nullptr, float* ga_part = nullptr) {
+                                               const float* __restrict__ A, const float* gl, unsigned long long active,
+                                               int k, int T, int B, int t, int b0, float J1, int w, int lane,
+                                               f32x4 (&acc)[NC], const float (*rp)[NC] = nullptr,
+                                               float* ga_part = nullptr) {
   using TL = Tile<NC>;
   constexpr int KG = TL::KG, NKG = TL::NKG;
   constexpr int UPM = NKG * NC;                 // weight units (one column tile x KG chunks) per matrix
@@ -78,29 +111,37 @@ __device__ __forceinline__ void gated_products(const bf16x8* __restrict__ xb, co
 #pragma unroll
   for (int c = 0; c < NC; ++c) acc[c] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  // The weights of a step stream from L2 as one linear sequence of units, matrix after matrix; what
-  // bounds the step is how many bytes are in flight, so the prefetch runs PD - 1 units ahead and
-  // straight across matrix boundaries (past the last matrix it re-reads the last unit, unused).
-  const int units = (k + 1) * UPM;
-  auto unit_ptr = [&](int u) {
-    u = u < units ? u : units - 1;
-    const int mm = u / UPM, rem = u % UPM, kg = rem / NC, c = rem % NC;
+  // The weights of a step stream from L2 as one linear sequence of units, active matrix after active
+  // matrix; what bounds the step is how many bytes are in flight, so the prefetch runs PD - 1 units
+  // ahead and straight across matrix boundaries (past the last matrix it re-reads that one, unused).
+  // Matrix 0 (Wo) is always active; matrix mm >= 1 is gated by channel mm - 1.
+  const bool skipping = gl != nullptr && !GA;   // dL/dA needs every product, also where the gate is zero
+  auto next_matrix = [&](int mm) {               // next active matrix after mm, or -1
+    if (!skipping) return mm < k ? mm + 1 : -1;
+    const unsigned long long rest = mm >= 64 ? 0ull : (active >> mm);   // channels mm, mm+1, ... <-> matrices mm+1, ...
+    return rest ? mm + 1 + (int)__builtin_ctzll(rest) : -1;
+  };
+  auto unit_ptr = [&](int mm, int ul) {
+    const int kg = ul / NC, c = ul % NC;
     return Wp + ((size_t)((mm * 4 + w) * NC + c) * TL::KCH + kg * KG) * 64 + lane;
   };
   bf16x8 wf[PD][KG];
 #pragma unroll
-  for (int d = 0; d < PD - 1; ++d) {
-    const bf16x8* src = unit_ptr(d);
+  for (int d = 0; d < PD - 1; ++d) {            // PD - 1 < UPM: the first units all belong to matrix 0
+    const bf16x8* src = unit_ptr(0, d);
 #pragma unroll
     for (int u = 0; u < KG; ++u) wf[d][u] = src[(size_t)u * 64];
   }
 
-  for (int mm = 0; mm <= k; ++mm) {
+  for (int mm = 0; mm >= 0;) {
+    const int nxt = next_matrix(mm);
+    const int pre = nxt >= 0 ? nxt : mm;        // matrix the prefetch runs into
     float coef[4];
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-      const int b = b0 + e;
-      coef[e] = (mm == 0) ? J1 : ((b < B) ? A[((size_t)b * T + t) * k + (mm - 1)] : 0.f);
+      if (mm == 0) coef[e] = J1;
+      else if (gl) coef[e] = gl[(4 * q + e) * GATE_KMAX + (mm - 1)];
+      else coef[e] = (b0 + e < B) ? A[((size_t)(b0 + e) * T + t) * k + (mm - 1)] : 0.f;
     }
     f32x4 p[NC];
 #pragma unroll
@@ -112,13 +153,12 @@ __device__ __forceinline__ void gated_products(const bf16x8* __restrict__ xb, co
       for (int u = 0; u < KG; ++u) af[u] = xb[((kg * KG + u) * 4 + q) * XG + n];
 #pragma unroll
       for (int c = 0; c < NC; ++c) {
-        constexpr int dummy = 0;
-        (void)dummy;
         const int ul = kg * NC + c;             // unit within the matrix; UPM % PD == 0 keeps buffer indices static
         {
-          const bf16x8* src = unit_ptr(mm * UPM + ul + PD - 1);
+          const int ahead = ul + PD - 1;
+          const bf16x8* src = ahead < UPM ? unit_ptr(mm, ahead) : unit_ptr(pre, ahead - UPM);
 #pragma unroll
-          for (int u = 0; u < KG; ++u) wf[(ul + PD - 1) % PD][u] = src[(size_t)u * 64];
+          for (int u = 0; u < KG; ++u) wf[ahead % PD][u] = src[(size_t)u * 64];
         }
 #pragma unroll
         for (int u = 0; u < KG; ++u) p[c] = mfma16(af[u], wf[ul % PD][u], p[c]);
@@ -140,6 +180,7 @@ __device__ __forceinline__ void gated_products(const bf16x8* __restrict__ xb, co
         }
       }
     }
+    mm = nxt;
   }
 }
 
@@ -177,6 +218,7 @@ __global__ __launch_bounds__(256) void ring_fwd_kernel(RingFwdArgs p) {
   using TL = Tile<NC>;
   __shared__ bf16x8 xbuf[2][TL::SLOTS];
   __shared__ float psum[2][64];
+  __shared__ float gl[2][16 * GATE_KMAX];
 
   const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, q = lane >> 4, n = lane & 15;
   const int bt = blockIdx.x;
@@ -184,11 +226,13 @@ __global__ __launch_bounds__(256) void ring_fwd_kernel(RingFwdArgs p) {
   const int i0 = 16 * NC * w + NC * n;
   const int N = p.N, B = p.B, T = p.T;
   const float oma = 1.f - p.alpha;
+  const bool staged = p.k <= GATE_KMAX;
 
   float r[4][NC];
   rows_load<NC>(p.r_init, N, B, b0, i0, r);
   write_operand<NC>(xbuf[0], r, w, q, n);
   publish_rowsum<NC>(psum[0], r, w, q, n);
+  if (staged) gates_stage(gl[0], p.A, p.k, T, B, 0, bt, tid);
   if (p.rfrag) {
     pair_store<NC>(p.rfrag, 0, p.nbt, bt, w, lane, r);
     pair_zero_tail<NC>(p.rfrag, T, p.nbt, bt, w, lane);
@@ -198,7 +242,9 @@ __global__ __launch_bounds__(256) void ring_fwd_kernel(RingFwdArgs p) {
   for (int t = 0; t < T; ++t) {
     const int cur = t & 1;
     f32x4 acc[NC];
-    gated_products<NC>(xbuf[cur], (const bf16x8*)p.Wpack, p.A, p.k, T, B, t, b0, p.J1, w, lane, acc);
+    if (staged && t + 1 < T) gates_stage(gl[cur ^ 1], p.A, p.k, T, B, t + 1, bt, tid);
+    gated_products<NC>(xbuf[cur], (const bf16x8*)p.Wpack, p.A, staged ? gl[cur] : nullptr,
+                       staged ? gates_active(gl[cur], p.k, lane) : ~0ull, p.k, T, B, t, b0, p.J1, w, lane, acc);
     float s[4];
     read_rowsum(psum[cur], q, s);
     float d[4][NC];
@@ -234,6 +280,7 @@ __global__ __launch_bounds__(256) void ring_rebuild_saved_kernel(RingFwdArgs p) 
   using TL = Tile<NC>;
   __shared__ bf16x8 xbuf[TL::SLOTS];
   __shared__ float psum[64];
+  __shared__ float gl[16 * GATE_KMAX];
 
   const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, q = lane >> 4, n = lane & 15;
   const int bt = blockIdx.x, t = blockIdx.y;
@@ -248,10 +295,13 @@ __global__ __launch_bounds__(256) void ring_rebuild_saved_kernel(RingFwdArgs p) 
   publish_rowsum<NC>(psum, r, w, q, n);
   pair_store<NC>(p.rfrag, t, p.nbt, bt, w, lane, r);
   if (t == T - 1) pair_zero_tail<NC>(p.rfrag, T, p.nbt, bt, w, lane);
+  const bool staged = p.k <= GATE_KMAX;
+  if (staged) gates_stage(gl, p.A, p.k, T, B, t, bt, tid);
   lds_barrier();
 
   f32x4 acc[NC];
-  gated_products<NC>(xbuf, (const bf16x8*)p.Wpack, p.A, p.k, T, B, t, b0, p.J1, w, lane, acc);
+  gated_products<NC>(xbuf, (const bf16x8*)p.Wpack, p.A, staged ? gl : nullptr, staged ? gates_active(gl, p.k, lane) : ~0ull,
+                     p.k, T, B, t, b0, p.J1, w, lane, acc);
   float s[4];
   read_rowsum(psum, q, s);
   float d[4][NC];
@@ -290,6 +340,7 @@ __global__ __launch_bounds__(256) void ring_bptt_kernel(RingBpttArgs p) {
   using TL = Tile<NC>;
   __shared__ bf16x8 xbuf[2][TL::SLOTS];
   __shared__ float psum[2][64];
+  __shared__ float gl[2][16 * GATE_KMAX];
   extern __shared__ float ga_buf[];   // [2][k][4 waves][16 rows] when GA
 
   const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, q = lane >> 4, n = lane & 15;
@@ -299,6 +350,7 @@ __global__ __launch_bounds__(256) void ring_bptt_kernel(RingBpttArgs p) {
   const int N = p.N, B = p.B, T = p.T;
   const float oma = 1.f - p.alpha;
 
+  const bool staged = p.k <= GATE_KMAX;
   float carry[4][NC];
 #pragma unroll
   for (int e = 0; e < 4; ++e)
@@ -321,7 +373,11 @@ __global__ __launch_bounds__(256) void ring_bptt_kernel(RingBpttArgs p) {
     write_operand<NC>(xbuf[cur], g, w, q, n);
     publish_rowsum<NC>(psum[cur], g, w, q, n);
     pair_store<NC>(p.gfrag, t, p.nbt, bt, w, lane, g);
+    // this step's gates: the buffer was last read two steps ago, before the previous barrier
+    if (staged) gates_stage(gl[cur], p.A, p.k, T, B, t, bt, tid);
     lds_barrier();
+    const float* glt = staged ? gl[cur] : nullptr;
+    const unsigned long long active = staged ? gates_active(gl[cur], p.k, lane) : ~0ull;
 
     f32x4 acc[NC];
     if constexpr (GA) {
@@ -329,10 +385,10 @@ __global__ __launch_bounds__(256) void ring_bptt_kernel(RingBpttArgs p) {
       if (t + 1 < T) bptt_flush_grad_A(p, ga_buf + (cur ^ 1) * p.k * 64, t + 1, bt, tid);
       float rp[4][NC];
       rows_load<NC>(t == 0 ? p.r_init : p.hist + (size_t)(t - 1) * B * N, N, B, b0, i0, rp);
-      gated_products<NC, true>(xbuf[cur], (const bf16x8*)p.Wpack, p.A, p.k, T, B, t, b0, p.J1, w, lane, acc, rp,
-                               ga_buf + cur * p.k * 64);
+      gated_products<NC, true>(xbuf[cur], (const bf16x8*)p.Wpack, p.A, glt, active, p.k, T, B, t, b0, p.J1, w, lane,
+                               acc, rp, ga_buf + cur * p.k * 64);
     } else {
-      gated_products<NC>(xbuf[cur], (const bf16x8*)p.Wpack, p.A, p.k, T, B, t, b0, p.J1, w, lane, acc);
+      gated_products<NC>(xbuf[cur], (const bf16x8*)p.Wpack, p.A, glt, active, p.k, T, B, t, b0, p.J1, w, lane, acc);
     }
     float s[4];
     read_rowsum(psum[cur], q, s);

@@ -42,6 +42,9 @@ CASES = [
     ("n512_tanh",      32,  16,  2, 512, "tanh", -0.1, 0.1, "dense"),
     ("n64_one_step",   16,   1,  2,  64, "gelu", -0.1, 0.1, "dense"),
     ("odd_shapes",     17,   9,  5, 130, "gelu", -0.05, 0.2, "spread"),
+    ("n64_lr",         32,   9,  2,  64, "tanh", -0.1, 0.1, "lr"),        # zero gates at the start: matrices skipped
+    ("n48_dense",      16,   3,  2,  48, "tanh", -0.1, 0.1, "dense"),
+    ("n512_k16_pad",   32,   6, 16, 512, "gelu", -0.1, 0.1, "lr"),        # zero-padded channels, widest tiling
 ]
 
 
