@@ -40,6 +40,8 @@ WORKLOADS = {
     "train_n120_b64_t120_tanh": dict(N=120, B=64, T=120, k=2, act="tanh", J0=-1.0 / 120, J1=1.0, mode="train"),
     "infer_n256_b1024_t120_relu": dict(N=256, B=1024, T=120, k=2, act="relu", J0=-1.0 / 256, J1=1.0, mode="infer"),
     "train_n512_b8192_t512_tanh": dict(N=512, B=8192, T=512, k=2, act="tanh", J0=-1.0 / 512, J1=1.0, mode="train"),
+    # the reference training script's own defaults: 16 action channels of which two are driven (zero padding)
+    "train_n256_b128_t100_k16pad_gelu": dict(N=256, B=128, T=100, k=16, act="gelu", J0=-0.1, J1=0.1, mode="train"),
 }
 
 
