@@ -34,9 +34,9 @@ MEASURED_TRAFFIC_BYTES = {
 }
 
 WORKLOADS = {
-    # BASELINE config 2 (headline; the default and the only workload the metric is quoted on)
+    # the headline training shape (the default and the only workload the metric is quoted on)
     "train_n256_b4096_t120_gelu": dict(N=256, B=4096, T=120, k=2, act="gelu", J0=-1.0 / 256, J1=1.0, mode="train"),
-    # the other BASELINE shapes, for reference figures (run with --workload; pick --steps to taste)
+    # the other benchmark shapes, for reference figures (run with --workload; pick --steps to taste)
     "train_n120_b64_t120_tanh": dict(N=120, B=64, T=120, k=2, act="tanh", J0=-1.0 / 120, J1=1.0, mode="train"),
     "infer_n256_b1024_t120_relu": dict(N=256, B=1024, T=120, k=2, act="relu", J0=-1.0 / 256, J1=1.0, mode="infer"),
     "train_n512_b8192_t512_tanh": dict(N=512, B=8192, T=512, k=2, act="tanh", J0=-1.0 / 512, J1=1.0, mode="train"),
@@ -117,7 +117,8 @@ def main():
                          "FETCH_SIZE / WRITE_SIZE counters")
     args = ap.parse_args()
     if args.gpus != 1:
-        sys.exit("bench.py: this build runs on exactly one GPU (the batch shards trivially; see DESIGN.md); use --gpus 1")
+        sys.exit("bench.py: this build runs on exactly one GPU (samples are independent, so the batch shards trivially "
+                 "over more); use --gpus 1")
 
     import torch
     from rnn_train_ring_attractor_amd import _lib, ring_rnn_cuda_func

@@ -19,7 +19,7 @@ def _t(x, dev):
 
 
 def test_config1_inference_full_size(gpu_device):
-    """Forward only: N=256, B=1024, T=120, relu, zero ratio 0.5 (BASELINE config 1)."""
+    """Forward only: N=256, B=1024, T=120, relu, zero ratio 0.5 (the forward-only inference shape)."""
     from rnn_train_ring_attractor_amd import ring_rnn_cuda_func
     print("[case] config1 N=256 B=1024 T=120 relu", flush=True)
     B, T, k, N = 1024, 120, 2, 256
@@ -41,7 +41,7 @@ def test_config1_inference_full_size(gpu_device):
 
 
 def test_config3_geometry_long_sequence(gpu_device):
-    """N=512, T=512, tanh (BASELINE config 3 at a batch the oracle can follow): 512 leak steps must not drift."""
+    """N=512, T=512, tanh (the long-sequence shape at a batch the oracle can follow): 512 leak steps must not drift."""
     from rnn_train_ring_attractor_amd import ring_rnn_cuda_func
     print("[case] config3 N=512 B=32 T=512 tanh", flush=True)
     B, T, k, N = 32, 512, 2, 512
@@ -63,7 +63,7 @@ def test_config3_geometry_long_sequence(gpu_device):
 
 
 def test_headline_size_properties(gpu_device):
-    """N=256, B=4096, T=120, gelu (BASELINE config 2).  The fp64 oracle checks a 64-row slice; the rest
+    """N=256, B=4096, T=120, gelu (the headline training shape).  The fp64 oracle checks a 64-row slice; the rest
     follows from properties that do not depend on the size."""
     from rnn_train_ring_attractor_amd import ring_rnn_cuda_func
     print("[case] headline N=256 B=4096 T=120 gelu", flush=True)
