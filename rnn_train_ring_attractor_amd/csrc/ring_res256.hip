@@ -17,6 +17,7 @@ constexpr int R_KCH = 8;
 constexpr int R_WLDS_SLOTS = 4 * R_NC * R_KCH * 64;   // 16-byte slots of the LDS-resident matrix
 constexpr int R_XSLOTS = R_KCH * 4 * XG;
 constexpr int R_GCH = 32;                             // time steps of action gates staged per LDS chunk
+constexpr int R_BPTT_DEPTH = 2;                       // BPTT steps whose grad_output / F' loads are in flight
 constexpr size_t R_LDS_BYTES = (size_t)(R_WLDS_SLOTS + 2 * R_XSLOTS) * 16 + 2 * R_GCH * 16 * 8;   // BPTT layout
 
 // Action gates (A[b,t,0], A[b,t,1]) reach the lanes through LDS in chunks of R_GCH steps, so the
@@ -327,7 +328,7 @@ __global__ __launch_bounds__(512) void ring_fwd_res256_kernel(RingFwdArgs p) {
 
 // ------------------------------------------------------------------------------------------------
 // BPTT recurrence, transposed weights resident.  Same contract as ring_bptt_kernel<4> with k == 2.
-// grad_output and F' are prefetched two steps ahead into two register stages (loop unrolled by 2).
+// grad_output and F' are prefetched R_BPTT_DEPTH steps ahead into register stages (loop unrolled to match).
 // ------------------------------------------------------------------------------------------------
 namespace {
 
@@ -419,9 +420,9 @@ __global__ __launch_bounds__(256) void ring_bptt_res256_kernel(RingBpttArgs p) {
     }
 
   pair_zero_tail<R_NC>(p.gfrag, T, p.nbt, bt, w, lane);
-  BpttStage st[2];
-  bptt_stage_load<FULL>(p, T - 1, bt, w, lane, b0, i0, st[0]);
-  bptt_stage_load<FULL>(p, T - 2, bt, w, lane, b0, i0, st[1]);
+  BpttStage st[R_BPTT_DEPTH];
+#pragma unroll
+  for (int d = 0; d < R_BPTT_DEPTH; ++d) bptt_stage_load<FULL>(p, T - 1 - d, bt, w, lane, b0, i0, st[d]);
   GateStage gs;
   gates_fetch(p.A, T, B, bt, 0, -1, tid, gs);
   gates_publish(gbuf, tid, B, bt, gs);
@@ -430,19 +431,19 @@ __global__ __launch_bounds__(256) void ring_bptt_res256_kernel(RingBpttArgs p) {
   for (int u = 0; u < R_KCH / 2; ++u) w0[0][u] = wl[u * 64];
   // (the first lds_barrier inside the loop also publishes the gates)
 
-  for (int u0 = 0; u0 < T; u0 += 2) {
+  for (int u0 = 0; u0 < T; u0 += R_BPTT_DEPTH) {
 #pragma unroll
-    for (int half = 0; half < 2; ++half) {
+    for (int half = 0; half < R_BPTT_DEPTH; ++half) {
       const int u = u0 + half;
       if (u >= T) break;
       const int t = T - 1 - u;
       const int cur = u & 1, ci = u / R_GCH, l = u % R_GCH;
       if (l == 0 && (ci + 1) * R_GCH < T) gates_fetch(p.A, T, B, bt, ci + 1, -1, tid, gs);
       BpttStage& S = st[half];
-      // issued after this stage's six loads: the previous step's four operand-copy stores and the other
-      // stage's six loads.  The counter is in order, so "at most ten outstanding" means this stage landed;
-      // a smaller number would also wait for those stores to be acknowledged by memory.
-      if constexpr (FULL) bptt_stage_wait<10>(S);
+      // issued after this stage's six loads: per step since then, four operand-copy stores and another
+      // stage's six loads.  The counter is in order, so "at most 10 * (depth - 1) outstanding" means this
+      // stage landed; a smaller number would also wait for later loads and for store acknowledgements.
+      if constexpr (FULL) bptt_stage_wait<10 * (R_BPTT_DEPTH - 1)>(S);
 
       float G[4][R_NC], g[4][R_NC];
 #pragma unroll
@@ -455,7 +456,7 @@ __global__ __launch_bounds__(256) void ring_bptt_res256_kernel(RingBpttArgs p) {
       bf16x8* xb = xbuf + cur * R_XSLOTS;
       write_operand<R_NC>(xb, g, w, q, n);
       pair_store<R_NC>(p.gfrag, t, p.nbt, bt, w, lane, g);
-      bptt_stage_load<FULL>(p, t - 2, bt, w, lane, b0, i0, S);
+      bptt_stage_load<FULL>(p, t - R_BPTT_DEPTH, bt, w, lane, b0, i0, S);
       lds_barrier();
 
       bf16x8 af[R_KCH];
@@ -505,11 +506,11 @@ __global__ __launch_bounds__(256) void ring_bptt_res256_kernel(RingBpttArgs p) {
       if (l == R_GCH - 1 && u + 1 < T) gates_publish(gbuf + ((ci + 1) & 1) * R_GCH * 16, tid, B, bt, gs);
     }
   }
-  // the last two iterations prefetched (clamped) steps that are never consumed: let those loads land
+  // the last iterations prefetched (clamped) steps that are never consumed: let those loads land
   // while their destination registers are still reserved, before anything below reuses them
   if constexpr (FULL) {
-    bptt_stage_wait<0>(st[0]);
-    bptt_stage_wait<0>(st[1]);
+#pragma unroll
+    for (int d = 0; d < R_BPTT_DEPTH; ++d) bptt_stage_wait<0>(st[d]);
   }
   if (p.grad_r_init) rows_store<R_NC>(p.grad_r_init, N, B, b0, i0, carry);
 }
