@@ -76,7 +76,9 @@ RINGATTR_API int ringattr_fwd(const void* A, const void* Wa, float J0, float J1,
 
 /* Reverse-time BPTT + weight gradients.
  * Replaces bwd_cuda (cpp/bwd.cu:4-52) and cpp/bwd.cpp:34-99.
- * `saved` may be NULL: F'(re) is then recomputed from bump_history.
+ * `saved` may be NULL: the saved record is then recomputed, from bump_history
+ * or (weight-resident geometry: a_dim == 2, 128 < N <= 256) by running the
+ * recurrence again from r_init, which reproduces the forward's own numbers.
  * grad_A [B,T,k] and grad_r_init [B,N] are optional outputs (NULL = skip), written
  * rather than accumulated; the reference returns None for both
  * (cpp/ring_rnn_cuda.py:144).  Asking for grad_A (a_dim <= 48) adds one read of

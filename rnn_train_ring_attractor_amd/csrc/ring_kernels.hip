@@ -657,8 +657,16 @@ hipError_t ring_launch_fwd(const RingFwdArgs& a, int NCv, hipStream_t st) {
   return hipGetLastError();
 }
 
+// For the weight-resident geometry the saved record is rebuilt by running the forward recurrence again
+// from r_init with its history stores switched off (a.hist is not read): the same kernel, the same
+// numbers the forward would have saved, and no pass over the weights per (batch tile, step).
 hipError_t ring_launch_rebuild(const RingFwdArgs& a, int NCv, hipStream_t st) {
   ProfScope prof(2, st);
+  if (ring_uses_resident(a.N, a.k)) {
+    RingFwdArgs f = a;
+    f.hist = nullptr;
+    return ring_launch_fwd_res256(f, st);
+  }
   RING_DISPATCH_NC(NCv, RING_DISPATCH_ACT(a.act, hipLaunchKernelGGL((ring_rebuild_saved_kernel<NC, ACT>), dim3(a.nbt, a.T), dim3(256), 0, st, a)));
   return hipGetLastError();
 }

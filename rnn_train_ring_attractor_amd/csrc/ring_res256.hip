@@ -194,6 +194,7 @@ __global__ __launch_bounds__(512) void ring_fwd_res256_kernel(RingFwdArgs p) {
   auto emit_store = [&](int t, int slot) {
     __builtin_amdgcn_sched_barrier(0);
     if (slot < 4) {
+      if (p.hist == nullptr) return;   // recompute of the saved record only: the history already exists
       const int e = slot;
       float* dst = p.hist + ((size_t)t * B + b0 + e) * N + i0;
       if constexpr (FULL) {

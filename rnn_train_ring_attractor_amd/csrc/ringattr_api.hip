@@ -193,7 +193,7 @@ int ringattr_bwd(const void* grad_output, const void* A, const void* Wa, float J
     _Float16* d = (_Float16*)ws;
     ws += g.side_bytes;
     __bf16* r = (__bf16*)ws;
-    hipError_t e = ring_launch_pack((const float*)Wo, (const float*)Wa, wf, N, a_dim, g.NC, 0, 0, 1.f, st);
+    hipError_t e = ring_launch_pack((const float*)Wo, (const float*)Wa, wf, N, a_dim, g.NC, 0, ring_uses_resident(N, a_dim) ? 1 : 0, 1.f, st);
     if (e != hipSuccess) return hip_fail(e, "pack weights");
     RingFwdArgs f;
     f.A = (const float*)A;
