@@ -90,6 +90,25 @@ RINGATTR_API int ringattr_bwd(const void* grad_output, const void* A, const void
                  const void* saved, void* grad_A, void* grad_r_init,
                  void* workspace, size_t workspace_bytes, void* stream);
 
+/* Fused decode + loss head over bump_history [T,B,N]: the cosine-similarity head-direction loss of the
+ * max-normalised cosine read-out plus bump_weight times the bump-amplitude loss.  No counterpart in the
+ * reference's extension: it replaces the chain of torch tensor ops in the training script (root
+ * train_general_ring_no_gain.py:113-116, 324-330; train/train_ring_attractor.py:190-220, 275-298), whose
+ * W_delta7 read-out has rank two, so a row contributes through three sums over its N values.
+ *   target_angle      [B,T] true angles (radians)
+ *   target_amplitude  [B] or NULL (NULL: the amplitude of the first step, which then also receives gradient)
+ *   loss_out          3 floats on the device: total, cos-sim loss, amplitude loss
+ *   upstream          one float on the device (d objective / d total) or NULL for 1
+ *   grad_history      [T,B,N], overwritten with d total / d bump_history * upstream
+ * ringattr_loss_bwd needs the workspace ringattr_loss_fwd filled for the same inputs.  N <= 1024. */
+RINGATTR_API size_t ringattr_loss_workspace_bytes(int N, int seq_len, int batch_size);
+RINGATTR_API int ringattr_loss_fwd(const void* bump_history, const void* target_angle, const void* target_amplitude,
+                      float bump_weight, void* loss_out, int N, int seq_len, int batch_size,
+                      void* workspace, size_t workspace_bytes, void* stream);
+RINGATTR_API int ringattr_loss_bwd(const void* bump_history, const void* target_angle, const void* target_amplitude,
+                      float bump_weight, const void* upstream, void* grad_history, int N, int seq_len,
+                      int batch_size, const void* workspace, size_t workspace_bytes, void* stream);
+
 /* Per-kernel timing for benchmarks; no counterpart in the reference.  While enabled, every kernel
  * launch is bracketed by two HIP events recorded on the launch stream.  ringattr_profile_read waits
  * for the recorded events, adds their durations into ms[RINGATTR_NUM_KERNELS] and the launch counts

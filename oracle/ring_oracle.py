@@ -316,3 +316,39 @@ def max_rel_err(x: np.ndarray, ref: np.ndarray) -> float:
     x = np.asarray(x, np.float64)
     ref = np.asarray(ref, np.float64)
     return float(np.max(np.abs(x - ref)) / (np.max(np.abs(ref)) + 1e-300))
+
+
+def loss_pair_rank2(bump_tbn, target_angle, bump_weight=0.2, target_amplitude=None):
+    """The training loss pair and its gradient through the rank-two form of the read-out.
+
+    Restates root train_general_ring_no_gain.py:113-116, 324-330 and train/train_ring_attractor.py:190-220,
+    275-298: W_delta7[i][j] = cos(phi_i - phi_j) makes proj_j = C cos(phi_j) + S sin(phi_j) with
+    C = sum_i r_i cos(phi_i), S = sum_i r_i sin(phi_i); the positive row maximum cancels in atan2.
+    Returns (total, cos_loss, amp_loss, d total / d bump_tbn).  Pinned in tests/test_oracle_helpers.py against the
+    literal chain (read-out, normalisation, decode, both losses) and its autograd gradient."""
+    r = np.asarray(bump_tbn, np.float64)
+    T, B, N = r.shape
+    a = np.asarray(target_angle, np.float64).T                      # [T,B]
+    j = np.arange(N)
+    phi = 2 * np.pi * j / N
+    pa = np.linspace(0.0, 2 * np.pi, N)
+    a1, a2 = np.sum(np.cos(phi) * np.cos(pa)), np.sum(np.sin(phi) * np.cos(pa))
+    b1, b2 = np.sum(np.cos(phi) * np.sin(pa)), np.sum(np.sin(phi) * np.sin(pa))
+    C, S = r @ np.cos(phi), r @ np.sin(phi)
+    X, Y = C * a1 + S * a2, C * b1 + S * b2
+    theta = np.arctan2(Y, X)
+    cos_loss = np.mean((np.cos(theta) - np.cos(a)) ** 2 + (np.sin(theta) - np.sin(a)) ** 2)
+    amp = np.abs(r).sum(axis=2)                                      # [T,B]
+    own = target_amplitude is None
+    tgt = amp[0] if own else np.asarray(target_amplitude, np.float64).reshape(B)
+    dev = amp - tgt[None, :]
+    amp_loss = np.mean(dev ** 2)
+    rows = T * B
+    dth = 2 * np.sin(theta - a) / np.maximum(X * X + Y * Y, 1e-300) / rows
+    kc, ks = dth * (X * b1 - Y * a1), dth * (X * b2 - Y * a2)
+    beta = 2 * dev
+    if own:
+        beta[0] -= 2 * dev.sum(axis=0)
+    beta = beta * bump_weight / rows
+    grad = kc[..., None] * np.cos(phi) + ks[..., None] * np.sin(phi) + beta[..., None] * np.sign(r)
+    return cos_loss + bump_weight * amp_loss, cos_loss, amp_loss, grad

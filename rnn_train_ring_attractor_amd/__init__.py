@@ -4,6 +4,7 @@ chongxi/rnn_train_ring_attractor's cpp/ring_rnn_cuda.py."""
 _EXPORTS = {
     "ring_rnn_cuda_func": "ring_rnn_cuda", "RingRnnCudaFunc": "ring_rnn_cuda",
     "fwd_cuda": "rnn_cuda", "bwd_cuda": "rnn_cuda",
+    "ring_loss_pair": "loss_head", "RingLossPair": "loss_head",
 }
 
 

@@ -63,6 +63,14 @@ bool ring_dw_tiled_applicable(int NC);
 int ring_dw_tiled_nz(int NC, int k, long nchunk);
 hipError_t ring_launch_dw_tiled(const RingDwArgs& a, int NC, hipStream_t st);
 
+// Fused decode + loss head over the state history (ring_loss.hip).
+size_t ring_loss_workspace_bytes(int T, int B);
+hipError_t ring_launch_loss_fwd(const float* hist, const float* angle, const float* target_amp, float bump_weight,
+                                float* loss_out, int N, int T, int B, void* workspace, hipStream_t st);
+hipError_t ring_launch_loss_bwd(const float* hist, const float* angle, const float* target_amp, float bump_weight,
+                                const float* upstream, float* grad_hist, int N, int T, int B, const void* workspace,
+                                hipStream_t st);
+
 // Optional event bracketing of launches (benchmark support).
 void ring_profile_set(bool on);
 bool ring_profile_on();

@@ -269,6 +269,55 @@ int ringattr_bwd(const void* grad_output, const void* A, const void* Wa, float J
   return RINGATTR_OK;
 }
 
+size_t ringattr_loss_workspace_bytes(int N, int seq_len, int batch_size) {
+  if (N <= 0 || seq_len <= 0 || batch_size <= 0) {
+    fail(RINGATTR_ERR_INVALID, "N, seq_len, batch_size must be positive (got %d, %d, %d)", N, seq_len, batch_size);
+    return 0;
+  }
+  if (N > 1024) {
+    fail(RINGATTR_ERR_INVALID, "the loss head supports N <= 1024 (got %d)", N);
+    return 0;
+  }
+  return align_up(ring_loss_workspace_bytes(seq_len, batch_size));
+}
+
+int ringattr_loss_fwd(const void* bump_history, const void* target_angle, const void* target_amplitude, float bump_weight,
+                      void* loss_out, int N, int seq_len, int batch_size, void* workspace, size_t workspace_bytes,
+                      void* stream) {
+  const size_t need = ringattr_loss_workspace_bytes(N, seq_len, batch_size);
+  if (need == 0) return RINGATTR_ERR_INVALID;
+  if (!bump_history || !target_angle || !loss_out) return fail(RINGATTR_ERR_INVALID, "ringattr_loss_fwd: null tensor pointer");
+  if (!aligned16(bump_history) || !aligned16(workspace))
+    return fail(RINGATTR_ERR_INVALID, "ringattr_loss_fwd: bump_history and workspace must be 16-byte aligned");
+  if (!workspace || workspace_bytes < need)
+    return fail(RINGATTR_ERR_WORKSPACE, "ringattr_loss_fwd: workspace of %zu bytes needed, %zu given", need,
+                workspace ? workspace_bytes : (size_t)0);
+  hipError_t e = ring_launch_loss_fwd((const float*)bump_history, (const float*)target_angle, (const float*)target_amplitude,
+                                      bump_weight, (float*)loss_out, N, seq_len, batch_size, workspace,
+                                      static_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return hip_fail(e, "loss head forward launch");
+  return RINGATTR_OK;
+}
+
+int ringattr_loss_bwd(const void* bump_history, const void* target_angle, const void* target_amplitude, float bump_weight,
+                      const void* upstream, void* grad_history, int N, int seq_len, int batch_size, const void* workspace,
+                      size_t workspace_bytes, void* stream) {
+  const size_t need = ringattr_loss_workspace_bytes(N, seq_len, batch_size);
+  if (need == 0) return RINGATTR_ERR_INVALID;
+  if (!bump_history || !target_angle || !grad_history)
+    return fail(RINGATTR_ERR_INVALID, "ringattr_loss_bwd: null tensor pointer");
+  if (!aligned16(bump_history) || !aligned16(grad_history) || !aligned16(workspace))
+    return fail(RINGATTR_ERR_INVALID, "ringattr_loss_bwd: bump_history, grad_history and workspace must be 16-byte aligned");
+  if (!workspace || workspace_bytes < need)
+    return fail(RINGATTR_ERR_WORKSPACE, "ringattr_loss_bwd: workspace of %zu bytes needed, %zu given", need,
+                workspace ? workspace_bytes : (size_t)0);
+  hipError_t e = ring_launch_loss_bwd((const float*)bump_history, (const float*)target_angle, (const float*)target_amplitude,
+                                      bump_weight, (const float*)upstream, (float*)grad_history, N, seq_len, batch_size,
+                                      workspace, static_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return hip_fail(e, "loss head backward launch");
+  return RINGATTR_OK;
+}
+
 int ringattr_profile_enable(int on) {
   ring_profile_set(on != 0);
   return RINGATTR_OK;

@@ -168,15 +168,19 @@ class GeneralizedRingAttractorNoGain(nn.Module):
         else:
             raise ValueError(f"Unknown initialization: {initialization}")
 
-    def forward(self, action_signal, r_init=None):
+    def forward_history(self, action_signal, r_init=None):
+        """bump_history [T,B,N] as the operator returns it (no read-out): the input of `ring_loss_pair`."""
         from .ring_rnn_cuda import ring_rnn_cuda_func
         batch_size, _, action_dim = action_signal.shape
         assert action_dim == self.action_dim, f"Expected action_dim {self.action_dim}, got {action_dim}"
         if r_init is None:
             angle = torch.full((batch_size,), math.pi, device=self.Wo.device)
             r_init = create_initial_bump(angle, self.num_neurons, device=self.Wo.device)
-        bump = ring_rnn_cuda_func(action_signal=action_signal, Wa=self.Wa, J0=self.J0, J1=self.J1, Wo=self.Wo,
-                                  r_init=r_init, alpha=0.15, activation=self.activation_name).permute(1, 0, 2)
+        return ring_rnn_cuda_func(action_signal=action_signal, Wa=self.Wa, J0=self.J0, J1=self.J1, Wo=self.Wo,
+                                  r_init=r_init, alpha=0.15, activation=self.activation_name)
+
+    def forward(self, action_signal, r_init=None):
+        bump = self.forward_history(action_signal, r_init).permute(1, 0, 2)
         proj = bump @ self.W_delta7
         return (proj / proj.max(dim=2, keepdim=True)[0]).clone(), bump.clone()
 

@@ -22,7 +22,8 @@ def _header_symbols():
 def test_library_exports_every_declared_symbol():
     lib = _lib.load()
     names = _header_symbols()
-    assert {"ringattr_fwd", "ringattr_bwd", "fwd_cuda", "bwd_cuda", "ringattr_saved_bytes"} <= set(names)
+    assert {"ringattr_fwd", "ringattr_bwd", "fwd_cuda", "bwd_cuda", "ringattr_saved_bytes", "ringattr_loss_fwd",
+            "ringattr_loss_bwd", "ringattr_loss_workspace_bytes"} <= set(names)
     for n in names:
         assert hasattr(lib, n), n
     assert sorted(_lib.PROTOTYPES) == names          # the ctypes table and the header agree

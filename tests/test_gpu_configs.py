@@ -189,6 +189,12 @@ def test_training_driver_reduces_loss(gpu_device):
                                lr=3e-3, activation="gelu", log_every=0, seed=1)
     assert all(np.isfinite(hist))
     assert np.mean(hist[-5:]) < np.mean(hist[:5])
+    # the same run with the fused loss head follows the same loss curve (same seed, same data)
+    _, hist_fused = drv.run_training(action_dim=2, num_neurons=128, training_steps=40, batch_size=64, seq_len=60,
+                                     lr=3e-3, activation="gelu", log_every=0, seed=1, fused_loss=True)
+    assert all(np.isfinite(hist_fused))
+    assert abs(hist_fused[0] - hist[0]) <= 1e-3 * abs(hist[0])
+    assert np.mean(hist_fused[-5:]) < np.mean(hist_fused[:5])
 
 
 def test_reference_signature_entry_points(gpu_device):

@@ -1,0 +1,68 @@
+"""Fused decode + loss head (ringattr_loss_fwd / ringattr_loss_bwd) against the fp64 oracle, whose rank-two form is
+itself pinned against the reference's literal chain of tensor ops and its autograd (tests/test_oracle_helpers.py)."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import ring_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+def _bumps(rng, T, B, N):
+    centre = rng.random((T, B)) * 2 * np.pi
+    idx = np.arange(N)
+    return (0.3 * np.exp(2.0 * (np.cos(2 * np.pi * idx / N - centre[..., None]) - 1.0))
+            + 0.02 * rng.standard_normal((T, B, N))).astype(np.float32)
+
+
+@pytest.mark.parametrize("T,B,N,own", [(20, 37, 256, True), (7, 5, 130, True), (9, 16, 512, False), (3, 4, 24, True),
+                                        (5, 3, 700, False)], ids=["n256", "n130_scalar", "n512_given_target", "n24", "n700"])
+def test_loss_and_gradient_match_the_oracle(T, B, N, own, gpu_device):
+    from rnn_train_ring_attractor_amd import ring_loss_pair
+    print(f"[case] loss head T={T} B={B} N={N}", flush=True)
+    rng = np.random.default_rng(T * 1000 + N)
+    bump = _bumps(rng, T, B, N)
+    angle = (rng.random((B, T)) * 2 * np.pi).astype(np.float32)
+    tgt = None if own else (rng.random(B) + 1.0).astype(np.float32)
+    want_total, want_cos, want_amp, want_grad = O.loss_pair_rank2(bump, angle, 0.2, tgt)
+    h = torch.tensor(bump, device=gpu_device, requires_grad=True)
+    total, lc, la = ring_loss_pair(h, torch.tensor(angle, device=gpu_device), 0.2,
+                                   None if own else torch.tensor(tgt, device=gpu_device))
+    (3.0 * total).backward()                      # an upstream factor other than one
+    torch.cuda.synchronize()
+    assert abs(float(total) - want_total) <= 2e-5 * max(1.0, abs(want_total))
+    assert abs(float(lc) - want_cos) <= 2e-5 * max(1.0, abs(want_cos))
+    assert abs(float(la) - want_amp) <= 2e-5 * max(1.0, abs(want_amp))
+    got = h.grad.cpu().numpy()
+    assert np.isfinite(got).all()
+    assert O.max_rel_err(got, 3.0 * want_grad) <= 2e-4
+    assert O.cosine(got, 3.0 * want_grad) >= 0.999999
+
+
+def test_loss_head_agrees_with_the_torch_chain_on_operator_output(gpu_device):
+    """End to end on the GPU: operator -> fused loss head, against operator -> the torch chain of the training script."""
+    from rnn_train_ring_attractor_amd import host, ring_loss_pair, ring_rnn_cuda_func
+    from tests.ring_cases import make_problem
+    print("[case] loss head after the operator N=256 B=48 T=30", flush=True)
+    p = make_problem(77, 48, 30, 2, 256, weights="perfect")
+    t = lambda x: torch.tensor(x, device=gpu_device)
+    angle = t(p["angle"])
+    grads = []
+    for fused in (True, False):
+        Wa, Wo = t(p["Wa"]).requires_grad_(True), t(p["Wo"]).requires_grad_(True)
+        hist = ring_rnn_cuda_func(t(p["A"]), Wa, -1.0 / 256, 1.0 / 128, Wo, t(p["r0"]), 0.15, "tanh")
+        if fused:
+            total, _, _ = ring_loss_pair(hist, angle, 0.2)
+        else:
+            bump = hist.permute(1, 0, 2)
+            idx = torch.arange(256, dtype=torch.float32, device=gpu_device)
+            proj = bump @ torch.cos(2 * np.pi * (idx[:, None] - idx[None, :]) / 256)
+            total = (host.cosine_similarity_loss(proj / proj.max(dim=2, keepdim=True)[0], angle)
+                     + 0.2 * host.bump_amplitude_loss(bump))
+        total.backward()
+        grads.append((float(total), Wo.grad.cpu().numpy(), Wa.grad.cpu().numpy()))
+    torch.cuda.synchronize()
+    assert abs(grads[0][0] - grads[1][0]) <= 1e-4 * max(1.0, abs(grads[1][0]))
+    assert O.cosine(grads[0][1], grads[1][1]) >= 0.9999 and O.cosine(grads[0][2], grads[1][2]) >= 0.9999
+    assert O.max_rel_err(grads[0][1], grads[1][1]) <= 2e-3

@@ -132,3 +132,27 @@ def test_comparison_helpers():
     assert abs(O.cosine(a, 2 * a) - 1.0) < 1e-15
     assert abs(O.cosine(a, -a) + 1.0) < 1e-15
     assert abs(O.max_rel_err(a + np.array([0, 0, 0.3]), a) - 0.1) < 1e-15
+
+
+def test_rank_two_loss_head_matches_the_literal_chain_and_its_autograd():
+    """loss_pair_rank2 (what the fused loss kernels implement) against the reference's chain of tensor ops:
+    read-out through W_delta7, max normalisation, atan2 decode, both losses, and torch autograd of all that."""
+    import torch
+    from oracle import torch_port as TP
+    rng = np.random.default_rng(5)
+    for (T, B, N, own) in [(6, 5, 24, True), (4, 3, 33, False), (3, 2, 256, True)]:
+        angle = rng.random((B, T)) * 2 * np.pi
+        centre = rng.random((T, B)) * 2 * np.pi
+        idx = np.arange(N)
+        bump = 0.3 * np.exp(2.0 * (np.cos(2 * np.pi * idx / N - centre[..., None]) - 1.0)) + 0.02 * rng.standard_normal((T, B, N))
+        tgt = None if own else rng.random(B) + 1.0
+        total, lc, la, grad = O.loss_pair_rank2(bump, angle, 0.2, tgt)
+        h = torch.tensor(bump, dtype=torch.float64, requires_grad=True)
+        ref = TP.loss_pair(h, torch.tensor(angle), 0.2, None if own else torch.tensor(tgt).reshape(B, 1))
+        ref.backward()
+        assert abs(total - float(ref)) <= 1e-10 * max(1.0, abs(float(ref)))
+        np.testing.assert_allclose(grad, h.grad.numpy(), rtol=0, atol=1e-9 * np.abs(h.grad.numpy()).max() + 1e-14)
+        # the parts
+        b = np.transpose(bump, (1, 0, 2))
+        assert abs(lc - O.cosine_similarity_loss(O.readout(b), angle)) <= 1e-10
+        assert abs(la - O.bump_amplitude_loss(b, None if own else tgt.reshape(B, 1))) <= 1e-10

@@ -1,5 +1,7 @@
 """Training driver with the reference script's import lines and call pattern (no plotting):
-AV batches -> action signal -> initial bump -> ring_rnn_cuda_func -> loss pair -> clip -> Adam."""
+AV batches -> action signal -> initial bump -> ring_rnn_cuda_func -> loss pair -> clip -> Adam.
+fused_loss=True computes the same loss pair and its gradient with the fused HIP loss head instead of the chain
+of torch tensor ops (one pass over the history each way instead of about a dozen)."""
 import numpy as np
 
 from utils.generate_av_integration_data import AVIntegrationDataset
@@ -10,7 +12,7 @@ from rnn_train_ring_attractor_amd.host import GeneralizedRingAttractorNoGain, av
 
 
 def run_training(action_dim=2, num_neurons=256, training_steps=1000, batch_size=128, seq_len=100, lr=1e-3,
-                 activation="gelu", log_every=10, seed=0):
+                 activation="gelu", log_every=10, seed=0, fused_loss=False):
     torch.manual_seed(seed)
     device = torch.device("cuda")
     data = AVIntegrationDataset(num_samples=min(training_steps * batch_size, 200_000), seq_len=seq_len,
@@ -22,9 +24,13 @@ def run_training(action_dim=2, num_neurons=256, training_steps=1000, batch_size=
         av, target = data.generate_batch(batch_size)
         action = av_to_action_signal_ND(av, action_dim)
         r_init = create_initial_bump(target[:, 0], num_neurons, device=device)
-        wave, bump = model(action, r_init=r_init)
-        loss = cosine_similarity_loss(wave, target)
-        total = loss + 0.2 * bump_amplitude_loss(bump)
+        if fused_loss:
+            from rnn_train_ring_attractor_amd import ring_loss_pair
+            total, loss, _ = ring_loss_pair(model.forward_history(action, r_init=r_init), target, 0.2)
+        else:
+            wave, bump = model(action, r_init=r_init)
+            loss = cosine_similarity_loss(wave, target)
+            total = loss + 0.2 * bump_amplitude_loss(bump)
         opt.zero_grad()
         total.backward()
         torch.nn.utils.clip_grad_norm_(model.parameters(), 1.0)
@@ -40,5 +46,6 @@ if __name__ == "__main__":
     ap = argparse.ArgumentParser(description="Train the ring attractor (no gain networks) on the HIP operator")
     ap.add_argument("--action_dim", type=int, default=16)
     ap.add_argument("--steps", type=int, default=1000)
+    ap.add_argument("--fused_loss", action="store_true", help="loss pair and its gradient by the fused HIP loss head")
     a = ap.parse_args()
-    run_training(action_dim=a.action_dim, training_steps=a.steps)
+    run_training(action_dim=a.action_dim, training_steps=a.steps, fused_loss=a.fused_loss)
