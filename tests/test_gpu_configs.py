@@ -100,6 +100,49 @@ def test_headline_size_properties(gpu_device):
     assert torch.isfinite(full[0]).all()
 
 
+def test_long_sequence_shape_at_full_size(gpu_device):
+    """N=512, B=8192, T=512, tanh at its real size (inputs generated on the device): bitwise repeatable, a 32-row
+    slice run alone reproduces its rows of the full batch bit for bit and agrees with the fp64 oracle, the
+    gradient is linear in grad_output, two half-batch shards add up to the full batch."""
+    from rnn_train_ring_attractor_amd import ring_rnn_cuda_func
+    print("[case] long sequence N=512 B=8192 T=512 tanh (full size)", flush=True)
+    B, T, k, N = 8192, 512, 2, 512
+    # contractive gain: with J1 = 1 random weights sit at the edge of chaos and 512 steps amplify any rounding
+    # difference, in every implementation
+    J0, J1 = -1.0 / N, 0.5
+    gen = torch.Generator(device=gpu_device).manual_seed(3)
+    Wa0 = torch.randn(k, N, N, device=gpu_device, generator=gen) / N ** 0.5
+    Wo0 = torch.randn(N, N, device=gpu_device, generator=gen) / N ** 0.5
+    A = torch.rand(B, T, k, device=gpu_device, generator=gen) * 0.3 * (torch.rand(B, T, 1, device=gpu_device, generator=gen) > 0.2)
+    r0 = torch.rand(B, N, device=gpu_device, generator=gen)
+    r0 = r0 / r0.norm(dim=1, keepdim=True)
+    G = torch.randn(T, B, N, device=gpu_device, generator=gen)
+
+    def run(rows, scale=1.0):
+        Wa, Wo = Wa0.clone().requires_grad_(True), Wo0.clone().requires_grad_(True)
+        h = ring_rnn_cuda_func(A[rows].contiguous(), Wa, J0, J1, Wo, r0[rows].contiguous(), 0.15, "tanh")
+        h.backward((G[:, rows] * scale).contiguous())
+        return h.detach(), Wa.grad, Wo.grad
+
+    full = run(slice(0, B))
+    again = run(slice(0, B))
+    assert all(torch.equal(a, b) for a, b in zip(full, again))
+    assert torch.isfinite(full[0]).all() and torch.isfinite(full[1]).all() and torch.isfinite(full[2]).all()
+    sl = slice(4096, 4128)
+    part = run(sl)
+    assert torch.equal(part[0], full[0][:, sl])
+    c = lambda x: x.cpu().numpy()
+    ref, _ = O.forward_dense(c(A[sl]), c(Wa0), J0, J1, c(Wo0), c(r0[sl]), 0.15, "tanh")
+    assert O.max_rel_err(c(part[0]), ref) <= TRAJ_TOL
+    g = O.backward_dense(c(G[:, sl]), c(A[sl]), c(Wa0), J0, J1, c(Wo0), ref, c(r0[sl]), 0.15, "tanh")
+    assert O.cosine(c(part[2]), g["grad_Wo"]) >= GRAD_COS and O.max_rel_err(c(part[2]), g["grad_Wo"]) <= GRAD_TOL
+    assert O.cosine(c(part[1]), g["grad_Wa"]) >= GRAD_COS and O.max_rel_err(c(part[1]), g["grad_Wa"]) <= GRAD_TOL
+    doubled = run(slice(0, B), 2.0)
+    assert O.max_rel_err(c(doubled[2]), 2.0 * c(full[2])) <= 1e-5 and O.max_rel_err(c(doubled[1]), 2.0 * c(full[1])) <= 1e-5
+    lo, hi = run(slice(0, B // 2)), run(slice(B // 2, B))
+    assert O.max_rel_err(c(lo[1] + hi[1]), c(full[1])) <= 1e-4 and O.max_rel_err(c(lo[2] + hi[2]), c(full[2])) <= 1e-4
+
+
 def test_streaming_and_resident_kernels_agree(gpu_device, monkeypatch):
     """The generic weight-streaming kernels and the weight-resident ones evaluate the same recurrence."""
     from rnn_train_ring_attractor_amd import ring_rnn_cuda_func
