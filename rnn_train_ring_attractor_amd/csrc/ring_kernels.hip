@@ -79,12 +79,14 @@ __device__ __forceinline__ void gates_stage(float* gl, const float* __restrict__
 }
 
 // bit c set <=> channel c has a non-zero gate in some row; every wave computes the same mask
-__device__ __forceinline__ unsigned long long gates_active(const float* gl, int k, int lane) {
+// (over the rt gate tiles that follow each other at gl)
+__device__ __forceinline__ unsigned long long gates_active(const float* gl, int k, int lane, int rt = 1) {
   unsigned long long m = 0;
   for (int c0 = 0; c0 < k; c0 += 4) {
     const int c = c0 + (lane >> 4);
-    const float v = c < k ? gl[(lane & 15) * GATE_KMAX + c] : 0.f;
-    const unsigned long long bal = __ballot(v != 0.f);
+    bool nz = false;
+    for (int i = 0; i < rt; ++i) nz |= c < k && gl[(i * 16 + (lane & 15)) * GATE_KMAX + c] != 0.f;
+    const unsigned long long bal = __ballot(nz);
 #pragma unroll
     for (int j = 0; j < 4; ++j)
       if ((bal >> (16 * j)) & 0xffffull) m |= 1ull << (c0 + j);
@@ -94,26 +96,52 @@ __device__ __forceinline__ unsigned long long gates_active(const float* gl, int 
   return ((unsigned long long)hi << 32) | lo;
 }
 
+// Weight pipeline geometry: a unit is one column tile x KG K chunks; PD register buffers, PD - 1 units in
+// flight ahead of the MFMAs.  With more than one batch tile the units are halved and twice as many are
+// kept in flight: the same bytes on their way, half the A-operand registers per tile.
+template <int NC, int RT>
+struct StreamCfg {
+  using TL = Tile<NC>;
+  static constexpr int KG = (RT > 1 && TL::KG == 8) ? 4 : TL::KG, NKG = TL::KCH / KG;
+  static constexpr int UPM = NKG * NC;                 // units per matrix
+  static constexpr int PDMAX = (RT > 1 && TL::KG == 8) ? 8 : 4;
+  static constexpr int PD = UPM >= PDMAX ? PDMAX : UPM;
+  static_assert(UPM % PD == 0, "static register-buffer indices need whole rounds per matrix");
+};
+
 // With GA, rp holds r_prev[row 4q+e][neuron tile c] and ga_part (k x 4 waves x 16 rows) receives, per action
 // matrix and batch row, this wave's share of  sum_j (X @ W_mm)[row][j] * r_prev[row][j]  (= dL/dA[b,t,mm-1]).
 // gl: this step's staged gates (null: read A from global); active: channels worth multiplying.
-template <int NC, bool GA = false>
+// RT: batch tiles of 16 rows that share every weight fragment a wave fetches (one L2 read feeds RT MFMAs).
+// Tile rt reads the operand buffer xb + rt * SLOTS and the gate tile gl + rt * 16 * GATE_KMAX, and its
+// rows start at b0 + 16 * rt.
+// wf: the caller's weight register buffers.  primed: they already hold the first PD - 1 units of matrix 0
+// (a previous call ran with carry_over, which points the prefetch of the last matrix at matrix 0 again:
+// the weights do not change between steps, so the next step's first units load during this step's epilogue).
+template <int NC, bool GA = false, int RT = 1>
 __device__ __forceinline__ void gated_products(const bf16x8* __restrict__ xb, const bf16x8* __restrict__ Wp,
                                                const float* __restrict__ A, const float* gl, unsigned long long active,
                                                int k, int T, int B, int t, int b0, float J1, int w, int lane,
-                                               f32x4 (&acc)[NC], const float (*rp)[NC] = nullptr,
-                                               float* ga_part = nullptr) {
+                                               f32x4 (&acc)[RT][NC],
+                                               bf16x8 (&wf)[StreamCfg<NC, RT>::PD][StreamCfg<NC, RT>::KG],
+                                               bool primed, bool carry_over, const float (*rp)[NC] = nullptr,
+                                               float* ga_part = nullptr, bool acc_preset = false) {
+  static_assert(!GA || RT == 1, "dL/dA is produced one batch tile at a time");
   using TL = Tile<NC>;
-  constexpr int KG = TL::KG, NKG = TL::NKG;
-  constexpr int UPM = NKG * NC;                 // weight units (one column tile x KG chunks) per matrix
-  constexpr int PD = UPM >= 4 ? 4 : UPM;        // register buffers: PD - 1 units are in flight ahead of the MFMAs
+  using SC = StreamCfg<NC, RT>;
+  constexpr int KG = SC::KG, NKG = SC::NKG, UPM = SC::UPM, PD = SC::PD;
   const int q = lane >> 4, n = lane & 15;
+  if (!acc_preset) {                            // otherwise the caller's values are what the products add to
 #pragma unroll
-  for (int c = 0; c < NC; ++c) acc[c] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+      for (int c = 0; c < NC; ++c) acc[rt][c] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
 
   // The weights of a step stream from L2 as one linear sequence of units, active matrix after active
   // matrix; what bounds the step is how many bytes are in flight, so the prefetch runs PD - 1 units
-  // ahead and straight across matrix boundaries (past the last matrix it re-reads that one, unused).
+  // ahead and straight across matrix boundaries (past the last matrix: into matrix 0 for the next step,
+  // or a re-read of that one, unused).
   // Matrix 0 (Wo) is always active; matrix mm >= 1 is gated by channel mm - 1.
   const bool skipping = gl != nullptr && !GA;   // dL/dA needs every product, also where the gate is zero
   auto next_matrix = [&](int mm) {               // next active matrix after mm, or -1
@@ -121,60 +149,88 @@ __device__ __forceinline__ void gated_products(const bf16x8* __restrict__ xb, co
     const unsigned long long rest = mm >= 64 ? 0ull : (active >> mm);   // channels mm, mm+1, ... <-> matrices mm+1, ...
     return rest ? mm + 1 + (int)__builtin_ctzll(rest) : -1;
   };
+  // A unit's address is a wave-uniform base (scalar registers) plus the lane's 16-byte slot: no vector
+  // registers are spent on addresses.
+  const int ws = __builtin_amdgcn_readfirstlane(w);
+  const unsigned lane_off = (unsigned)lane * 16u;
   auto unit_ptr = [&](int mm, int ul) {
     const int kg = ul / NC, c = ul % NC;
-    return Wp + ((size_t)((mm * 4 + w) * NC + c) * TL::KCH + kg * KG) * 64 + lane;
+    return reinterpret_cast<const char*>(Wp) + ((size_t)((mm * 4 + ws) * NC + c) * TL::KCH + kg * KG) * 1024;
   };
-  bf16x8 wf[PD][KG];
+  auto unit_load = [&](const char* base, int u) {
+    return *reinterpret_cast<const bf16x8*>(base + u * 1024 + lane_off);
+  };
+  if (!primed) {
 #pragma unroll
-  for (int d = 0; d < PD - 1; ++d) {            // PD - 1 < UPM: the first units all belong to matrix 0
-    const bf16x8* src = unit_ptr(0, d);
+    for (int d = 0; d < PD - 1; ++d) {          // PD - 1 < UPM: the first units all belong to matrix 0
+      const char* src = unit_ptr(0, d);
 #pragma unroll
-    for (int u = 0; u < KG; ++u) wf[d][u] = src[(size_t)u * 64];
+      for (int u = 0; u < KG; ++u) wf[d][u] = unit_load(src, u);
+    }
   }
 
   for (int mm = 0; mm >= 0;) {
     const int nxt = next_matrix(mm);
-    const int pre = nxt >= 0 ? nxt : mm;        // matrix the prefetch runs into
-    float coef[4];
+    const int pre = nxt >= 0 ? nxt : (carry_over ? 0 : mm);   // matrix the prefetch runs into
+    float coef[RT][4];
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      if (mm == 0) coef[e] = J1;
-      else if (gl) coef[e] = gl[(4 * q + e) * GATE_KMAX + (mm - 1)];
-      else coef[e] = (b0 + e < B) ? A[((size_t)(b0 + e) * T + t) * k + (mm - 1)] : 0.f;
-    }
-    f32x4 p[NC];
+    for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
-    for (int c = 0; c < NC; ++c) p[c] = f32x4{0.f, 0.f, 0.f, 0.f};
+      for (int e = 0; e < 4; ++e) {
+        const int b = b0 + 16 * rt + e;
+        if (mm == 0) coef[rt][e] = J1;
+        else if (gl) coef[rt][e] = gl[(rt * 16 + 4 * q + e) * GATE_KMAX + (mm - 1)];
+        else coef[rt][e] = (b < B) ? A[((size_t)b * T + t) * k + (mm - 1)] : 0.f;
+      }
+    f32x4 p[RT][NC];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+      for (int c = 0; c < NC; ++c) p[rt][c] = f32x4{0.f, 0.f, 0.f, 0.f};
+    // The A operands do not depend on the matrix.  With one batch tile they are read from LDS once per
+    // step and kept; with more, that would take the registers the weight pipeline needs, so they are read
+    // again for every matrix (xo is opaque to the compiler so that it does not hoist the reads).
+    int xo = q * XG + n;
+    if constexpr (RT > 1) asm volatile("" : "+v"(xo));
 #pragma unroll
     for (int kg = 0; kg < NKG; ++kg) {
-      bf16x8 af[KG];
+      bf16x8 af[RT][KG];
 #pragma unroll
-      for (int u = 0; u < KG; ++u) af[u] = xb[((kg * KG + u) * 4 + q) * XG + n];
+      for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+        for (int u = 0; u < KG; ++u) af[rt][u] = xb[rt * TL::SLOTS + (kg * KG + u) * 4 * XG + xo];
 #pragma unroll
       for (int c = 0; c < NC; ++c) {
         const int ul = kg * NC + c;             // unit within the matrix; UPM % PD == 0 keeps buffer indices static
         {
           const int ahead = ul + PD - 1;
-          const bf16x8* src = ahead < UPM ? unit_ptr(mm, ahead) : unit_ptr(pre, ahead - UPM);
+          const char* src = ahead < UPM ? unit_ptr(mm, ahead) : unit_ptr(pre, ahead - UPM);
 #pragma unroll
-          for (int u = 0; u < KG; ++u) wf[ahead % PD][u] = src[(size_t)u * 64];
+          for (int u = 0; u < KG; ++u) wf[ahead % PD][u] = unit_load(src, u);
         }
+        // Pin the order "loads of unit ul + PD - 1, then MFMAs of unit ul": left to itself the scheduler
+        // sinks the loads towards their use (to save registers) and the prefetch distance is gone.
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int u = 0; u < KG; ++u) p[c] = mfma16(af[u], wf[ul % PD][u], p[c]);
+        for (int u = 0; u < KG; ++u)
+#pragma unroll
+          for (int rt = 0; rt < RT; ++rt) p[rt][c] = mfma16(af[rt][u], wf[ul % PD][u], p[rt][c]);
+        __builtin_amdgcn_sched_barrier(0);
       }
     }
 #pragma unroll
-    for (int c = 0; c < NC; ++c)
+    for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
-      for (int e = 0; e < 4; ++e) acc[c][e] += coef[e] * p[c][e];
+      for (int c = 0; c < NC; ++c)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc[rt][c][e] += coef[rt][e] * p[rt][c][e];
     if constexpr (GA) {
       if (mm > 0) {
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           float d = 0.f;
 #pragma unroll
-          for (int c = 0; c < NC; ++c) d = fmaf(p[c][e], rp[e][c], d);
+          for (int c = 0; c < NC; ++c) d = fmaf(p[0][c][e], rp[e][c], d);
           d = row16_sum(d);
           if (n == 0) ga_part[((mm - 1) * 4 + w) * 16 + 4 * q + e] = d;
         }
@@ -208,64 +264,109 @@ __device__ __forceinline__ void read_rowsum(const float* psum, int q, float (&s)
 }
 
 // ------------------------------------------------------------------------------------------------
-// Forward: one workgroup = 16 batch rows for all T steps.  r lives in fp32 registers; its bf16 copy
-// is exchanged between the four waves through a double-buffered LDS operand buffer (one barrier
-// per step).  Writes bump_history [T,B,N] fp32 and, when training, F'(re) (fp16) and the bf16
-// operand copy of r_prev in tile order.
+// Forward: one workgroup = RT tiles of 16 batch rows for all T steps.  r lives in fp32 registers; its
+// bf16 copy is exchanged between the four waves through a double-buffered LDS operand buffer (one
+// barrier per step).  Writes bump_history [T,B,N] fp32 and, when training, F'(re) (fp16) and the bf16
+// operand copy of r_prev in tile order.  The operand buffers [2][RT][SLOTS] are dynamic shared memory.
 // ------------------------------------------------------------------------------------------------
-template <int NC, int ACT>
+template <int NC, int RT>
+constexpr size_t stream_lds_bytes() { return (size_t)2 * RT * Tile<NC>::SLOTS * sizeof(bf16x8); }
+
+// With more than one batch tile per workgroup the forward keeps its fp32 state in LDS between steps
+// (one read and one write per lane and step) instead of in registers the weight pipeline needs.
+template <int NC, int RT>
+constexpr size_t fwd_state_lds_bytes() { return RT > 1 ? (size_t)RT * 4 * NC * 256 * sizeof(float) : 0; }
+
+template <int NC, int ACT, int RT>
 __global__ __launch_bounds__(256) void ring_fwd_kernel(RingFwdArgs p) {
   using TL = Tile<NC>;
-  __shared__ bf16x8 xbuf[2][TL::SLOTS];
-  __shared__ float psum[2][64];
-  __shared__ float gl[2][16 * GATE_KMAX];
+  extern __shared__ __attribute__((aligned(16))) char stream_lds[];
+  bf16x8* const xbuf = reinterpret_cast<bf16x8*>(stream_lds);   // [2][RT][SLOTS]
+  __shared__ float psum[2][RT][64];
+  __shared__ float gl[2][RT * 16 * GATE_KMAX];
 
   const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, q = lane >> 4, n = lane & 15;
-  const int bt = blockIdx.x;
-  const int b0 = 16 * bt + 4 * q;
+  const int bt0 = blockIdx.x * RT;             // tile rt is batch tile bt0 + rt (past the last one: all rows masked)
+  const int b0 = 16 * bt0 + 4 * q;
   const int i0 = 16 * NC * w + NC * n;
   const int N = p.N, B = p.B, T = p.T;
   const float oma = 1.f - p.alpha;
   const bool staged = p.k <= GATE_KMAX;
+  auto xb = [&](int buf, int rt) { return xbuf + (size_t)(buf * RT + rt) * TL::SLOTS; };
 
-  float r[4][NC];
-  rows_load<NC>(p.r_init, N, B, b0, i0, r);
-  write_operand<NC>(xbuf[0], r, w, q, n);
-  publish_rowsum<NC>(psum[0], r, w, q, n);
-  if (staged) gates_stage(gl[0], p.A, p.k, T, B, 0, bt, tid);
-  if (p.rfrag) {
-    pair_store<NC>(p.rfrag, 0, p.nbt, bt, w, lane, r);
-    pair_zero_tail<NC>(p.rfrag, T, p.nbt, bt, w, lane);
+  constexpr bool LDS_STATE = RT > 1;
+  float* const state = reinterpret_cast<float*>(stream_lds + stream_lds_bytes<NC, RT>());   // [RT][4][NC][256 lanes]
+  float rkeep[4][NC];
+  auto state_get = [&](int rt, float (&v)[4][NC]) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+#pragma unroll
+      for (int c = 0; c < NC; ++c) v[e][c] = LDS_STATE ? state[((rt * 4 + e) * NC + c) * 256 + tid] : rkeep[e][c];
+  };
+  auto state_put = [&](int rt, const float (&v)[4][NC]) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+#pragma unroll
+      for (int c = 0; c < NC; ++c) {
+        if constexpr (LDS_STATE) state[((rt * 4 + e) * NC + c) * 256 + tid] = v[e][c];
+        else rkeep[e][c] = v[e][c];
+      }
+  };
+
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    float r[4][NC];
+    rows_load<NC>(p.r_init, N, B, b0 + 16 * rt, i0, r);
+    state_put(rt, r);
+    write_operand<NC>(xb(0, rt), r, w, q, n);
+    publish_rowsum<NC>(psum[0][rt], r, w, q, n);
+    if (staged) gates_stage(gl[0] + rt * 16 * GATE_KMAX, p.A, p.k, T, B, 0, bt0 + rt, tid);
+    if (p.rfrag && bt0 + rt < p.nbt) {
+      pair_store<NC>(p.rfrag, 0, p.nbt, bt0 + rt, w, lane, r);
+      pair_zero_tail<NC>(p.rfrag, T, p.nbt, bt0 + rt, w, lane);
+    }
   }
   lds_barrier();
 
+  bf16x8 wf[StreamCfg<NC, RT>::PD][StreamCfg<NC, RT>::KG];
   for (int t = 0; t < T; ++t) {
     const int cur = t & 1;
-    f32x4 acc[NC];
-    if (staged && t + 1 < T) gates_stage(gl[cur ^ 1], p.A, p.k, T, B, t + 1, bt, tid);
-    gated_products<NC>(xbuf[cur], (const bf16x8*)p.Wpack, p.A, staged ? gl[cur] : nullptr,
-                       staged ? gates_active(gl[cur], p.k, lane) : ~0ull, p.k, T, B, t, b0, p.J1, w, lane, acc);
-    float s[4];
-    read_rowsum(psum[cur], q, s);
-    float d[4][NC];
+    f32x4 acc[RT][NC];
+    if (staged && t + 1 < T) {
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-#pragma unroll
-      for (int c = 0; c < NC; ++c) {
-        const float x = acc[c][e] + p.J0 * s[e];
-        float F, D;
-        act_fast<ACT>(x, F, D);
-        const bool ok = (b0 + e < B) && (i0 + c < N);
-        r[e][c] = ok ? (oma * r[e][c] + p.alpha * F) : 0.f;
-        d[e][c] = ok ? p.alpha * D : 0.f;   // the saved record is alpha * F'(re)
-      }
+      for (int rt = 0; rt < RT; ++rt) gates_stage(gl[cur ^ 1] + rt * 16 * GATE_KMAX, p.A, p.k, T, B, t + 1, bt0 + rt, tid);
     }
-    rows_store<NC>(p.hist + (size_t)t * B * N, N, B, b0, i0, r);
-    if (p.dfrag) side_store<NC, f16x4, _Float16>(p.dfrag + side_offset<NC>(t, p.nbt, bt, w, lane), d);
-    if (t + 1 < T) {
-      write_operand<NC>(xbuf[cur ^ 1], r, w, q, n);
-      publish_rowsum<NC>(psum[cur ^ 1], r, w, q, n);
-      if (p.rfrag) pair_store<NC>(p.rfrag, t + 1, p.nbt, bt, w, lane, r);
+    gated_products<NC, false, RT>(xb(cur, 0), (const bf16x8*)p.Wpack, p.A, staged ? gl[cur] : nullptr,
+                                  staged ? gates_active(gl[cur], p.k, lane, RT) : ~0ull, p.k, T, B, t, b0, p.J1, w, lane,
+                                  acc, wf, t > 0, t + 1 < T);
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+      const int bq = b0 + 16 * rt;
+      float s[4];
+      read_rowsum(psum[cur][rt], q, s);
+      float r[4][NC], d[4][NC];
+      state_get(rt, r);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+#pragma unroll
+        for (int c = 0; c < NC; ++c) {
+          const float x = acc[rt][c][e] + p.J0 * s[e];
+          float F, D;
+          act_fast<ACT>(x, F, D);
+          const bool ok = (bq + e < B) && (i0 + c < N);
+          r[e][c] = ok ? (oma * r[e][c] + p.alpha * F) : 0.f;
+          d[e][c] = ok ? p.alpha * D : 0.f;   // the saved record is alpha * F'(re)
+        }
+      }
+      const bool live = bt0 + rt < p.nbt;
+      rows_store<NC>(p.hist + (size_t)t * B * N, N, B, bq, i0, r);
+      if (p.dfrag && live) side_store<NC, f16x4, _Float16>(p.dfrag + side_offset<NC>(t, p.nbt, bt0 + rt, w, lane), d);
+      if (t + 1 < T) {
+        state_put(rt, r);
+        write_operand<NC>(xb(cur ^ 1, rt), r, w, q, n);
+        publish_rowsum<NC>(psum[cur ^ 1][rt], r, w, q, n);
+        if (p.rfrag && live) pair_store<NC>(p.rfrag, t + 1, p.nbt, bt0 + rt, w, lane, r);
+      }
     }
     lds_barrier();
   }
@@ -275,46 +376,57 @@ __global__ __launch_bounds__(256) void ring_fwd_kernel(RingFwdArgs p) {
 // Rebuild of the saved activations from the state history (used when the forward's buffer was not
 // kept): one workgroup per (batch tile, step); no recurrence.
 // ------------------------------------------------------------------------------------------------
-template <int NC, int ACT>
+template <int NC, int ACT, int RT>
 __global__ __launch_bounds__(256) void ring_rebuild_saved_kernel(RingFwdArgs p) {
   using TL = Tile<NC>;
-  __shared__ bf16x8 xbuf[TL::SLOTS];
-  __shared__ float psum[64];
-  __shared__ float gl[16 * GATE_KMAX];
+  __shared__ bf16x8 xbuf[RT * TL::SLOTS];
+  __shared__ float psum[RT][64];
+  __shared__ float gl[RT * 16 * GATE_KMAX];
 
   const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, q = lane >> 4, n = lane & 15;
-  const int bt = blockIdx.x, t = blockIdx.y;
-  const int b0 = 16 * bt + 4 * q;
+  const int bt0 = blockIdx.x * RT, t = blockIdx.y;
+  const int b0 = 16 * bt0 + 4 * q;
   const int i0 = 16 * NC * w + NC * n;
   const int N = p.N, B = p.B, T = p.T;
-
-  float r[4][NC];
-  const float* prev = (t == 0) ? p.r_init : p.hist + (size_t)(t - 1) * B * N;
-  rows_load<NC>(prev, N, B, b0, i0, r);
-  write_operand<NC>(xbuf, r, w, q, n);
-  publish_rowsum<NC>(psum, r, w, q, n);
-  pair_store<NC>(p.rfrag, t, p.nbt, bt, w, lane, r);
-  if (t == T - 1) pair_zero_tail<NC>(p.rfrag, T, p.nbt, bt, w, lane);
   const bool staged = p.k <= GATE_KMAX;
-  if (staged) gates_stage(gl, p.A, p.k, T, B, t, bt, tid);
+
+  const float* prev = (t == 0) ? p.r_init : p.hist + (size_t)(t - 1) * B * N;
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    float r[4][NC];
+    rows_load<NC>(prev, N, B, b0 + 16 * rt, i0, r);
+    write_operand<NC>(xbuf + rt * TL::SLOTS, r, w, q, n);
+    publish_rowsum<NC>(psum[rt], r, w, q, n);
+    if (bt0 + rt < p.nbt) {
+      pair_store<NC>(p.rfrag, t, p.nbt, bt0 + rt, w, lane, r);
+      if (t == T - 1) pair_zero_tail<NC>(p.rfrag, T, p.nbt, bt0 + rt, w, lane);
+    }
+    if (staged) gates_stage(gl + rt * 16 * GATE_KMAX, p.A, p.k, T, B, t, bt0 + rt, tid);
+  }
   lds_barrier();
 
-  f32x4 acc[NC];
-  gated_products<NC>(xbuf, (const bf16x8*)p.Wpack, p.A, staged ? gl : nullptr, staged ? gates_active(gl, p.k, lane) : ~0ull,
-                     p.k, T, B, t, b0, p.J1, w, lane, acc);
-  float s[4];
-  read_rowsum(psum, q, s);
-  float d[4][NC];
+  f32x4 acc[RT][NC];
+  bf16x8 wf[StreamCfg<NC, RT>::PD][StreamCfg<NC, RT>::KG];
+  gated_products<NC, false, RT>(xbuf, (const bf16x8*)p.Wpack, p.A, staged ? gl : nullptr,
+                                staged ? gates_active(gl, p.k, lane, RT) : ~0ull, p.k, T, B, t, b0, p.J1, w, lane, acc,
+                                wf, false, false);
 #pragma unroll
-  for (int e = 0; e < 4; ++e) {
+  for (int rt = 0; rt < RT; ++rt) {
+    if (bt0 + rt >= p.nbt) continue;
+    float s[4];
+    read_rowsum(psum[rt], q, s);
+    float d[4][NC];
 #pragma unroll
-    for (int c = 0; c < NC; ++c) {
-      float F, D;
-      act_fast<ACT>(acc[c][e] + p.J0 * s[e], F, D);
-      d[e][c] = ((b0 + e < B) && (i0 + c < N)) ? p.alpha * D : 0.f;
+    for (int e = 0; e < 4; ++e) {
+#pragma unroll
+      for (int c = 0; c < NC; ++c) {
+        float F, D;
+        act_fast<ACT>(acc[rt][c][e] + p.J0 * s[e], F, D);
+        d[e][c] = ((b0 + 16 * rt + e < B) && (i0 + c < N)) ? p.alpha * D : 0.f;
+      }
     }
+    side_store<NC, f16x4, _Float16>(p.dfrag + side_offset<NC>(t, p.nbt, bt0 + rt, w, lane), d);
   }
-  side_store<NC, f16x4, _Float16>(p.dfrag + side_offset<NC>(t, p.nbt, bt, w, lane), d);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -332,79 +444,108 @@ __device__ __forceinline__ void bptt_flush_grad_A(const RingBpttArgs& p, const f
   }
 }
 
-// GA: also produce grad_A[b,t,c] = sum_j (g Wa[c])[j] * r_prev[j].  The per-wave shares of a step go to
-// a double-buffered LDS array (dynamic shared memory, 2*k*64 floats) and are summed in wave order and
-// written out after the next step's barrier.
-template <int NC, bool GA>
+// GA: also produce grad_A[b,t,c] = sum_j (g Wa[c])[j] * r_prev[j] (one batch tile per workgroup).  The
+// per-wave shares of a step go to a double-buffered LDS array (2*k*64 floats behind the operand buffers
+// in dynamic shared memory) and are summed in wave order and written out after the next step's barrier.
+template <int NC, bool GA, int RT>
 __global__ __launch_bounds__(256) void ring_bptt_kernel(RingBpttArgs p) {
+  static_assert(!GA || RT == 1, "dL/dA is produced one batch tile at a time");
   using TL = Tile<NC>;
-  __shared__ bf16x8 xbuf[2][TL::SLOTS];
-  __shared__ float psum[2][64];
-  __shared__ float gl[2][16 * GATE_KMAX];
-  extern __shared__ float ga_buf[];   // [2][k][4 waves][16 rows] when GA
+  extern __shared__ __attribute__((aligned(16))) char stream_lds[];
+  bf16x8* const xbuf = reinterpret_cast<bf16x8*>(stream_lds);                              // [2][RT][SLOTS]
+  float* const ga_buf = reinterpret_cast<float*>(stream_lds + stream_lds_bytes<NC, RT>());  // [2][k][4 waves][16 rows] when GA
+  __shared__ float psum[2][RT][64];
+  __shared__ float gl[2][RT * 16 * GATE_KMAX];
 
   const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, q = lane >> 4, n = lane & 15;
-  const int bt = blockIdx.x;
-  const int b0 = 16 * bt + 4 * q;
+  const int bt0 = blockIdx.x * RT;
+  const int b0 = 16 * bt0 + 4 * q;
   const int i0 = 16 * NC * w + NC * n;
   const int N = p.N, B = p.B, T = p.T;
   const float oma = 1.f - p.alpha;
+  auto xb = [&](int buf, int rt) { return xbuf + (size_t)(buf * RT + rt) * TL::SLOTS; };
 
   const bool staged = p.k <= GATE_KMAX;
-  float carry[4][NC];
+  float carry[RT][4][NC];
 #pragma unroll
-  for (int e = 0; e < 4; ++e)
+  for (int rt = 0; rt < RT; ++rt) {
 #pragma unroll
-    for (int c = 0; c < NC; ++c) carry[e][c] = 0.f;
-  pair_zero_tail<NC>(p.gfrag, T, p.nbt, bt, w, lane);
+    for (int e = 0; e < 4; ++e)
+#pragma unroll
+      for (int c = 0; c < NC; ++c) carry[rt][e][c] = 0.f;
+    if (bt0 + rt < p.nbt) pair_zero_tail<NC>(p.gfrag, T, p.nbt, bt0 + rt, w, lane);
+  }
 
+  // The weight pipeline restarts every step here: a step begins by waiting for grad_output and the saved
+  // record from HBM, which hides the refill, and carrying the buffers over would cost registers.
+  bf16x8 wf[StreamCfg<NC, RT>::PD][StreamCfg<NC, RT>::KG];
   for (int t = T - 1; t >= 0; --t) {
     const int cur = (T - 1 - t) & 1;
-    float G[4][NC], g[4][NC];
-    rows_load<NC>(p.grad_out + (size_t)t * B * N, N, B, b0, i0, G);
-    side_load_f16<NC>(p.dfrag + side_offset<NC>(t, p.nbt, bt, w, lane), g);
+    // The accumulators start at (1-alpha) G, so that G itself is dead before the products begin.
+    f32x4 acc[RT][NC];
 #pragma unroll
-    for (int e = 0; e < 4; ++e)
+    for (int rt = 0; rt < RT; ++rt) {
+      const bool live = bt0 + rt < p.nbt;
+      float G[4][NC], g[4][NC];
+      rows_load<NC>(p.grad_out + (size_t)t * B * N, N, B, b0 + 16 * rt, i0, G);
+      if (live) {
+        side_load_f16<NC>(p.dfrag + side_offset<NC>(t, p.nbt, bt0 + rt, w, lane), g);
+      } else {
 #pragma unroll
-      for (int c = 0; c < NC; ++c) {
-        G[e][c] += carry[e][c];
-        g[e][c] = g[e][c] * G[e][c];   // the saved record already carries alpha
+        for (int e = 0; e < 4; ++e)
+#pragma unroll
+          for (int c = 0; c < NC; ++c) g[e][c] = 0.f;
       }
-    write_operand<NC>(xbuf[cur], g, w, q, n);
-    publish_rowsum<NC>(psum[cur], g, w, q, n);
-    pair_store<NC>(p.gfrag, t, p.nbt, bt, w, lane, g);
-    // this step's gates: the buffer was last read two steps ago, before the previous barrier
-    if (staged) gates_stage(gl[cur], p.A, p.k, T, B, t, bt, tid);
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+#pragma unroll
+        for (int c = 0; c < NC; ++c) {
+          G[e][c] += carry[rt][e][c];
+          g[e][c] = g[e][c] * G[e][c];   // the saved record already carries alpha
+          acc[rt][c][e] = oma * G[e][c];
+        }
+      write_operand<NC>(xb(cur, rt), g, w, q, n);
+      publish_rowsum<NC>(psum[cur][rt], g, w, q, n);
+      if (live) pair_store<NC>(p.gfrag, t, p.nbt, bt0 + rt, w, lane, g);
+      // this step's gates: the buffer was last read two steps ago, before the previous barrier
+      if (staged) gates_stage(gl[cur] + rt * 16 * GATE_KMAX, p.A, p.k, T, B, t, bt0 + rt, tid);
+    }
     lds_barrier();
     const float* glt = staged ? gl[cur] : nullptr;
-    const unsigned long long active = staged ? gates_active(gl[cur], p.k, lane) : ~0ull;
+    const unsigned long long active = staged ? gates_active(gl[cur], p.k, lane, RT) : ~0ull;
 
-    f32x4 acc[NC];
     if constexpr (GA) {
       // the shares of step t+1 are complete (every wave passed the barrier above after writing them)
-      if (t + 1 < T) bptt_flush_grad_A(p, ga_buf + (cur ^ 1) * p.k * 64, t + 1, bt, tid);
+      if (t + 1 < T) bptt_flush_grad_A(p, ga_buf + (cur ^ 1) * p.k * 64, t + 1, bt0, tid);
       float rp[4][NC];
       rows_load<NC>(t == 0 ? p.r_init : p.hist + (size_t)(t - 1) * B * N, N, B, b0, i0, rp);
-      gated_products<NC, true>(xbuf[cur], (const bf16x8*)p.Wpack, p.A, glt, active, p.k, T, B, t, b0, p.J1, w, lane,
-                               acc, rp, ga_buf + cur * p.k * 64);
+      gated_products<NC, true, 1>(xb(cur, 0), (const bf16x8*)p.Wpack, p.A, glt, active, p.k, T, B, t, b0, p.J1, w, lane,
+                                  acc, wf, false, false, rp, ga_buf + cur * p.k * 64, true);
     } else {
-      gated_products<NC>(xbuf[cur], (const bf16x8*)p.Wpack, p.A, glt, active, p.k, T, B, t, b0, p.J1, w, lane, acc);
+      gated_products<NC, false, RT>(xb(cur, 0), (const bf16x8*)p.Wpack, p.A, glt, active, p.k, T, B, t, b0, p.J1, w,
+                                    lane, acc, wf, false, false, nullptr, nullptr, true);
     }
-    float s[4];
-    read_rowsum(psum[cur], q, s);
 #pragma unroll
-    for (int e = 0; e < 4; ++e)
+    for (int rt = 0; rt < RT; ++rt) {
+      float s[4];
+      read_rowsum(psum[cur][rt], q, s);
 #pragma unroll
-      for (int c = 0; c < NC; ++c) {
-        const bool ok = (b0 + e < B) && (i0 + c < N);
-        carry[e][c] = ok ? (oma * G[e][c] + p.J0 * s[e] + acc[c][e]) : 0.f;
-      }
+      for (int e = 0; e < 4; ++e)
+#pragma unroll
+        for (int c = 0; c < NC; ++c) {
+          const bool ok = (b0 + 16 * rt + e < B) && (i0 + c < N);
+          carry[rt][e][c] = ok ? (acc[rt][c][e] + p.J0 * s[e]) : 0.f;
+        }
+    }
   }
   if constexpr (GA) {
     lds_barrier();
-    bptt_flush_grad_A(p, ga_buf + ((T - 1) & 1) * p.k * 64, 0, bt, tid);
+    bptt_flush_grad_A(p, ga_buf + ((T - 1) & 1) * p.k * 64, 0, bt0, tid);
   }
-  if (p.grad_r_init) rows_store<NC>(p.grad_r_init, N, B, b0, i0, carry);
+  if (p.grad_r_init) {
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) rows_store<NC>(p.grad_r_init, N, B, b0 + 16 * rt, i0, carry[rt]);
+  }
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -650,11 +791,49 @@ bool ring_uses_resident(int N, int k) {
   return !(v && v[0] == '1');
 }
 
+// Batch tiles per workgroup of the streaming kernels.  A step of these kernels is bound by the weight
+// bytes a compute unit can pull from L2, and two tiles share every fetched fragment; pairing pays when
+// the workgroups would otherwise run in more rounds than the paired ones (more tiles than compute units).
+// RINGATTR_ROW_TILES=1|2 overrides the choice (tests cross-check the two forms).
+static int stream_row_tiles(int NCv, int nbt, bool one_workgroup_per_step) {
+  if (NCv < 4 || nbt < 2) return 1;
+  const char* v = getenv("RINGATTR_ROW_TILES");
+  if (v && (v[0] == '1' || v[0] == '2')) return v[0] - '0';
+  if (one_workgroup_per_step) return NCv >= 8 ? 2 : 1;   // a grid of tiles x steps fills the device; pairing pays at the widest tiling
+  static int cus = 0;
+  if (cus == 0) {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    cus = n;
+  }
+  const long rounds1 = (nbt + cus - 1) / cus, rounds2 = ((nbt + 1) / 2 + cus - 1) / cus;
+  return 4 * rounds2 < 3 * rounds1 ? 2 : 1;    // a paired step takes about 1.4 times a single one
+}
+
+template <typename K, typename Args>
+static hipError_t launch_stream(K kern, dim3 grid, size_t dyn, hipStream_t st, const Args& a) {
+  if (dyn > 48 * 1024) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)dyn);
+    if (e != hipSuccess) return e;
+  }
+  hipLaunchKernelGGL(kern, grid, dim3(256), dyn, st, a);
+  return hipGetLastError();
+}
+
+#define RING_DISPATCH_RT(RTv, CALL)                                         \
+  if ((RTv) == 2) { constexpr int RT = 2; if constexpr (NC >= 4) { CALL; } } \
+  else { constexpr int RT = 1; CALL; }
+
 hipError_t ring_launch_fwd(const RingFwdArgs& a, int NCv, hipStream_t st) {
   ProfScope prof(1, st);
   if (ring_uses_resident(a.N, a.k)) return ring_launch_fwd_res256(a, st);
-  RING_DISPATCH_NC(NCv, RING_DISPATCH_ACT(a.act, hipLaunchKernelGGL((ring_fwd_kernel<NC, ACT>), dim3(a.nbt), dim3(256), 0, st, a)));
-  return hipGetLastError();
+  const int rt = stream_row_tiles(NCv, a.nbt, false);
+  hipError_t e = hipErrorInvalidValue;
+  RING_DISPATCH_NC(NCv, RING_DISPATCH_ACT(a.act, RING_DISPATCH_RT(rt,
+      e = launch_stream(ring_fwd_kernel<NC, ACT, RT>, dim3((a.nbt + RT - 1) / RT),
+                        stream_lds_bytes<NC, RT>() + fwd_state_lds_bytes<NC, RT>(), st, a))));
+  return e;
 }
 
 // For the weight-resident geometry the saved record is rebuilt by running the forward recurrence again
@@ -667,20 +846,26 @@ hipError_t ring_launch_rebuild(const RingFwdArgs& a, int NCv, hipStream_t st) {
     f.hist = nullptr;
     return ring_launch_fwd_res256(f, st);
   }
-  RING_DISPATCH_NC(NCv, RING_DISPATCH_ACT(a.act, hipLaunchKernelGGL((ring_rebuild_saved_kernel<NC, ACT>), dim3(a.nbt, a.T), dim3(256), 0, st, a)));
-  return hipGetLastError();
+  const int rt = stream_row_tiles(NCv, a.nbt, true);
+  hipError_t e = hipErrorInvalidValue;
+  RING_DISPATCH_NC(NCv, RING_DISPATCH_ACT(a.act, RING_DISPATCH_RT(rt,
+      e = launch_stream(ring_rebuild_saved_kernel<NC, ACT, RT>, dim3((a.nbt + RT - 1) / RT, a.T), 0, st, a))));
+  return e;
 }
 
 hipError_t ring_launch_bptt(const RingBpttArgs& a, int NCv, hipStream_t st) {
   ProfScope prof(3, st);
+  hipError_t e = hipErrorInvalidValue;
   if (a.grad_A) {   // the generic kernel is the one that also produces dL/dA
-    const size_t dyn = (size_t)2 * a.k * 64 * sizeof(float);
-    RING_DISPATCH_NC(NCv, hipLaunchKernelGGL((ring_bptt_kernel<NC, true>), dim3(a.nbt), dim3(256), dyn, st, a));
-    return hipGetLastError();
+    RING_DISPATCH_NC(NCv, e = launch_stream(ring_bptt_kernel<NC, true, 1>, dim3(a.nbt),
+                                            stream_lds_bytes<NC, 1>() + (size_t)2 * a.k * 64 * sizeof(float), st, a));
+    return e;
   }
   if (ring_uses_resident(a.N, a.k)) return ring_launch_bptt_res256(a, st);
-  RING_DISPATCH_NC(NCv, hipLaunchKernelGGL((ring_bptt_kernel<NC, false>), dim3(a.nbt), dim3(256), 0, st, a));
-  return hipGetLastError();
+  const int rt = stream_row_tiles(NCv, a.nbt, false);
+  RING_DISPATCH_NC(NCv, RING_DISPATCH_RT(rt,
+      e = launch_stream(ring_bptt_kernel<NC, false, RT>, dim3((a.nbt + RT - 1) / RT), stream_lds_bytes<NC, RT>(), st, a)));
+  return e;
 }
 
 hipError_t ring_launch_dw(const RingDwArgs& a, int NCv, hipStream_t st) {

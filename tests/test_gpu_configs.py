@@ -163,6 +163,46 @@ def test_streaming_and_resident_kernels_agree(gpu_device, monkeypatch):
     assert O.max_rel_err(outs["0"][2], model["grad_Wo"]) <= 5e-3
 
 
+@pytest.mark.parametrize("B,T,k,N,act,saved", [
+    (40, 9, 2, 512, "tanh", True),      # three batch tiles: the second workgroup's partner tile does not exist
+    (33, 5, 3, 300, "gelu", True),      # ragged rows and neurons
+    (48, 6, 4, 256, "silu", True),      # a_dim > 2 at N <= 256: the four-column-tile geometry
+    (40, 7, 2, 512, "tanh", False),     # backward rebuilds the saved record (paired there as well)
+])
+def test_paired_batch_tiles_equal_single_tiles(B, T, k, N, act, saved, gpu_device, monkeypatch):
+    """The streaming kernels may give a workgroup two batch tiles that share every weight fragment it
+    fetches.  Per element the arithmetic is that of the one-tile kernels up to how the compiler contracts the
+    fp32 epilogue into fused multiply-adds, so history and gradients agree to fp32 rounding; the paired run
+    is also held to the oracle."""
+    from rnn_train_ring_attractor_amd import rnn_cuda
+    print(f"[case] paired tiles B={B} T={T} k={k} N={N} {act} saved={saved}", flush=True)
+    p = make_problem(77 + N + k, B, T, k, N)
+    acts = {"relu": 0, "gelu": 1, "tanh": 2, "silu": 3}
+    outs = {}
+    for mode in ("1", "2"):
+        monkeypatch.setenv("RINGATTR_ROW_TILES", mode)
+        A, Wa, Wo, r0, G = (_t(p[x], gpu_device) for x in ("A", "Wa", "Wo", "r0", "G"))
+        hist = torch.empty(T, B, N, device=gpu_device)
+        sv = torch.empty(rnn_cuda.saved_nbytes(N, k, T, B), dtype=torch.uint8, device=gpu_device) if saved else None
+        rnn_cuda.fwd_cuda.fwd(A=A, Wa=Wa, J0=-0.1, J1=0.3, Wo=Wo, r_init=r0, bump_history=hist, alpha=0.15,
+                              activation_type=acts[act], saved=sv)
+        gWa, gWo = torch.zeros_like(Wa), torch.zeros_like(Wo)
+        gr0 = torch.empty_like(r0)
+        rnn_cuda.bwd_cuda.bwd(grad_output=G, A=A, Wa=Wa, J0=-0.1, J1=0.3, Wo=Wo, bump_history=hist, r_init=r0,
+                              grad_Wa=gWa, grad_Wo=gWo, alpha=0.15, activation_type=acts[act],
+                              saved=sv, grad_r_init=gr0)
+        torch.cuda.synchronize()
+        outs[mode] = [x.cpu().numpy() for x in (hist, gWa, gWo, gr0)]
+    # a last-bit difference in fp32 can flip the bf16 rounding of an operand copy, which the gradients see
+    for (a, b), tol in zip(zip(outs["1"], outs["2"]), (1e-4, 2e-3, 2e-3, 2e-3)):
+        assert O.max_rel_err(a, b) <= tol
+    ref_hist, _ = O.forward_dense(p["A"], p["Wa"], -0.1, 0.3, p["Wo"], p["r0"], 0.15, act)
+    assert O.max_rel_err(outs["2"][0], ref_hist) <= TRAJ_TOL
+    ref = O.backward_dense(p["G"], p["A"], p["Wa"], -0.1, 0.3, p["Wo"], ref_hist, p["r0"], 0.15, act)
+    assert O.cosine(outs["2"][2], ref["grad_Wo"]) >= 0.999 and O.cosine(outs["2"][1], ref["grad_Wa"]) >= 0.999
+    assert O.cosine(outs["2"][3], ref["grad_r_init"]) >= 0.999
+
+
 @pytest.mark.parametrize("T", [1, 2, 3, 32, 33, 64, 65])
 def test_sequence_length_edges_of_the_resident_kernels(T, gpu_device):
     """Sequence lengths around the kernels' internal boundaries (first/last step peeling, paired time steps,
