@@ -11,9 +11,10 @@
 //   * the action gates of a chunk (16 rows x 2 steps x up to 3 matrices) are fetched one value per
 //     thread and handed round through a small LDS stage next to the r_prev one: per-lane gate loads
 //     (eight scattered 4-byte loads per wave and chunk) cost more than the whole gating arithmetic;
-//   * the eight r_prev fragments every wave needs are copied verbatim into a double-buffered LDS
-//     stage once per workgroup (8 KiB per chunk) and read back with conflict-free ds_read_b128 --
-//     L2 -> CU traffic stays at 16 KiB per chunk and the LDS pipe at 40 KiB, both under the MFMA time.
+//   * the eight r_prev fragments every wave needs are copied verbatim into an LDS stage of DW_LDS
+//     buffers once per workgroup (8 KiB per chunk) and read back with conflict-free ds_read_b128, one
+//     chunk ahead of the MFMAs that use them -- L2 -> CU traffic stays at 16 KiB per chunk and the LDS
+//     pipe at 40 KiB, both under the MFMA time.
 // DW_DEPTH chunks are in flight in registers; a trip of the main loop is one basic block containing
 // loads only, so the compiler waits for exactly the oldest chunk (s_waitcnt vmcnt(n), n > 0).
 // Partials are written once per wave; a fixed-order reduction follows.
@@ -25,6 +26,7 @@ namespace {
 constexpr int DW_WI = 2;      // MFMA row tiles per wave (32 neurons of g)
 constexpr int DW_WJ = 8;      // MFMA column tiles per wave (128 neurons of r_prev)
 constexpr int DW_DEPTH = 4;   // K chunks in flight per wave
+constexpr int DW_LDS = 4;     // LDS stage buffers (chunk c lives in buffer c % DW_LDS)
 
 template <int NG>
 struct DwStage {
@@ -76,8 +78,8 @@ __global__ __launch_bounds__(256) void ring_dw_direct_kernel(RingDwArgs p, int m
   constexpr int NT = 4 * NC;
   constexpr int NB = NT / 8;             // 128-neuron blocks per side
   constexpr int NG = NMAT - (FIRST ? 1 : 0);
-  __shared__ __attribute__((aligned(16))) f32x4 lds_b[2][DW_WJ * 64];
-  __shared__ __attribute__((aligned(16))) float lds_g[2][4][16][2];   // [buffer][gated matrix][row][step]
+  __shared__ __attribute__((aligned(16))) f32x4 lds_b[DW_LDS][DW_WJ * 64];
+  __shared__ __attribute__((aligned(16))) float lds_g[DW_LDS][4][16][2];   // [buffer][gated matrix][row][step]
   const int tid = threadIdx.x, wv = tid >> 6, lane = tid & 63;
   const int tiles = NB * NB;
   // keep the workgroups that share a K split on one XCD (workgroup ids are dealt round-robin to
@@ -131,24 +133,31 @@ __global__ __launch_bounds__(256) void ring_dw_direct_kernel(RingDwArgs p, int m
     fb = wrap ? 0 : fb;
     ft += wrap;
   };
-  auto compute = [&](const DwStage<NG>& s, int cur) {
+  // The LDS stage has DW_LDS buffers and is read one chunk ahead of the MFMAs that use it: the reads of
+  // chunk i+1 are issued before the MFMAs of chunk i and land while those run.  A chunk is therefore
+  // published two chunks before it is used, with a barrier between the publication and the read.
+  struct DwOperands {
     bf16x8 b[DW_WJ];
-#pragma unroll
-    for (int u = 0; u < DW_WJ; ++u) b[u] = *reinterpret_cast<const bf16x8*>(&lds_b[cur][u * 64 + lane]);
     f32x4 g8[NG > 0 ? NG : 1][2];
+  };
+  auto lds_read = [&](DwOperands& o, int buf) {
+#pragma unroll
+    for (int u = 0; u < DW_WJ; ++u) o.b[u] = *reinterpret_cast<const bf16x8*>(&lds_b[buf][u * 64 + lane]);
 #pragma unroll
     for (int a = 0; a < NG; ++a) {
-      const f32x4* gp = reinterpret_cast<const f32x4*>(&lds_g[cur][a][4 * (lane >> 4)][0]);
-      g8[a][0] = gp[0];
-      g8[a][1] = gp[1];
+      const f32x4* gp = reinterpret_cast<const f32x4*>(&lds_g[buf][a][4 * (lane >> 4)][0]);
+      o.g8[a][0] = gp[0];
+      o.g8[a][1] = gp[1];
     }
+  };
+  auto compute = [&](const DwStage<NG>& s, const DwOperands& o) {
 #pragma unroll
     for (int a = 0; a < NMAT; ++a) {
 #pragma unroll
       for (int ii = 0; ii < DW_WI; ++ii) {
-        const bf16x8 gg = (FIRST && a == 0) ? s.a[ii] : gate_frag(s.a[ii], g8[a - (FIRST ? 1 : 0)]);
+        const bf16x8 gg = (FIRST && a == 0) ? s.a[ii] : gate_frag(s.a[ii], o.g8[a - (FIRST ? 1 : 0)]);
 #pragma unroll
-        for (int u = 0; u < DW_WJ; ++u) acc[a][ii][u] = mfma16(gg, b[u], acc[a][ii][u]);
+        for (int u = 0; u < DW_WJ; ++u) acc[a][ii][u] = mfma16(gg, o.b[u], acc[a][ii][u]);
       }
     }
   };
@@ -159,30 +168,39 @@ __global__ __launch_bounds__(256) void ring_dw_direct_kernel(RingDwArgs p, int m
   };
 
   if (ch0 < ch1) {
+    static_assert(DW_DEPTH == DW_LDS, "stage d of the register pipeline and LDS buffer d hold the same chunk");
     DwStage<NG> st[DW_DEPTH];
+    DwOperands op[2];
 #pragma unroll
     for (int d = 0; d < DW_DEPTH; ++d) fetch_next(st[d]);
     publish(st[0], 0);
+    publish(st[1], 1);
     lds_barrier();
+    lds_read(op[0], 0);
+    // Invariant at the top of step d (chunk base + d): op[d & 1] holds (or is about to receive) that chunk's
+    // operands, buffer d + 1 holds the next chunk behind a barrier, stage d + 2 is the next to publish.
     int base = ch0;
     for (; base + DW_DEPTH <= ch1; base += DW_DEPTH) {
 #pragma unroll
       for (int d = 0; d < DW_DEPTH; ++d) {
-        compute(st[d], d & 1);                      // DW_DEPTH is even: chunk parity == d parity
+        lds_read(op[(d + 1) & 1], (d + 1) % DW_LDS);
+        __builtin_amdgcn_sched_barrier(0);          // issue the reads first: left alone they sink below the MFMAs
+        compute(st[d], op[d & 1]);
         fetch_next(st[d]);                          // refill DW_DEPTH chunks ahead
-        publish(st[(d + 1) % DW_DEPTH], (d & 1) ^ 1);
+        publish(st[(d + 2) % DW_DEPTH], (d + 2) % DW_LDS);
         lds_barrier();
         // keep the refill of stage d where it is: the scheduler would otherwise sink all refills of
         // a trip to its end and drain the whole queue once per trip
         __builtin_amdgcn_sched_barrier(0);
       }
     }
-    // tail (< DW_DEPTH chunks): stage d holds chunk base+d, LDS buffer 0 holds the r_prev of `base`
+    // tail (< DW_DEPTH chunks): stage d holds chunk base + d (past the split's end: copies of its last chunk)
 #pragma unroll
     for (int d = 0; d < DW_DEPTH - 1; ++d) {
       if (base + d >= ch1) break;
-      compute(st[d], d & 1);
-      publish(st[d + 1], (d & 1) ^ 1);
+      lds_read(op[(d + 1) & 1], (d + 1) % DW_LDS);
+      compute(st[d], op[d & 1]);
+      publish(st[(d + 2) % DW_DEPTH], (d + 2) % DW_LDS);
       lds_barrier();
     }
   }
