@@ -45,6 +45,8 @@ CASES = [
     ("n64_lr",         32,   9,  2,  64, "tanh", -0.1, 0.1, "lr"),        # zero gates at the start: matrices skipped
     ("n48_dense",      16,   3,  2,  48, "tanh", -0.1, 0.1, "dense"),
     ("n512_k16_pad",   32,   6, 16, 512, "gelu", -0.1, 0.1, "lr"),        # zero-padded channels, widest tiling
+    ("k70_wide_action", 20,  4, 70,  96, "tanh", -0.1, 0.1, "dense"),     # more channels than the LDS gate stage holds
+    ("n300_k5_spread", 48,   5,  5, 300, "silu", -0.05, 0.2, "spread"),   # widest tiling, several matrix groups
 ]
 
 
