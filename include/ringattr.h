@@ -109,6 +109,24 @@ RINGATTR_API int ringattr_loss_bwd(const void* bump_history, const void* target_
                       float bump_weight, const void* upstream, void* grad_history, int N, int seq_len,
                       int batch_size, const void* workspace, size_t workspace_bytes, void* stream);
 
+/* ringattr_bwd with the loss head's gradient in place of grad_output: the backward of
+ *   total = loss_pair(bump_history),  bump_history = forward(...)
+ * in one call.  No counterpart in the reference (its training script lets autograd chain the torch loss ops into
+ * RingRnnCudaFunc.backward, cpp/ring_rnn_cuda.py:81-144).  loss_workspace is the workspace ringattr_loss_fwd
+ * filled for this bump_history; upstream is one device float (d objective / d total) or NULL for 1; every other
+ * argument is ringattr_bwd's.  For the weight-resident geometry (a_dim == 2, 128 < N <= 256, no grad_A) the BPTT
+ * kernel forms grad_output in registers from bump_history and the loss head's per-row coefficients, and the
+ * [T,B,N] gradient never goes through HBM; otherwise the library writes it into its workspace and reads it back
+ * (what ringattr_loss_bwd followed by ringattr_bwd would do; the workspace query below then includes that buffer). */
+RINGATTR_API size_t ringattr_bwd_loss_workspace_bytes(int N, int a_dim, int seq_len, int batch_size, int have_saved,
+                      int want_grad_A);
+RINGATTR_API int ringattr_bwd_loss(const void* loss_workspace, const void* upstream, const void* A, const void* Wa,
+                      float J0, float J1, const void* Wo, const void* bump_history, const void* r_init,
+                      void* grad_Wa, void* grad_Wo, float alpha,
+                      int N, int a_dim, int seq_len, int batch_size, int activation_type,
+                      const void* saved, void* grad_A, void* grad_r_init,
+                      void* workspace, size_t workspace_bytes, void* stream);
+
 /* Per-kernel timing for benchmarks; no counterpart in the reference.  While enabled, every kernel
  * launch is bracketed by two HIP events recorded on the launch stream.  ringattr_profile_read waits
  * for the recorded events, adds their durations into ms[RINGATTR_NUM_KERNELS] and the launch counts

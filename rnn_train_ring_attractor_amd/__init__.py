@@ -5,6 +5,7 @@ _EXPORTS = {
     "ring_rnn_cuda_func": "ring_rnn_cuda", "RingRnnCudaFunc": "ring_rnn_cuda",
     "fwd_cuda": "rnn_cuda", "bwd_cuda": "rnn_cuda",
     "ring_loss_pair": "loss_head", "RingLossPair": "loss_head",
+    "ring_rnn_loss_func": "loss_head", "RingRnnLossFunc": "loss_head",
 }
 
 

@@ -26,6 +26,11 @@ struct RingBpttArgs {
   float* grad_A;         // [B,T,k] or null (written, not accumulated); needs hist and r_init
   const float* hist;     // [T,B,N] state history (r_prev of step t is hist[t-1]); only read for grad_A
   const float* r_init;   // [B,N]
+  // Loss head fused into the weight-resident BPTT kernel (null: grad_out is read).  loss_coef[t*B + b] holds the
+  // row's (kc, ks, beta, -) as ring_loss_stats/rows/decode left them; the kernel then reads hist, not grad_out.
+  const ring_f32x4* loss_coef;
+  const float* loss_upstream;   // one float on the device, or null for 1
+  float loss_inv_rows;          // 1 / (T * B)
   float J0, J1, alpha;
   int N, k, T, B, nbt;
 };
@@ -70,6 +75,8 @@ hipError_t ring_launch_loss_fwd(const float* hist, const float* angle, const flo
 hipError_t ring_launch_loss_bwd(const float* hist, const float* angle, const float* target_amp, float bump_weight,
                                 const float* upstream, float* grad_hist, int N, int T, int B, const void* workspace,
                                 hipStream_t st);
+// the per-row coefficients (kc, ks, beta, -) inside a workspace that ring_launch_loss_fwd filled
+const ring_f32x4* ring_loss_row_coefficients(const void* workspace);
 
 // Optional event bracketing of launches (benchmark support).
 void ring_profile_set(bool on);

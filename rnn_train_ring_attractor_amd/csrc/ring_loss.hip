@@ -335,6 +335,10 @@ hipError_t ring_launch_loss_fwd(const float* hist, const float* angle, const flo
   return hipGetLastError();
 }
 
+const ring_f32x4* ring_loss_row_coefficients(const void* workspace) {
+  return reinterpret_cast<const ring_f32x4*>(workspace);   // carve(): the stats array leads the workspace
+}
+
 // The workspace must be the one ring_launch_loss_fwd filled for the same history: it holds the rows' coefficients.
 hipError_t ring_launch_loss_bwd(const float* hist, const float* angle, const float* target_amp, float bump_weight,
                                 const float* upstream, float* grad_hist, int N, int T, int B, const void* workspace,

@@ -333,13 +333,16 @@ __global__ __launch_bounds__(512) void ring_fwd_res256_kernel(RingFwdArgs p) {
 // ------------------------------------------------------------------------------------------------
 namespace {
 
-// One step's inputs in flight: grad_output rows (4 x 16 B) and the saved F' record (2 x 16 B, fp16).
+// One step's inputs in flight: grad_output rows (4 x 16 B) and the saved F' record (2 x 16 B, fp16).  With the
+// loss head fused in (LOSS) the rows are those of the state history instead and C holds the four rows' loss
+// coefficients (kc, ks, beta, -), from which the kernel forms grad_output itself.
 struct BpttStage {
   f32x4 G[4];
   f32x4 D[2];
+  f32x4 C[4];
 };
 
-// In the unmasked variant the six loads of a stage are issued with inline assembly and waited for
+// In the unmasked variant the loads of a stage are issued with inline assembly and waited for
 // with an explicit vmcnt.  The compiler, seeing loads and stores share that counter, would otherwise
 // drain it completely (vmcnt(0)) before every use and expose a full HBM round trip per time step.
 // Safety of bptt_stage_wait<K>: vector-memory operations leave the counter in issue order, so once at
@@ -352,32 +355,53 @@ __device__ __forceinline__ f32x4 async_load16(const void* ptr) {
   return v;
 }
 
-template <int K>
+template <int K, bool LOSS>
 __device__ __forceinline__ void bptt_stage_wait(BpttStage& s) {
-  asm volatile(".Lring_async_wait_%=:\n\ts_waitcnt vmcnt(%6)"
-               : "+v"(s.G[0]), "+v"(s.G[1]), "+v"(s.G[2]), "+v"(s.G[3]), "+v"(s.D[0]), "+v"(s.D[1])
-               : "n"(K)
-               : "memory");
+  if constexpr (LOSS) {
+    asm volatile(".Lring_async_wait_%=:\n\ts_waitcnt vmcnt(%10)"
+                 : "+v"(s.G[0]), "+v"(s.G[1]), "+v"(s.G[2]), "+v"(s.G[3]), "+v"(s.D[0]), "+v"(s.D[1]), "+v"(s.C[0]),
+                   "+v"(s.C[1]), "+v"(s.C[2]), "+v"(s.C[3])
+                 : "n"(K)
+                 : "memory");
+  } else {
+    asm volatile(".Lring_async_wait_%=:\n\ts_waitcnt vmcnt(%6)"
+                 : "+v"(s.G[0]), "+v"(s.G[1]), "+v"(s.G[2]), "+v"(s.G[3]), "+v"(s.D[0]), "+v"(s.D[1])
+                 : "n"(K)
+                 : "memory");
+  }
 }
 
-template <bool FULL>
+template <bool FULL, bool LOSS>
 __device__ __forceinline__ void bptt_stage_load(const RingBpttArgs& p, int t, int bt, int w, int lane, int b0, int i0,
                                                 BpttStage& s) {
   if (t < 0) t = 0;   // redundant reload past the start of the sequence; never consumed
   const _Float16* drec = p.dfrag + side_offset<R_NC>(t, p.nbt, bt, w, lane);
+  const float* rows = LOSS ? p.hist : p.grad_out;
   if constexpr (FULL) {
-    const float* grow = p.grad_out + ((size_t)t * p.B + b0) * p.N + i0;
+    const float* grow = rows + ((size_t)t * p.B + b0) * p.N + i0;
 #pragma unroll
     for (int e = 0; e < 4; ++e) s.G[e] = async_load16(grow + (size_t)e * p.N);
     s.D[0] = async_load16(drec);
     s.D[1] = async_load16(drec + 8);
+    if constexpr (LOSS) {
+      const ring_f32x4* crow = p.loss_coef + (size_t)t * p.B + b0;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) s.C[e] = async_load16(crow + e);
+    }
   } else {
     float G[4][R_NC];
-    rows_load<R_NC>(p.grad_out + (size_t)t * p.B * p.N, p.N, p.B, b0, i0, G);
+    rows_load<R_NC>(rows + (size_t)t * p.B * p.N, p.N, p.B, b0, i0, G);
 #pragma unroll
     for (int e = 0; e < 4; ++e) s.G[e] = f32x4{G[e][0], G[e][1], G[e][2], G[e][3]};
     s.D[0] = *reinterpret_cast<const f32x4*>(drec);
     s.D[1] = *reinterpret_cast<const f32x4*>(drec + 8);
+    if constexpr (LOSS) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int b = b0 + e < p.B ? b0 + e : p.B - 1;   // rows past the batch meet a zero F' record
+        s.C[e] = p.loss_coef[(size_t)t * p.B + b];
+      }
+    }
   }
 }
 
@@ -389,7 +413,10 @@ __device__ __forceinline__ float stage_dact(const BpttStage& s, int e, int c) {
 
 }  // namespace
 
-template <bool FULL>
+// LOSS: grad_output is not read; it is formed per element from the state history and the loss head's row
+// coefficients,  up * (kc cos(phi_i) + ks sin(phi_i) + beta sign(r_i)),  phi_i = 2 pi i / N,
+// up = upstream / (T * B)  (what ring_loss_grad_kernel would have written to HBM for this kernel to read back).
+template <bool FULL, bool LOSS>
 __global__ __launch_bounds__(256) void ring_bptt_res256_kernel(RingBpttArgs p) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
   bf16x8* wlds = reinterpret_cast<bf16x8*>(smem);
@@ -420,10 +447,21 @@ __global__ __launch_bounds__(256) void ring_bptt_res256_kernel(RingBpttArgs p) {
       okf[e][c] = ((b0 + e < B) && (i0 + c < N)) ? 1.f : 0.f;
     }
 
+  float cs[R_NC], sn[R_NC], up = 0.f;
+  if constexpr (LOSS) {
+#pragma unroll
+    for (int c = 0; c < R_NC; ++c) {
+      const float phi = 6.2831853071795864769f * (float)(i0 + c) / (float)N;
+      cs[c] = cosf(phi);
+      sn[c] = sinf(phi);
+    }
+    up = (p.loss_upstream ? p.loss_upstream[0] : 1.f) * p.loss_inv_rows;
+  }
+
   pair_zero_tail<R_NC>(p.gfrag, T, p.nbt, bt, w, lane);
   BpttStage st[R_BPTT_DEPTH];
 #pragma unroll
-  for (int d = 0; d < R_BPTT_DEPTH; ++d) bptt_stage_load<FULL>(p, T - 1 - d, bt, w, lane, b0, i0, st[d]);
+  for (int d = 0; d < R_BPTT_DEPTH; ++d) bptt_stage_load<FULL, LOSS>(p, T - 1 - d, bt, w, lane, b0, i0, st[d]);
   GateStage gs;
   gates_fetch(p.A, T, B, bt, 0, -1, tid, gs);
   gates_publish(gbuf, tid, B, bt, gs);
@@ -444,20 +482,34 @@ __global__ __launch_bounds__(256) void ring_bptt_res256_kernel(RingBpttArgs p) {
       // issued after this stage's six loads: per step since then, four operand-copy stores and another
       // stage's six loads.  The counter is in order, so "at most 10 * (depth - 1) outstanding" means this
       // stage landed; a smaller number would also wait for later loads and for store acknowledgements.
-      if constexpr (FULL) bptt_stage_wait<10 * (R_BPTT_DEPTH - 1)>(S);
+      // (with the loss head fused in a stage has four more loads: 14 per step)
+      if constexpr (FULL) bptt_stage_wait<(LOSS ? 14 : 10) * (R_BPTT_DEPTH - 1), LOSS>(S);
 
       float G[4][R_NC], g[4][R_NC];
 #pragma unroll
-      for (int e = 0; e < 4; ++e)
+      for (int e = 0; e < 4; ++e) {
+        float kc = 0.f, ks = 0.f, beta = 0.f;
+        if constexpr (LOSS) {
+          kc = S.C[e][0] * up;
+          ks = S.C[e][1] * up;
+          beta = S.C[e][2] * up;
+        }
 #pragma unroll
         for (int c = 0; c < R_NC; ++c) {
-          G[e][c] = S.G[e][c] + carry[e][c];
+          float go = S.G[e][c];
+          if constexpr (LOSS) {
+            const float r = go;                                      // the stage holds the state, not a gradient
+            const float sb = r != 0.f ? __builtin_copysignf(beta, r) : 0.f;   // beta * sign(r), sign(0) = 0
+            go = fmaf(kc, cs[c], fmaf(ks, sn[c], sb));
+          }
+          G[e][c] = go + carry[e][c];
           g[e][c] = stage_dact(S, e, c) * G[e][c];
         }
+      }
       bf16x8* xb = xbuf + cur * R_XSLOTS;
       write_operand<R_NC>(xb, g, w, q, n);
       pair_store<R_NC>(p.gfrag, t, p.nbt, bt, w, lane, g);
-      bptt_stage_load<FULL>(p, t - R_BPTT_DEPTH, bt, w, lane, b0, i0, S);
+      bptt_stage_load<FULL, LOSS>(p, t - R_BPTT_DEPTH, bt, w, lane, b0, i0, S);
       lds_barrier();
 
       bf16x8 af[R_KCH];
@@ -511,7 +563,7 @@ __global__ __launch_bounds__(256) void ring_bptt_res256_kernel(RingBpttArgs p) {
   // while their destination registers are still reserved, before anything below reuses them
   if constexpr (FULL) {
 #pragma unroll
-    for (int d = 0; d < R_BPTT_DEPTH; ++d) bptt_stage_wait<0>(st[d]);
+    for (int d = 0; d < R_BPTT_DEPTH; ++d) bptt_stage_wait<0, LOSS>(st[d]);
   }
   if (p.grad_r_init) rows_store<R_NC>(p.grad_r_init, N, B, b0, i0, carry);
 }
@@ -548,9 +600,9 @@ hipError_t ring_launch_fwd_res256(const RingFwdArgs& a, hipStream_t st) {
   }
 }
 
-template <bool FULL>
+template <bool FULL, bool LOSS>
 static hipError_t launch_bptt_variant(const RingBpttArgs& a, hipStream_t st) {
-  auto kern = ring_bptt_res256_kernel<FULL>;
+  auto kern = ring_bptt_res256_kernel<FULL, LOSS>;
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                                      (int)R_LDS_BYTES);
   if (e != hipSuccess) return e;
@@ -560,5 +612,6 @@ static hipError_t launch_bptt_variant(const RingBpttArgs& a, hipStream_t st) {
 
 hipError_t ring_launch_bptt_res256(const RingBpttArgs& a, hipStream_t st) {
   const bool full = (a.N == 256) && (a.B % 16 == 0);
-  return full ? launch_bptt_variant<true>(a, st) : launch_bptt_variant<false>(a, st);
+  if (a.loss_coef) return full ? launch_bptt_variant<true, true>(a, st) : launch_bptt_variant<false, true>(a, st);
+  return full ? launch_bptt_variant<true, false>(a, st) : launch_bptt_variant<false, false>(a, st);
 }

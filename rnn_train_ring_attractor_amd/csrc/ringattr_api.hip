@@ -152,27 +152,80 @@ int ringattr_fwd(const void* A, const void* Wa, float J0, float J1, const void* 
   return RINGATTR_OK;
 }
 
+// Whether the BPTT kernel for this problem can form grad_output from the loss head's row coefficients itself.
+static bool loss_fuses_into_bptt(int N, int a_dim, bool want_grad_A) { return ring_uses_resident(N, a_dim) && !want_grad_A; }
+
+size_t ringattr_bwd_loss_workspace_bytes(int N, int a_dim, int seq_len, int batch_size, int have_saved, int want_grad_A) {
+  const size_t base = ringattr_bwd_workspace_bytes(N, a_dim, seq_len, batch_size, have_saved);
+  if (base == 0 || loss_fuses_into_bptt(N, a_dim, want_grad_A != 0)) return base;
+  // the two-pass route (other geometries, or grad_A requested) keeps grad_output [T,B,N] behind the plain workspace
+  return base + align_up((size_t)seq_len * batch_size * N * sizeof(float));
+}
+
+// grad_output != null: plain backward.  Otherwise loss_workspace (filled by ringattr_loss_fwd) describes grad_output.
+static int bwd_impl(const char* who, const void* grad_output, const void* loss_workspace, const void* upstream, const void* A,
+                    const void* Wa, float J0, float J1, const void* Wo, const void* bump_history, const void* r_init,
+                    void* grad_Wa, void* grad_Wo, float alpha, int N, int a_dim, int seq_len, int batch_size,
+                    int activation_type, const void* saved, void* grad_A, void* grad_r_init, void* workspace,
+                    size_t workspace_bytes, void* stream);
+
 int ringattr_bwd(const void* grad_output, const void* A, const void* Wa, float J0, float J1, const void* Wo,
                  const void* bump_history, const void* r_init, void* grad_Wa, void* grad_Wo, float alpha, int N,
                  int a_dim, int seq_len, int batch_size, int activation_type, const void* saved, void* grad_A,
                  void* grad_r_init, void* workspace, size_t workspace_bytes, void* stream) {
+  if (!grad_output) return fail(RINGATTR_ERR_INVALID, "ringattr_bwd: null tensor pointer");
+  return bwd_impl("ringattr_bwd", grad_output, nullptr, nullptr, A, Wa, J0, J1, Wo, bump_history, r_init, grad_Wa, grad_Wo,
+                  alpha, N, a_dim, seq_len, batch_size, activation_type, saved, grad_A, grad_r_init, workspace,
+                  workspace_bytes, stream);
+}
+
+int ringattr_bwd_loss(const void* loss_workspace, const void* upstream, const void* A, const void* Wa, float J0, float J1,
+                      const void* Wo, const void* bump_history, const void* r_init, void* grad_Wa, void* grad_Wo,
+                      float alpha, int N, int a_dim, int seq_len, int batch_size, int activation_type, const void* saved,
+                      void* grad_A, void* grad_r_init, void* workspace, size_t workspace_bytes, void* stream) {
+  if (!loss_workspace) return fail(RINGATTR_ERR_INVALID, "ringattr_bwd_loss: null loss workspace");
+  if (!aligned16(loss_workspace)) return fail(RINGATTR_ERR_INVALID, "ringattr_bwd_loss: every pointer must be 16-byte aligned");
+  if (N > 1024) return fail(RINGATTR_ERR_INVALID, "the loss head supports N <= 1024 (got %d)", N);
+  return bwd_impl("ringattr_bwd_loss", nullptr, loss_workspace, upstream, A, Wa, J0, J1, Wo, bump_history, r_init, grad_Wa,
+                  grad_Wo, alpha, N, a_dim, seq_len, batch_size, activation_type, saved, grad_A, grad_r_init, workspace,
+                  workspace_bytes, stream);
+}
+
+static int bwd_impl(const char* who, const void* grad_output, const void* loss_workspace, const void* upstream, const void* A,
+                    const void* Wa, float J0, float J1, const void* Wo, const void* bump_history, const void* r_init,
+                    void* grad_Wa, void* grad_Wo, float alpha, int N, int a_dim, int seq_len, int batch_size,
+                    int activation_type, const void* saved, void* grad_A, void* grad_r_init, void* workspace,
+                    size_t workspace_bytes, void* stream) {
   Geo g;
   int rc = make_geo(N, a_dim, seq_len, batch_size, g);
   if (rc) return rc;
   if ((rc = check_act(activation_type))) return rc;
-  if (!grad_output || !A || !Wa || !Wo || !bump_history || !r_init || !grad_Wa || !grad_Wo)
-    return fail(RINGATTR_ERR_INVALID, "ringattr_bwd: null tensor pointer");
+  if (!A || !Wa || !Wo || !bump_history || !r_init || !grad_Wa || !grad_Wo)
+    return fail(RINGATTR_ERR_INVALID, "%s: null tensor pointer", who);
   if (grad_A && (size_t)2 * a_dim * 64 * sizeof(float) > 24 * 1024)
-    return fail(RINGATTR_ERR_INVALID, "ringattr_bwd: grad_A is supported for a_dim <= 48 (got %d)", a_dim);
+    return fail(RINGATTR_ERR_INVALID, "%s: grad_A is supported for a_dim <= 48 (got %d)", who, a_dim);
   if (!aligned16(grad_output) || !aligned16(A) || !aligned16(Wa) || !aligned16(Wo) || !aligned16(bump_history) ||
       !aligned16(r_init) || !aligned16(grad_Wa) || !aligned16(grad_Wo) || !aligned16(saved) ||
       !aligned16(grad_r_init) || !aligned16(grad_A) || !aligned16(workspace))
-    return fail(RINGATTR_ERR_INVALID, "ringattr_bwd: every pointer must be 16-byte aligned");
-  const size_t need = ringattr_bwd_workspace_bytes(N, a_dim, seq_len, batch_size, saved != nullptr);
+    return fail(RINGATTR_ERR_INVALID, "%s: every pointer must be 16-byte aligned", who);
+  const size_t base_need = ringattr_bwd_workspace_bytes(N, a_dim, seq_len, batch_size, saved != nullptr);
+  const size_t need = loss_workspace ? ringattr_bwd_loss_workspace_bytes(N, a_dim, seq_len, batch_size, saved != nullptr,
+                                                                         grad_A != nullptr)
+                                     : base_need;
   if (!workspace || workspace_bytes < need)
-    return fail(RINGATTR_ERR_WORKSPACE, "ringattr_bwd: workspace of %zu bytes needed, %zu given", need,
+    return fail(RINGATTR_ERR_WORKSPACE, "%s: workspace of %zu bytes needed, %zu given", who, need,
                 workspace ? workspace_bytes : (size_t)0);
   hipStream_t st = static_cast<hipStream_t>(stream);
+
+  const bool fused_loss = loss_workspace && loss_fuses_into_bptt(N, a_dim, grad_A != nullptr);
+  if (loss_workspace && !fused_loss) {
+    // two passes: write grad_output behind the plain backward's workspace, then read it back below
+    float* G = (float*)((char*)workspace + base_need);
+    hipError_t e = ring_launch_loss_bwd((const float*)bump_history, nullptr, nullptr, 0.f, (const float*)upstream, G, N, seq_len,
+                                        batch_size, loss_workspace, st);
+    if (e != hipSuccess) return hip_fail(e, "loss head backward launch");
+    grad_output = G;
+  }
 
   char* ws = (char*)workspace;
   void* wb = ws;
@@ -239,6 +292,9 @@ int ringattr_bwd(const void* grad_output, const void* A, const void* Wa, float J
   b.grad_A = (float*)grad_A;
   b.hist = (const float*)bump_history;
   b.r_init = (const float*)r_init;
+  b.loss_coef = fused_loss ? ring_loss_row_coefficients(loss_workspace) : nullptr;
+  b.loss_upstream = (const float*)upstream;
+  b.loss_inv_rows = 1.f / ((float)seq_len * (float)batch_size);
   b.J0 = J0;
   b.J1 = J1;
   b.alpha = alpha;

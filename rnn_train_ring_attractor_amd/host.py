@@ -179,6 +179,18 @@ class GeneralizedRingAttractorNoGain(nn.Module):
         return ring_rnn_cuda_func(action_signal=action_signal, Wa=self.Wa, J0=self.J0, J1=self.J1, Wo=self.Wo,
                                   r_init=r_init, alpha=0.15, activation=self.activation_name)
 
+    def loss_pair(self, action_signal, target_angle, r_init=None, bump_weight=0.2):
+        """(total, cos_loss, amp_loss, bump_history) of the training script's objective, time loop and loss head as
+        one operator: its backward forms the loss gradient inside the BPTT kernel where the geometry allows."""
+        from .loss_head import ring_rnn_loss_func
+        batch_size, _, action_dim = action_signal.shape
+        assert action_dim == self.action_dim, f"Expected action_dim {self.action_dim}, got {action_dim}"
+        if r_init is None:
+            angle = torch.full((batch_size,), math.pi, device=self.Wo.device)
+            r_init = create_initial_bump(angle, self.num_neurons, device=self.Wo.device)
+        return ring_rnn_loss_func(action_signal, self.Wa, self.J0, self.J1, self.Wo, r_init, 0.15, self.activation_name,
+                                  target_angle, bump_weight)
+
     def forward(self, action_signal, r_init=None):
         bump = self.forward_history(action_signal, r_init).permute(1, 0, 2)
         proj = bump @ self.W_delta7

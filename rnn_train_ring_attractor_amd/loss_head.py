@@ -20,6 +20,7 @@ import torch
 from torch.autograd import Function
 
 from . import _lib
+from .rnn_cuda import fwd_cuda, bwd_cuda, saved_nbytes
 
 
 def _check(name, t, shape, device):
@@ -83,3 +84,67 @@ def ring_loss_pair(bump_history, target_angle, bump_weight=0.2, target_amplitude
     """Returns (total, cos_loss, amp_loss) as 0-dim tensors; only `total` is differentiable."""
     total, parts = RingLossPair.apply(bump_history, target_angle, bump_weight, target_amplitude)
     return total, parts[1], parts[2]
+
+
+class RingRnnLossFunc(Function):
+    """The time loop and the loss pair as one differentiable operator: forward = `ring_rnn_cuda_func` followed by
+    the fused loss head; backward = one library call in which the BPTT kernel forms the loss gradient itself
+    (weight-resident geometry) instead of reading a [T,B,N] grad_output tensor that a loss backward wrote."""
+
+    @staticmethod
+    def forward(ctx, action_signal, Wa, J0, J1, Wo, r_init, alpha, activation_name, target_angle, bump_weight,
+                target_amplitude):
+        from .ring_rnn_cuda import _activation_id
+        act = _activation_id(activation_name)
+        B, T, k = action_signal.shape
+        N = Wa.shape[1]
+        dev = action_signal.device
+        A, Wa_c, Wo_c, r0 = action_signal.contiguous(), Wa.contiguous(), Wo.contiguous(), r_init.contiguous()
+        angle = target_angle.contiguous()
+        _check("target_angle", angle, (B, T), dev)
+        amp = None
+        if target_amplitude is not None:
+            amp = target_amplitude.reshape(-1).contiguous()
+            _check("target_amplitude", amp, (B,), dev)
+        hist = torch.empty(T, B, N, device=dev, dtype=A.dtype)
+        needs_grad = any(ctx.needs_input_grad[i] for i in (0, 1, 4, 5))
+        saved = torch.empty(saved_nbytes(N, k, T, B), dtype=torch.uint8, device=dev) if needs_grad else None
+        fwd_cuda.fwd(A=A, Wa=Wa_c, J0=J0, J1=J1, Wo=Wo_c, r_init=r0, bump_history=hist, alpha=alpha,
+                     activation_type=act, saved=saved)
+        lib = _lib.load()
+        with torch.cuda.device(dev):
+            nbytes = lib.ringattr_loss_workspace_bytes(N, T, B)
+            if nbytes == 0:
+                _lib.check(1)
+            lws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+            out = torch.empty(3, dtype=torch.float32, device=dev)
+            _lib.check(lib.ringattr_loss_fwd(hist.data_ptr(), angle.data_ptr(), amp.data_ptr() if amp is not None else None,
+                                             float(bump_weight), out.data_ptr(), N, T, B, lws.data_ptr(), nbytes,
+                                             torch.cuda.current_stream(dev).cuda_stream))
+        ctx.save_for_backward(A, Wa_c, Wo_c, hist, r0, saved, lws)
+        ctx.J0, ctx.J1, ctx.alpha, ctx.act = J0, J1, alpha, act
+        ctx.mark_non_differentiable(out, hist)
+        return out[0].clone(), out, hist
+
+    @staticmethod
+    def backward(ctx, grad_total, _grad_parts, _grad_hist):
+        A, Wa, Wo, hist, r0, saved, lws = ctx.saved_tensors
+        grad_Wa, grad_Wo = torch.zeros_like(Wa), torch.zeros_like(Wo)
+        grad_A = torch.empty_like(A) if ctx.needs_input_grad[0] else None
+        grad_r0 = torch.empty_like(r0) if ctx.needs_input_grad[5] else None
+        up = grad_total.to(torch.float32).reshape(1).contiguous()
+        bwd_cuda.bwd(grad_output=None, A=A, Wa=Wa, J0=ctx.J0, J1=ctx.J1, Wo=Wo, bump_history=hist, r_init=r0,
+                     grad_Wa=grad_Wa, grad_Wo=grad_Wo, alpha=ctx.alpha, activation_type=ctx.act, saved=saved,
+                     grad_A=grad_A, grad_r_init=grad_r0, loss_workspace=lws, loss_upstream=up)
+        return grad_A, grad_Wa, None, None, grad_Wo, grad_r0, None, None, None, None, None
+
+
+def ring_rnn_loss_func(action_signal, Wa, J0, J1, Wo, r_init, alpha, activation, target_angle, bump_weight=0.2,
+                       target_amplitude=None):
+    """`ring_rnn_cuda_func(...)` and `ring_loss_pair(...)` in one operator.
+
+    Returns (total, cos_loss, amp_loss, bump_history); only `total` is differentiable (w.r.t. Wa, Wo and, when they
+    require it, action_signal and r_init); bump_history [T,B,N] is returned detached for decoding and logging."""
+    total, parts, hist = RingRnnLossFunc.apply(action_signal, Wa, J0, J1, Wo, r_init, alpha, activation, target_angle,
+                                               bump_weight, target_amplitude)
+    return total, parts[1], parts[2], hist

@@ -130,8 +130,14 @@ class _Bwd:
     def bwd(grad_output, A, Wa, J0, J1, Wo, bump_history, re_history=None, r_init=None, grad_Wa=None, grad_Wo=None,
             alpha=None, activation_type=None, grad_r=None, W_eff_temp=None, grad_re_temp=None,
             grad_W_eff_temp_bf16=None, A_t_temp_bf16=None, grad_re_temp_T=None, cublas_handle=None,
-            saved=None, grad_r_init=None, grad_A=None, stream=None):
-        for name, t in (("grad_output", grad_output), ("A", A), ("Wa", Wa), ("Wo", Wo),
+            saved=None, grad_r_init=None, grad_A=None, stream=None, loss_workspace=None, loss_upstream=None):
+        # loss_workspace (what the fused loss head's forward filled for this bump_history) in place of grad_output:
+        # the gradient of the loss pair is then formed inside the backward, scaled by loss_upstream (1-element tensor)
+        if (grad_output is None) == (loss_workspace is None):
+            raise TypeError("bwd() needs exactly one of grad_output and loss_workspace")
+        if grad_output is not None:
+            _contig("grad_output", grad_output)
+        for name, t in (("A", A), ("Wa", Wa), ("Wo", Wo),
                         ("bump_history", bump_history), ("r_init", r_init), ("grad_Wa", grad_Wa), ("grad_Wo", grad_Wo)):
             _contig(name, t)
         # the reference's workspaces: contiguity is all it ever checked (cpp/bwd.cpp:66-72); unused here
@@ -146,9 +152,13 @@ class _Bwd:
         act = _act(activation_type)
         J0, J1, alpha = _scalar("J0", J0), _scalar("J1", J1), _scalar("alpha", alpha)
         dev = A.device
-        specs = [("A", A, (B, T, k)), ("grad_output", grad_output, (T, B, N)), ("Wa", Wa, (k, N, N)),
+        specs = [("A", A, (B, T, k)), ("Wa", Wa, (k, N, N)),
                  ("Wo", Wo, (N, N)), ("bump_history", bump_history, (T, B, N)), ("r_init", r_init, (B, N)),
                  ("grad_Wa", grad_Wa, (k, N, N)), ("grad_Wo", grad_Wo, (N, N))]
+        if grad_output is not None:
+            specs.append(("grad_output", grad_output, (T, B, N)))
+        if loss_upstream is not None:
+            specs.append(("loss_upstream", loss_upstream, (1,)))
         if grad_r_init is not None:
             specs.append(("grad_r_init", grad_r_init, (B, N)))
         if grad_A is not None:
@@ -160,6 +170,25 @@ class _Bwd:
             need = lib.ringattr_saved_bytes(N, k, T, B)
             if saved.dtype != torch.uint8 or saved.numel() < need or saved.device != dev:
                 raise ValueError(f"saved must be a uint8 tensor of at least {need} bytes on {dev}")
+        if loss_workspace is not None:
+            _contig("loss_workspace", loss_workspace)
+            need = lib.ringattr_loss_workspace_bytes(N, T, B)
+            if need == 0:
+                _lib.check(1)
+            if loss_workspace.dtype != torch.uint8 or loss_workspace.numel() < need or loss_workspace.device != dev:
+                raise ValueError(f"loss_workspace must be a uint8 tensor of at least {need} bytes on {dev}")
+            with torch.cuda.device(dev):
+                ws_bytes = lib.ringattr_bwd_loss_workspace_bytes(N, k, T, B, 1 if saved is not None else 0,
+                                                                 1 if grad_A is not None else 0)
+                if ws_bytes == 0:
+                    _lib.check(1)
+                ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+                rc = lib.ringattr_bwd_loss(_ptr(loss_workspace), _ptr(loss_upstream), _ptr(A), _ptr(Wa), J0, J1, _ptr(Wo),
+                                           _ptr(bump_history), _ptr(r_init), _ptr(grad_Wa), _ptr(grad_Wo), alpha, N, k, T,
+                                           B, act, _ptr(saved), _ptr(grad_A), _ptr(grad_r_init), _ptr(ws), ws_bytes,
+                                           _stream_ptr(stream, dev))
+            _lib.check(rc)
+            return None
         with torch.cuda.device(dev):
             ws_bytes = lib.ringattr_bwd_workspace_bytes(N, k, T, B, 1 if saved is not None else 0)
             if ws_bytes == 0:

@@ -66,3 +66,56 @@ def test_loss_head_agrees_with_the_torch_chain_on_operator_output(gpu_device):
     assert abs(grads[0][0] - grads[1][0]) <= 1e-4 * max(1.0, abs(grads[1][0]))
     assert O.cosine(grads[0][1], grads[1][1]) >= 0.9999 and O.cosine(grads[0][2], grads[1][2]) >= 0.9999
     assert O.max_rel_err(grads[0][1], grads[1][1]) <= 2e-3
+
+
+@pytest.mark.parametrize("B,T,k,N,act,own,streaming", [
+    (64, 24, 2, 256, "gelu", True, "0"),        # weight-resident geometry, unmasked kernel: gradient formed inside BPTT
+    (37, 9, 2, 200, "tanh", False, "0"),        # weight-resident geometry, masked rows and neurons
+    (37, 9, 2, 200, "tanh", False, "1"),        # same problem on the streaming kernels: two passes inside the library
+    (20, 6, 3, 96, "silu", True, "0"),          # a geometry that always takes the two passes
+], ids=["n256_full", "n200_masked", "n200_streaming", "n96_k3"])
+def test_time_loop_and_loss_as_one_operator(B, T, k, N, act, own, streaming, gpu_device, monkeypatch):
+    """ring_rnn_loss_func (one backward call, the loss gradient formed inside the BPTT kernel where the geometry
+    allows) against ring_rnn_cuda_func + ring_loss_pair, and against the fp64 oracle: loss pair of the oracle's
+    trajectory, its gradient pushed through the oracle's BPTT."""
+    from rnn_train_ring_attractor_amd import ring_loss_pair, ring_rnn_cuda_func, ring_rnn_loss_func
+    from tests.ring_cases import make_problem
+    print(f"[case] time loop + loss operator B={B} T={T} k={k} N={N} {act} own_target={own} streaming={streaming}", flush=True)
+    monkeypatch.setenv("RINGATTR_STREAMING", streaming)
+    p = make_problem(300 + N + B, B, T, k, N, weights="perfect" if k == 2 else "random")
+    J0, J1 = (-1.0 / N, 2.0 / N) if k == 2 else (-0.1, 0.1)
+    t = lambda x: torch.tensor(np.ascontiguousarray(x), device=gpu_device)
+    rng = np.random.default_rng(5)
+    angle = t(p["angle"]) if "angle" in p else t((rng.random((B, T)) * 2 * np.pi).astype(np.float32))
+    tgt_np = None if own else (rng.random(B) + 1.0).astype(np.float32)
+    tgt = None if own else t(tgt_np)
+    res = {}
+    for fused in (True, False):
+        Wa, Wo = t(p["Wa"]).requires_grad_(True), t(p["Wo"]).requires_grad_(True)
+        r0 = t(p["r0"]).requires_grad_(True)
+        if fused:
+            total, lc, la, hist = ring_rnn_loss_func(t(p["A"]), Wa, J0, J1, Wo, r0, 0.15, act, angle, 0.2, tgt)
+        else:
+            hist = ring_rnn_cuda_func(t(p["A"]), Wa, J0, J1, Wo, r0, 0.15, act)
+            total, lc, la = ring_loss_pair(hist, angle, 0.2, tgt)
+        (2.5 * total).backward()
+        torch.cuda.synchronize()
+        res[fused] = (float(total), float(lc), float(la), hist.detach().cpu().numpy(), Wo.grad.cpu().numpy(),
+                      Wa.grad.cpu().numpy(), r0.grad.cpu().numpy())
+    f, s = res[True], res[False]
+    assert f[0] == s[0] and f[1] == s[1] and f[2] == s[2] and np.array_equal(f[3], s[3])     # same forward kernels
+    for a, b in zip(f[4:], s[4:]):
+        assert np.isfinite(a).all()
+        assert O.max_rel_err(a, b) <= 2e-3 and O.cosine(a, b) >= 0.99999
+    # fp64: the oracle's trajectory and its loss pair; the loss gradient is taken at the trajectory the kernel saw
+    # (it divides by the squared read-out amplitude, so it amplifies the bf16-level trajectory difference, which
+    # the trajectory tolerance already covers) and pushed through the oracle's BPTT
+    ang_np = angle.cpu().numpy()
+    ref_hist, _ = O.forward_dense(p["A"], p["Wa"], J0, J1, p["Wo"], p["r0"], 0.15, act)
+    want_total = O.loss_pair_rank2(ref_hist, ang_np, 0.2, tgt_np)[0]
+    gl = O.loss_pair_rank2(f[3], ang_np, 0.2, tgt_np)[3]
+    ref = O.backward_dense(2.5 * gl, p["A"], p["Wa"], J0, J1, p["Wo"], ref_hist, p["r0"], 0.15, act)
+    assert abs(f[0] - want_total) <= 1e-2 * max(1.0, abs(want_total))
+    for got, key in ((f[4], "grad_Wo"), (f[5], "grad_Wa"), (f[6], "grad_r_init")):
+        assert O.cosine(got, ref[key]) >= 0.999, key
+        assert O.max_rel_err(got, ref[key]) <= 2e-2, key

@@ -1,7 +1,7 @@
 """Training driver with the reference script's import lines and call pattern (no plotting):
 AV batches -> action signal -> initial bump -> ring_rnn_cuda_func -> loss pair -> clip -> Adam.
-fused_loss=True computes the same loss pair and its gradient with the fused HIP loss head instead of the chain
-of torch tensor ops (one pass over the history each way instead of about a dozen)."""
+fused_loss=True computes the same loss pair with the fused HIP loss head instead of the chain of torch tensor ops
+(one pass over the history instead of about a dozen) and lets the backward kernels form its gradient themselves."""
 import numpy as np
 
 from utils.generate_av_integration_data import AVIntegrationDataset
@@ -25,8 +25,7 @@ def run_training(action_dim=2, num_neurons=256, training_steps=1000, batch_size=
         action = av_to_action_signal_ND(av, action_dim)
         r_init = create_initial_bump(target[:, 0], num_neurons, device=device)
         if fused_loss:
-            from rnn_train_ring_attractor_amd import ring_loss_pair
-            total, loss, _ = ring_loss_pair(model.forward_history(action, r_init=r_init), target, 0.2)
+            total, loss, _, _ = model.loss_pair(action, target, r_init=r_init, bump_weight=0.2)
         else:
             wave, bump = model(action, r_init=r_init)
             loss = cosine_similarity_loss(wave, target)
