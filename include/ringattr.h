@@ -114,12 +114,9 @@ RINGATTR_API int ringattr_loss_bwd(const void* bump_history, const void* target_
  * in one call.  No counterpart in the reference (its training script lets autograd chain the torch loss ops into
  * RingRnnCudaFunc.backward, cpp/ring_rnn_cuda.py:81-144).  loss_workspace is the workspace ringattr_loss_fwd
  * filled for this bump_history; upstream is one device float (d objective / d total) or NULL for 1; every other
- * argument is ringattr_bwd's.  For the weight-resident geometry (a_dim == 2, 128 < N <= 256, no grad_A) the BPTT
- * kernel forms grad_output in registers from bump_history and the loss head's per-row coefficients, and the
- * [T,B,N] gradient never goes through HBM; otherwise the library writes it into its workspace and reads it back
- * (what ringattr_loss_bwd followed by ringattr_bwd would do; the workspace query below then includes that buffer). */
-RINGATTR_API size_t ringattr_bwd_loss_workspace_bytes(int N, int a_dim, int seq_len, int batch_size, int have_saved,
-                      int want_grad_A);
+ * argument is ringattr_bwd's, the workspace included (ringattr_bwd_workspace_bytes).  The BPTT kernels form
+ * grad_output in registers from the bump_history rows they load in its place and the loss head's per-row
+ * coefficients, so the [T,B,N] gradient is neither written nor read. */
 RINGATTR_API int ringattr_bwd_loss(const void* loss_workspace, const void* upstream, const void* A, const void* Wa,
                       float J0, float J1, const void* Wo, const void* bump_history, const void* r_init,
                       void* grad_Wa, void* grad_Wo, float alpha,

@@ -37,7 +37,6 @@ PROTOTYPES = {
                                   c_void_p, c_size_t, c_void_p]),
     "ringattr_loss_bwd": (c_int, [c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_int, c_int, c_int,
                                   c_void_p, c_size_t, c_void_p]),
-    "ringattr_bwd_loss_workspace_bytes": (c_size_t, [c_int] * 6),
     "ringattr_bwd_loss": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_float, c_void_p, c_void_p, c_void_p,
                                   c_void_p, c_void_p, c_float, c_int, c_int, c_int, c_int, c_int,
                                   c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),

@@ -447,7 +447,9 @@ __device__ __forceinline__ void bptt_flush_grad_A(const RingBpttArgs& p, const f
 // GA: also produce grad_A[b,t,c] = sum_j (g Wa[c])[j] * r_prev[j] (one batch tile per workgroup).  The
 // per-wave shares of a step go to a double-buffered LDS array (2*k*64 floats behind the operand buffers
 // in dynamic shared memory) and are summed in wave order and written out after the next step's barrier.
-template <int NC, bool GA, int RT>
+// LOSS: grad_output is not read; it is formed per element from the state history and the loss head's row
+// coefficients,  up * (kc cos(phi_i) + ks sin(phi_i) + beta sign(r_i)),  phi_i = 2 pi i / N,  up = upstream / (T * B).
+template <int NC, bool GA, int RT, bool LOSS>
 __global__ __launch_bounds__(256) void ring_bptt_kernel(RingBpttArgs p) {
   static_assert(!GA || RT == 1, "dL/dA is produced one batch tile at a time");
   using TL = Tile<NC>;
@@ -475,6 +477,23 @@ __global__ __launch_bounds__(256) void ring_bptt_kernel(RingBpttArgs p) {
       for (int c = 0; c < NC; ++c) carry[rt][e][c] = 0.f;
     if (bt0 + rt < p.nbt) pair_zero_tail<NC>(p.gfrag, T, p.nbt, bt0 + rt, w, lane);
   }
+  // the lane's cos(phi_i), sin(phi_i): in registers, or (paired tiles, where registers are short) in LDS
+  constexpr bool CS_LDS = LOSS && RT > 1;
+  __shared__ float cs_lds[CS_LDS ? 2 * NC * 256 : 1];
+  float cs[NC], sn[NC], up = 0.f;
+  if constexpr (LOSS) {
+#pragma unroll
+    for (int c = 0; c < NC; ++c) {
+      const float phi = 6.2831853071795864769f * (float)(i0 + c) / (float)N;
+      cs[c] = cosf(phi);
+      sn[c] = sinf(phi);
+      if constexpr (CS_LDS) {
+        cs_lds[(2 * c) * 256 + tid] = cs[c];
+        cs_lds[(2 * c + 1) * 256 + tid] = sn[c];
+      }
+    }
+    up = (p.loss_upstream ? p.loss_upstream[0] : 1.f) * p.loss_inv_rows;
+  }
 
   // The weight pipeline restarts every step here: a step begins by waiting for grad_output and the saved
   // record from HBM, which hides the refill, and carrying the buffers over would cost registers.
@@ -487,7 +506,23 @@ __global__ __launch_bounds__(256) void ring_bptt_kernel(RingBpttArgs p) {
     for (int rt = 0; rt < RT; ++rt) {
       const bool live = bt0 + rt < p.nbt;
       float G[4][NC], g[4][NC];
-      rows_load<NC>(p.grad_out + (size_t)t * B * N, N, B, b0 + 16 * rt, i0, G);
+      rows_load<NC>((LOSS ? p.hist : p.grad_out) + (size_t)t * B * N, N, B, b0 + 16 * rt, i0, G);
+      if constexpr (LOSS) {   // G holds the state rows; columns past N get a finite value that meets F' = 0
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int b = b0 + 16 * rt + e;
+          const ring_f32x4 cf = p.loss_coef[(size_t)t * B + (b < B ? b : B - 1)];
+          const float kc = cf[0] * up, ks = cf[1] * up, beta = cf[2] * up;
+#pragma unroll
+          for (int c = 0; c < NC; ++c) {
+            const float r = G[e][c];
+            const float sb = r > 0.f ? beta : (r < 0.f ? -beta : 0.f);          // beta * sign(r), sign(0) = 0
+            const float co = CS_LDS ? cs_lds[(2 * c) * 256 + tid] : cs[c];
+            const float si = CS_LDS ? cs_lds[(2 * c + 1) * 256 + tid] : sn[c];
+            G[e][c] = fmaf(kc, co, fmaf(ks, si, sb));
+          }
+        }
+      }
       if (live) {
         side_load_f16<NC>(p.dfrag + side_offset<NC>(t, p.nbt, bt0 + rt, w, lane), g);
       } else {
@@ -856,15 +891,25 @@ hipError_t ring_launch_rebuild(const RingFwdArgs& a, int NCv, hipStream_t st) {
 hipError_t ring_launch_bptt(const RingBpttArgs& a, int NCv, hipStream_t st) {
   ProfScope prof(3, st);
   hipError_t e = hipErrorInvalidValue;
+  const bool loss = a.loss_coef != nullptr;
   if (a.grad_A) {   // the generic kernel is the one that also produces dL/dA
-    RING_DISPATCH_NC(NCv, e = launch_stream(ring_bptt_kernel<NC, true, 1>, dim3(a.nbt),
-                                            stream_lds_bytes<NC, 1>() + (size_t)2 * a.k * 64 * sizeof(float), st, a));
+    const size_t ga = (size_t)2 * a.k * 64 * sizeof(float);
+    if (loss) {
+      RING_DISPATCH_NC(NCv, e = launch_stream(ring_bptt_kernel<NC, true, 1, true>, dim3(a.nbt), stream_lds_bytes<NC, 1>() + ga, st, a));
+    } else {
+      RING_DISPATCH_NC(NCv, e = launch_stream(ring_bptt_kernel<NC, true, 1, false>, dim3(a.nbt), stream_lds_bytes<NC, 1>() + ga, st, a));
+    }
     return e;
   }
   if (ring_uses_resident(a.N, a.k)) return ring_launch_bptt_res256(a, st);
   const int rt = stream_row_tiles(NCv, a.nbt, false);
-  RING_DISPATCH_NC(NCv, RING_DISPATCH_RT(rt,
-      e = launch_stream(ring_bptt_kernel<NC, false, RT>, dim3((a.nbt + RT - 1) / RT), stream_lds_bytes<NC, RT>(), st, a)));
+  if (loss) {
+    RING_DISPATCH_NC(NCv, RING_DISPATCH_RT(rt,
+        e = launch_stream(ring_bptt_kernel<NC, false, RT, true>, dim3((a.nbt + RT - 1) / RT), stream_lds_bytes<NC, RT>(), st, a)));
+  } else {
+    RING_DISPATCH_NC(NCv, RING_DISPATCH_RT(rt,
+        e = launch_stream(ring_bptt_kernel<NC, false, RT, false>, dim3((a.nbt + RT - 1) / RT), stream_lds_bytes<NC, RT>(), st, a)));
+  }
   return e;
 }
 

@@ -499,7 +499,7 @@ __global__ __launch_bounds__(256) void ring_bptt_res256_kernel(RingBpttArgs p) {
           float go = S.G[e][c];
           if constexpr (LOSS) {
             const float r = go;                                      // the stage holds the state, not a gradient
-            const float sb = r != 0.f ? __builtin_copysignf(beta, r) : 0.f;   // beta * sign(r), sign(0) = 0
+            const float sb = r > 0.f ? beta : (r < 0.f ? -beta : 0.f);          // beta * sign(r), sign(0) = 0
             go = fmaf(kc, cs[c], fmaf(ks, sn[c], sb));
           }
           G[e][c] = go + carry[e][c];

@@ -152,16 +152,6 @@ int ringattr_fwd(const void* A, const void* Wa, float J0, float J1, const void* 
   return RINGATTR_OK;
 }
 
-// Whether the BPTT kernel for this problem can form grad_output from the loss head's row coefficients itself.
-static bool loss_fuses_into_bptt(int N, int a_dim, bool want_grad_A) { return ring_uses_resident(N, a_dim) && !want_grad_A; }
-
-size_t ringattr_bwd_loss_workspace_bytes(int N, int a_dim, int seq_len, int batch_size, int have_saved, int want_grad_A) {
-  const size_t base = ringattr_bwd_workspace_bytes(N, a_dim, seq_len, batch_size, have_saved);
-  if (base == 0 || loss_fuses_into_bptt(N, a_dim, want_grad_A != 0)) return base;
-  // the two-pass route (other geometries, or grad_A requested) keeps grad_output [T,B,N] behind the plain workspace
-  return base + align_up((size_t)seq_len * batch_size * N * sizeof(float));
-}
-
 // grad_output != null: plain backward.  Otherwise loss_workspace (filled by ringattr_loss_fwd) describes grad_output.
 static int bwd_impl(const char* who, const void* grad_output, const void* loss_workspace, const void* upstream, const void* A,
                     const void* Wa, float J0, float J1, const void* Wo, const void* bump_history, const void* r_init,
@@ -208,24 +198,11 @@ static int bwd_impl(const char* who, const void* grad_output, const void* loss_w
       !aligned16(r_init) || !aligned16(grad_Wa) || !aligned16(grad_Wo) || !aligned16(saved) ||
       !aligned16(grad_r_init) || !aligned16(grad_A) || !aligned16(workspace))
     return fail(RINGATTR_ERR_INVALID, "%s: every pointer must be 16-byte aligned", who);
-  const size_t base_need = ringattr_bwd_workspace_bytes(N, a_dim, seq_len, batch_size, saved != nullptr);
-  const size_t need = loss_workspace ? ringattr_bwd_loss_workspace_bytes(N, a_dim, seq_len, batch_size, saved != nullptr,
-                                                                         grad_A != nullptr)
-                                     : base_need;
+  const size_t need = ringattr_bwd_workspace_bytes(N, a_dim, seq_len, batch_size, saved != nullptr);
   if (!workspace || workspace_bytes < need)
     return fail(RINGATTR_ERR_WORKSPACE, "%s: workspace of %zu bytes needed, %zu given", who, need,
                 workspace ? workspace_bytes : (size_t)0);
   hipStream_t st = static_cast<hipStream_t>(stream);
-
-  const bool fused_loss = loss_workspace && loss_fuses_into_bptt(N, a_dim, grad_A != nullptr);
-  if (loss_workspace && !fused_loss) {
-    // two passes: write grad_output behind the plain backward's workspace, then read it back below
-    float* G = (float*)((char*)workspace + base_need);
-    hipError_t e = ring_launch_loss_bwd((const float*)bump_history, nullptr, nullptr, 0.f, (const float*)upstream, G, N, seq_len,
-                                        batch_size, loss_workspace, st);
-    if (e != hipSuccess) return hip_fail(e, "loss head backward launch");
-    grad_output = G;
-  }
 
   char* ws = (char*)workspace;
   void* wb = ws;
@@ -292,7 +269,7 @@ static int bwd_impl(const char* who, const void* grad_output, const void* loss_w
   b.grad_A = (float*)grad_A;
   b.hist = (const float*)bump_history;
   b.r_init = (const float*)r_init;
-  b.loss_coef = fused_loss ? ring_loss_row_coefficients(loss_workspace) : nullptr;
+  b.loss_coef = loss_workspace ? ring_loss_row_coefficients(loss_workspace) : nullptr;
   b.loss_upstream = (const float*)upstream;
   b.loss_inv_rows = 1.f / ((float)seq_len * (float)batch_size);
   b.J0 = J0;

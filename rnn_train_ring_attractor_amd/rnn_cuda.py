@@ -178,8 +178,7 @@ class _Bwd:
             if loss_workspace.dtype != torch.uint8 or loss_workspace.numel() < need or loss_workspace.device != dev:
                 raise ValueError(f"loss_workspace must be a uint8 tensor of at least {need} bytes on {dev}")
             with torch.cuda.device(dev):
-                ws_bytes = lib.ringattr_bwd_loss_workspace_bytes(N, k, T, B, 1 if saved is not None else 0,
-                                                                 1 if grad_A is not None else 0)
+                ws_bytes = lib.ringattr_bwd_workspace_bytes(N, k, T, B, 1 if saved is not None else 0)
                 if ws_bytes == 0:
                     _lib.check(1)
                 ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)

@@ -68,22 +68,24 @@ def test_loss_head_agrees_with_the_torch_chain_on_operator_output(gpu_device):
     assert O.max_rel_err(grads[0][1], grads[1][1]) <= 2e-3
 
 
-@pytest.mark.parametrize("B,T,k,N,act,own,streaming", [
-    (64, 24, 2, 256, "gelu", True, "0"),        # weight-resident geometry, unmasked kernel: gradient formed inside BPTT
-    (37, 9, 2, 200, "tanh", False, "0"),        # weight-resident geometry, masked rows and neurons
-    (37, 9, 2, 200, "tanh", False, "1"),        # same problem on the streaming kernels: two passes inside the library
-    (20, 6, 3, 96, "silu", True, "0"),          # a geometry that always takes the two passes
-], ids=["n256_full", "n200_masked", "n200_streaming", "n96_k3"])
-def test_time_loop_and_loss_as_one_operator(B, T, k, N, act, own, streaming, gpu_device, monkeypatch):
-    """ring_rnn_loss_func (one backward call, the loss gradient formed inside the BPTT kernel where the geometry
-    allows) against ring_rnn_cuda_func + ring_loss_pair, and against the fp64 oracle: loss pair of the oracle's
-    trajectory, its gradient pushed through the oracle's BPTT."""
+@pytest.mark.parametrize("B,T,k,N,act,own,streaming,weights", [
+    (64, 24, 2, 256, "gelu", True, "0", "perfect"),   # weight-resident geometry, unmasked kernel
+    (48, 12, 2, 256, "tanh", True, "0", "random"),    # amplitude deviations of both signs (own target, drifting bump)
+    (37, 9, 2, 200, "tanh", False, "0", "perfect"),   # weight-resident geometry, masked rows and neurons
+    (37, 9, 2, 200, "tanh", True, "1", "random"),     # the streaming kernels, four column tiles
+    (20, 6, 3, 96, "silu", True, "0", "random"),      # the streaming kernels, two column tiles, three action channels
+    (40, 5, 2, 512, "tanh", True, "0", "random"),     # widest tiling
+], ids=["n256_full", "n256_random", "n200_masked", "n200_streaming", "n96_k3", "n512"])
+def test_time_loop_and_loss_as_one_operator(B, T, k, N, act, own, streaming, weights, gpu_device, monkeypatch):
+    """ring_rnn_loss_func (one backward call, the loss gradient formed inside the BPTT kernel) against
+    ring_rnn_cuda_func + ring_loss_pair (the gradient written to HBM and read back), and against the fp64 oracle:
+    loss pair of the oracle's trajectory, its gradient pushed through the oracle's BPTT."""
     from rnn_train_ring_attractor_amd import ring_loss_pair, ring_rnn_cuda_func, ring_rnn_loss_func
     from tests.ring_cases import make_problem
     print(f"[case] time loop + loss operator B={B} T={T} k={k} N={N} {act} own_target={own} streaming={streaming}", flush=True)
     monkeypatch.setenv("RINGATTR_STREAMING", streaming)
-    p = make_problem(300 + N + B, B, T, k, N, weights="perfect" if k == 2 else "random")
-    J0, J1 = (-1.0 / N, 2.0 / N) if k == 2 else (-0.1, 0.1)
+    p = make_problem(300 + N + B, B, T, k, N, weights=weights)
+    J0, J1 = (-1.0 / N, 2.0 / N) if weights == "perfect" else (-0.1, 0.1)
     t = lambda x: torch.tensor(np.ascontiguousarray(x), device=gpu_device)
     rng = np.random.default_rng(5)
     angle = t(p["angle"]) if "angle" in p else t((rng.random((B, T)) * 2 * np.pi).astype(np.float32))
