@@ -1,10 +1,11 @@
-// Weight-resident kernels for the headline geometry: 192 < N <= 256 (NPAD = 256, NC = 4), a_dim = 2.
+// Weight-resident kernels for the headline geometry: 128 < N <= 256 (NPAD = 256, NC = 4), a_dim = 2.
 //
 // [Wo|Wl|Wr] in bf16 is 384 KiB -- more than one CU's LDS (160 KiB) but less than its register
-// file (512 KiB).  Each of the 4 waves keeps its 64-neuron slice of two matrices (64 fragments,
-// 256 VGPRs) in registers for the whole sequence and the slice of the third in LDS (128 KiB per
-// workgroup, read back by the lane that wrote it), so no weight byte is fetched from L2/HBM inside
-// the time loop.  One workgroup per CU, one wave per SIMD, 16 batch rows per workgroup.
+// file (512 KiB).  A workgroup keeps the slices of the two gated matrices in registers for the whole
+// sequence (accumulation VGPRs, which MFMA reads as B operands) and the Wo slices in LDS (128 KiB per
+// workgroup, each read back by the lane that wrote it), so no weight byte is fetched from L2/HBM inside
+// the time loop.  One workgroup per CU and 16 batch rows per workgroup; the forward runs eight waves
+// (two per SIMD, in two roles half a step apart), BPTT four (one per SIMD).
 #include "ring_common.hpp"
 #include "ring_kernels.hpp"
 
