@@ -2,6 +2,8 @@
 same seeded inputs.  Tolerances (bf16 operands, fp32 accumulation): state trajectories and decoded
 angles within 1e-2 (max error over max magnitude); weight gradients cosine >= 0.999 and max error
 over max magnitude <= 2e-2."""
+import os
+
 import numpy as np
 import pytest
 import torch
@@ -27,7 +29,7 @@ ACTS = {"relu": 0, "gelu": 1, "tanh": 2, "silu": 3}
 def _rowsum_rounded(N, k):
     """The weight-resident kernels (a_dim == 2, 128 < N <= 256) take the J0 row sums over the bf16 operand copy
     of the state, the generic ones over the fp32 state; the rounding model follows the kernel under test."""
-    return k == 2 and 128 < N <= 256
+    return k == 2 and 128 < N <= 256 and os.environ.get("RINGATTR_STREAMING") != "1"
 
 
 CASES = [
