@@ -145,6 +145,10 @@ def ring_rnn_loss_func(action_signal, Wa, J0, J1, Wo, r_init, alpha, activation,
 
     Returns (total, cos_loss, amp_loss, bump_history); only `total` is differentiable (w.r.t. Wa, Wo and, when they
     require it, action_signal and r_init); bump_history [T,B,N] is returned detached for decoding and logging."""
+    from .ring_rnn_cuda import _silent_channel_view
+    compact = _silent_channel_view(action_signal, Wa)
+    if compact is not None:
+        action_signal, Wa = compact
     total, parts, hist = RingRnnLossFunc.apply(action_signal, Wa, J0, J1, Wo, r_init, alpha, activation, target_angle,
                                                bump_weight, target_amplitude)
     return total, parts[1], parts[2], hist

@@ -25,7 +25,40 @@ def ring_rnn_cuda_func(action_signal, Wa, J0, J1, Wo, r_init, alpha, activation=
     action_signal (B,T,k); Wa (k,N,N); J0, J1 scalars; Wo (N,N); r_init (B,N); alpha float;
     activation in {'relu','gelu','tanh','silu'}.  Returns bump_history (T,B,N).
     """
+    compact = _silent_channel_view(action_signal, Wa)
+    if compact is not None:
+        action_signal, Wa = compact
     return RingRnnCudaFunc.apply(action_signal, Wa, J0, J1, Wo, r_init, alpha, activation)
+
+
+def _silent_channel_view(action_signal, Wa):
+    """The training script pads the two driven action channels with zeros up to a_dim = 16
+    (train_general_ring_no_gain.py:52-66 of the reference).  A channel that is zero for every sample and step
+    contributes nothing forward and has an exactly zero weight gradient, so when at most two channels are driven
+    and N fits the weight-resident kernels (128 < N <= 256), the operator runs on those two channels: the slices
+    below are ordinary differentiable indexing, autograd scatters the gradients back (zeros elsewhere).
+    Finding the driven channels reads the action signal back once per call (a small reduction and one
+    device-to-host copy); RINGATTR_COMPACT_CHANNELS=0 switches this off (e.g. under graph capture)."""
+    import os
+    if os.environ.get("RINGATTR_COMPACT_CHANNELS", "1") == "0":
+        return None
+    if action_signal.dim() != 3 or Wa.dim() != 3 or not action_signal.is_cuda:
+        return None
+    k, N = action_signal.shape[2], Wa.shape[1]
+    if k <= 2 or not (128 < N <= 256) or Wa.shape[0] != k:
+        return None
+    if action_signal.requires_grad:        # dL/dA of a silent channel is not zero: keep every channel
+        return None
+    driven = torch.nonzero((action_signal != 0).flatten(0, 1).any(dim=0)).flatten().tolist()
+    if len(driven) > 2:
+        return None
+    for c in range(k):                     # fewer than two driven: fill up with silent ones (their gates are zero)
+        if len(driven) == 2:
+            break
+        if c not in driven:
+            driven.append(c)
+    idx = torch.tensor(sorted(driven), device=Wa.device)
+    return action_signal.index_select(2, idx), Wa.index_select(0, idx)
 
 
 class RingRnnCudaFunc(Function):

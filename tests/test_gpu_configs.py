@@ -203,6 +203,41 @@ def test_paired_batch_tiles_equal_single_tiles(B, T, k, N, act, saved, gpu_devic
     assert O.cosine(outs["2"][3], ref["grad_r_init"]) >= 0.999
 
 
+@pytest.mark.parametrize("driven", [(3, 9), (5,), (), (0, 1, 2)], ids=["two", "one", "none", "three"])
+def test_silent_action_channels_are_compacted(driven, gpu_device, monkeypatch):
+    """With a_dim > 2 and at most two channels ever driven, the Python operator runs the time loop on those two
+    (the weight-resident kernels at 128 < N <= 256).  Results must agree with the uncompacted run on all channels
+    (the streaming kernels), and the silent channels' weight gradients must be exactly zero either way."""
+    from rnn_train_ring_attractor_amd import ring_rnn_cuda_func
+    B, T, k, N = 40, 12, 12, 256
+    print(f"[case] silent channels, driven={driven}", flush=True)
+    p = make_problem(91, B, T, k, N, action="dense")
+    A = np.zeros_like(p["A"])
+    for c in driven:
+        A[..., c] = p["A"][..., c]
+    outs = {}
+    for mode in ("1", "0"):
+        monkeypatch.setenv("RINGATTR_COMPACT_CHANNELS", mode)
+        Wa, Wo = _t(p["Wa"], gpu_device).requires_grad_(True), _t(p["Wo"], gpu_device).requires_grad_(True)
+        r0 = _t(p["r0"], gpu_device).requires_grad_(True)
+        h = ring_rnn_cuda_func(_t(A, gpu_device), Wa, -0.1, 0.3, Wo, r0, 0.15, "tanh")
+        h.backward(_t(p["G"], gpu_device))
+        torch.cuda.synchronize()
+        outs[mode] = [x.cpu().numpy() for x in (h.detach(), Wa.grad, Wo.grad, r0.grad)]
+        for c in range(k):
+            if c not in driven:
+                assert np.abs(outs[mode][1][c]).max() == 0.0
+    for a, b in zip(outs["1"], outs["0"]):
+        assert a.shape == b.shape
+        assert O.max_rel_err(a, b) <= 5e-3          # two kernel families: same operands, different row-sum rounding
+    ref_hist, _ = O.forward_dense(A, p["Wa"], -0.1, 0.3, p["Wo"], p["r0"], 0.15, "tanh")
+    ref = O.backward_dense(p["G"], A, p["Wa"], -0.1, 0.3, p["Wo"], ref_hist, p["r0"], 0.15, "tanh")
+    assert O.max_rel_err(outs["1"][0], ref_hist) <= TRAJ_TOL
+    assert O.cosine(outs["1"][2], ref["grad_Wo"]) >= GRAD_COS and O.max_rel_err(outs["1"][2], ref["grad_Wo"]) <= GRAD_TOL
+    for c in driven:
+        assert O.cosine(outs["1"][1][c], ref["grad_Wa"][c]) >= GRAD_COS
+
+
 @pytest.mark.parametrize("T", [1, 2, 3, 32, 33, 64, 65])
 def test_sequence_length_edges_of_the_resident_kernels(T, gpu_device):
     """Sequence lengths around the kernels' internal boundaries (first/last step peeling, paired time steps,
