@@ -78,6 +78,31 @@ __device__ __forceinline__ void gates_stage(float* gl, const float* __restrict__
   }
 }
 
+// The same in two halves, for the time loops: the loads go into registers a step ahead (GATE_KMAX * 16 / 256
+// values per thread) and are written to LDS later in the step, when they have landed; a load followed at once
+// by its LDS store would wait for the load and, the memory counter being in order, for the acknowledgement of
+// every history store issued before it.
+constexpr int GATE_REGS = GATE_KMAX * 16 / 256;
+
+__device__ __forceinline__ void gates_fetch_regs(float (&gv)[GATE_REGS], const float* __restrict__ A, int k, int T, int B, int t,
+                                                 int bt, int tid) {
+#pragma unroll
+  for (int j = 0; j < GATE_REGS; ++j) {
+    const int idx = tid + 256 * j;
+    const int row = idx / k, c = idx - row * k, b = 16 * bt + row;
+    gv[j] = (idx < 16 * k && b < B) ? A[((size_t)b * T + t) * k + c] : 0.f;
+  }
+}
+
+__device__ __forceinline__ void gates_publish_regs(float* gl, const float (&gv)[GATE_REGS], int k, int tid) {
+#pragma unroll
+  for (int j = 0; j < GATE_REGS; ++j) {
+    const int idx = tid + 256 * j;
+    const int row = idx / k, c = idx - row * k;
+    if (idx < 16 * k) gl[row * GATE_KMAX + c] = gv[j];
+  }
+}
+
 // bit c set <=> channel c has a non-zero gate in some row; every wave computes the same mask
 // (over the rt gate tiles that follow each other at gl)
 __device__ __forceinline__ unsigned long long gates_active(const float* gl, int k, int lane, int rt = 1) {
@@ -272,16 +297,35 @@ __device__ __forceinline__ void read_rowsum(const float* psum, int q, float (&s)
 template <int NC, int RT>
 constexpr size_t stream_lds_bytes() { return (size_t)2 * RT * Tile<NC>::SLOTS * sizeof(bf16x8); }
 
+// Bytes of the packed weights (all matrices), and the copy of them into LDS by the whole workgroup.
+template <int NC>
+__host__ __device__ constexpr size_t packed_weight_bytes(int k) { return (size_t)(1 + k) * 4 * NC * Tile<NC>::KCH * 64 * sizeof(bf16x8); }
+
+template <int NC>
+__device__ __forceinline__ void weights_to_lds(bf16x8* wl, const bf16x8* __restrict__ Wp, int k, int tid) {
+  const int frags = (1 + k) * 4 * NC * Tile<NC>::KCH * 64;
+  for (int i = tid; i < frags; i += 256) wl[i] = Wp[i];
+}
+
 // With more than one batch tile per workgroup the forward keeps its fp32 state in LDS between steps
 // (one read and one write per lane and step) instead of in registers the weight pipeline needs.
 template <int NC, int RT>
 constexpr size_t fwd_state_lds_bytes() { return RT > 1 ? (size_t)RT * 4 * NC * 256 * sizeof(float) : 0; }
 
-template <int NC, int ACT, int RT>
+// WL: the packed weights of all 1 + a_dim matrices fit in LDS next to the operand buffers (small N): the workgroup
+// copies them there once and the per-step "stream" reads LDS instead of L2.
+template <int NC, int ACT, int RT, bool WL>
 __global__ __launch_bounds__(256) void ring_fwd_kernel(RingFwdArgs p) {
   using TL = Tile<NC>;
   extern __shared__ __attribute__((aligned(16))) char stream_lds[];
   bf16x8* const xbuf = reinterpret_cast<bf16x8*>(stream_lds);   // [2][RT][SLOTS]
+  static_assert(!WL || RT == 1, "LDS-resident weights go with one batch tile per workgroup");
+  const bf16x8* wsrc = (const bf16x8*)p.Wpack;
+  if constexpr (WL) {
+    bf16x8* wl = reinterpret_cast<bf16x8*>(stream_lds + stream_lds_bytes<NC, RT>());
+    weights_to_lds<NC>(wl, (const bf16x8*)p.Wpack, p.k, threadIdx.x);   // published by the barrier before the loop
+    wsrc = wl;
+  }
   __shared__ float psum[2][RT][64];
   __shared__ float gl[2][RT * 16 * GATE_KMAX];
 
@@ -332,13 +376,25 @@ __global__ __launch_bounds__(256) void ring_fwd_kernel(RingFwdArgs p) {
   for (int t = 0; t < T; ++t) {
     const int cur = t & 1;
     f32x4 acc[RT][NC];
-    if (staged && t + 1 < T) {
+    // next step's gates: loaded now, written to LDS after the products (nothing waits for them before that).
+    // Two paired tiles at the widest tiling have no registers to hold them and stage them in one go.
+    constexpr bool GATE_PIPE = !(NC == 8 && RT > 1);
+    float gv[RT][GATE_REGS];
+    const bool stage_next = staged && t + 1 < T;
+    if (stage_next) {
 #pragma unroll
-      for (int rt = 0; rt < RT; ++rt) gates_stage(gl[cur ^ 1] + rt * 16 * GATE_KMAX, p.A, p.k, T, B, t + 1, bt0 + rt, tid);
+      for (int rt = 0; rt < RT; ++rt) {
+        if constexpr (GATE_PIPE) gates_fetch_regs(gv[rt], p.A, p.k, T, B, t + 1, bt0 + rt, tid);
+        else gates_stage(gl[cur ^ 1] + rt * 16 * GATE_KMAX, p.A, p.k, T, B, t + 1, bt0 + rt, tid);
+      }
     }
-    gated_products<NC, false, RT>(xb(cur, 0), (const bf16x8*)p.Wpack, p.A, staged ? gl[cur] : nullptr,
+    gated_products<NC, false, RT>(xb(cur, 0), wsrc, p.A, staged ? gl[cur] : nullptr,
                                   staged ? gates_active(gl[cur], p.k, lane, RT) : ~0ull, p.k, T, B, t, b0, p.J1, w, lane,
                                   acc, wf, t > 0, t + 1 < T);
+    if (GATE_PIPE && stage_next) {
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) gates_publish_regs(gl[cur ^ 1] + rt * 16 * GATE_KMAX, gv[rt], p.k, tid);
+    }
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
       const int bq = b0 + 16 * rt;
@@ -449,13 +505,20 @@ __device__ __forceinline__ void bptt_flush_grad_A(const RingBpttArgs& p, const f
 // in dynamic shared memory) and are summed in wave order and written out after the next step's barrier.
 // LOSS: grad_output is not read; it is formed per element from the state history and the loss head's row
 // coefficients,  up * (kc cos(phi_i) + ks sin(phi_i) + beta sign(r_i)),  phi_i = 2 pi i / N,  up = upstream / (T * B).
-template <int NC, bool GA, int RT, bool LOSS>
+template <int NC, bool GA, int RT, bool LOSS, bool WL>
 __global__ __launch_bounds__(256) void ring_bptt_kernel(RingBpttArgs p) {
   static_assert(!GA || RT == 1, "dL/dA is produced one batch tile at a time");
+  static_assert(!WL || RT == 1, "LDS-resident weights go with one batch tile per workgroup");
   using TL = Tile<NC>;
   extern __shared__ __attribute__((aligned(16))) char stream_lds[];
   bf16x8* const xbuf = reinterpret_cast<bf16x8*>(stream_lds);                              // [2][RT][SLOTS]
   float* const ga_buf = reinterpret_cast<float*>(stream_lds + stream_lds_bytes<NC, RT>());  // [2][k][4 waves][16 rows] when GA
+  const bf16x8* wsrc = (const bf16x8*)p.Wpack;
+  if constexpr (WL) {   // behind the operand buffers and the dL/dA shares
+    bf16x8* wl = reinterpret_cast<bf16x8*>(stream_lds + stream_lds_bytes<NC, RT>() + (GA ? (size_t)2 * p.k * 64 * sizeof(float) : 0));
+    weights_to_lds<NC>(wl, (const bf16x8*)p.Wpack, p.k, threadIdx.x);   // published by the first step's barrier
+    wsrc = wl;
+  }
   __shared__ float psum[2][RT][64];
   __shared__ float gl[2][RT * 16 * GATE_KMAX];
 
@@ -495,8 +558,47 @@ __global__ __launch_bounds__(256) void ring_bptt_kernel(RingBpttArgs p) {
     up = (p.loss_upstream ? p.loss_upstream[0] : 1.f) * p.loss_inv_rows;
   }
 
-  // The weight pipeline restarts every step here: a step begins by waiting for grad_output and the saved
-  // record from HBM, which hides the refill, and carrying the buffers over would cost registers.
+  // A step's inputs -- grad_output (or, with the loss head fused in, the state rows and their coefficient
+  // records) and the saved F' record -- are loaded one step ahead into registers, right after the previous
+  // step consumed them, so that their HBM latency runs under that step's products.  (The variants of the widest
+  // tiling that have no registers left for that load at the top of the step.)
+  constexpr bool PREFETCH = NC <= 4 || (RT == 1 && !GA && !LOSS);
+  constexpr bool GATE_PIPE = PREFETCH;
+  struct StepIn {
+    float G[4][NC];
+    f16x4 d[NC];
+    ring_f32x4 cf[LOSS ? 4 : 1];
+  };
+  auto fetch_in = [&](int t, int rt, StepIn& in) {
+    rows_load<NC>((LOSS ? p.hist : p.grad_out) + (size_t)t * B * N, N, B, b0 + 16 * rt, i0, in.G);
+    if (bt0 + rt < p.nbt) {
+      const _Float16* src = p.dfrag + side_offset<NC>(t, p.nbt, bt0 + rt, w, lane);
+#pragma unroll
+      for (int c = 0; c < NC; ++c) in.d[c] = *reinterpret_cast<const f16x4*>(src + 4 * c);
+    } else {
+#pragma unroll
+      for (int c = 0; c < NC; ++c) in.d[c] = f16x4{(_Float16)0.f, (_Float16)0.f, (_Float16)0.f, (_Float16)0.f};
+    }
+    if constexpr (LOSS) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int b = b0 + 16 * rt + e;
+        in.cf[e] = p.loss_coef[(size_t)t * B + (b < B ? b : B - 1)];
+      }
+    }
+  };
+  StepIn in[RT];
+  float gv[RT][GATE_REGS];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    if constexpr (PREFETCH) fetch_in(T - 1, rt, in[rt]);
+    if (GATE_PIPE && staged) {
+      gates_fetch_regs(gv[rt], p.A, p.k, T, B, T - 1, bt0 + rt, tid);
+      gates_publish_regs(gl[0] + rt * 16 * GATE_KMAX, gv[rt], p.k, tid);   // published by the first step's barrier
+    }
+  }
+
+  // The weight pipeline restarts every step here; carrying its buffers over would cost registers.
   bf16x8 wf[StreamCfg<NC, RT>::PD][StreamCfg<NC, RT>::KG];
   for (int t = T - 1; t >= 0; --t) {
     const int cur = (T - 1 - t) & 1;
@@ -505,45 +607,43 @@ __global__ __launch_bounds__(256) void ring_bptt_kernel(RingBpttArgs p) {
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
       const bool live = bt0 + rt < p.nbt;
+      if constexpr (!PREFETCH) fetch_in(t, rt, in[rt]);
       float G[4][NC], g[4][NC];
-      rows_load<NC>((LOSS ? p.hist : p.grad_out) + (size_t)t * B * N, N, B, b0 + 16 * rt, i0, G);
-      if constexpr (LOSS) {   // G holds the state rows; columns past N get a finite value that meets F' = 0
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const int b = b0 + 16 * rt + e;
-          const ring_f32x4 cf = p.loss_coef[(size_t)t * B + (b < B ? b : B - 1)];
-          const float kc = cf[0] * up, ks = cf[1] * up, beta = cf[2] * up;
+      for (int e = 0; e < 4; ++e) {
+        float kc = 0.f, ks = 0.f, beta = 0.f;
+        if constexpr (LOSS) {
+          kc = in[rt].cf[e][0] * up;
+          ks = in[rt].cf[e][1] * up;
+          beta = in[rt].cf[e][2] * up;
+        }
 #pragma unroll
-          for (int c = 0; c < NC; ++c) {
-            const float r = G[e][c];
+        for (int c = 0; c < NC; ++c) {
+          float go = in[rt].G[e][c];
+          if constexpr (LOSS) {   // the rows are the state; columns past N get a finite value that meets F' = 0
+            const float r = go;
             const float sb = r > 0.f ? beta : (r < 0.f ? -beta : 0.f);          // beta * sign(r), sign(0) = 0
             const float co = CS_LDS ? cs_lds[(2 * c) * 256 + tid] : cs[c];
             const float si = CS_LDS ? cs_lds[(2 * c + 1) * 256 + tid] : sn[c];
-            G[e][c] = fmaf(kc, co, fmaf(ks, si, sb));
+            go = fmaf(kc, co, fmaf(ks, si, sb));
           }
-        }
-      }
-      if (live) {
-        side_load_f16<NC>(p.dfrag + side_offset<NC>(t, p.nbt, bt0 + rt, w, lane), g);
-      } else {
-#pragma unroll
-        for (int e = 0; e < 4; ++e)
-#pragma unroll
-          for (int c = 0; c < NC; ++c) g[e][c] = 0.f;
-      }
-#pragma unroll
-      for (int e = 0; e < 4; ++e)
-#pragma unroll
-        for (int c = 0; c < NC; ++c) {
-          G[e][c] += carry[rt][e][c];
-          g[e][c] = g[e][c] * G[e][c];   // the saved record already carries alpha
+          G[e][c] = go + carry[rt][e][c];
+          g[e][c] = (float)in[rt].d[c][e] * G[e][c];   // the saved record already carries alpha
           acc[rt][c][e] = oma * G[e][c];
         }
+      }
+      if constexpr (PREFETCH) {
+        if (t > 0) fetch_in(t - 1, rt, in[rt]);
+      }
+      // the gates of the next step (t - 1): loaded now, written to LDS after the products
+      if constexpr (GATE_PIPE) {
+        if (staged && t > 0) gates_fetch_regs(gv[rt], p.A, p.k, T, B, t - 1, bt0 + rt, tid);
+      } else {
+        if (staged) gates_stage(gl[cur] + rt * 16 * GATE_KMAX, p.A, p.k, T, B, t, bt0 + rt, tid);
+      }
       write_operand<NC>(xb(cur, rt), g, w, q, n);
       publish_rowsum<NC>(psum[cur][rt], g, w, q, n);
       if (live) pair_store<NC>(p.gfrag, t, p.nbt, bt0 + rt, w, lane, g);
-      // this step's gates: the buffer was last read two steps ago, before the previous barrier
-      if (staged) gates_stage(gl[cur] + rt * 16 * GATE_KMAX, p.A, p.k, T, B, t, bt0 + rt, tid);
     }
     lds_barrier();
     const float* glt = staged ? gl[cur] : nullptr;
@@ -554,14 +654,16 @@ __global__ __launch_bounds__(256) void ring_bptt_kernel(RingBpttArgs p) {
       if (t + 1 < T) bptt_flush_grad_A(p, ga_buf + (cur ^ 1) * p.k * 64, t + 1, bt0, tid);
       float rp[4][NC];
       rows_load<NC>(t == 0 ? p.r_init : p.hist + (size_t)(t - 1) * B * N, N, B, b0, i0, rp);
-      gated_products<NC, true, 1>(xb(cur, 0), (const bf16x8*)p.Wpack, p.A, glt, active, p.k, T, B, t, b0, p.J1, w, lane,
+      gated_products<NC, true, 1>(xb(cur, 0), wsrc, p.A, glt, active, p.k, T, B, t, b0, p.J1, w, lane,
                                   acc, wf, false, false, rp, ga_buf + cur * p.k * 64, true);
     } else {
-      gated_products<NC, false, RT>(xb(cur, 0), (const bf16x8*)p.Wpack, p.A, glt, active, p.k, T, B, t, b0, p.J1, w,
+      gated_products<NC, false, RT>(xb(cur, 0), wsrc, p.A, glt, active, p.k, T, B, t, b0, p.J1, w,
                                     lane, acc, wf, false, false, nullptr, nullptr, true);
     }
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
+      // the other gate buffer was last read during the previous step's products, before this step's barrier
+      if (GATE_PIPE && staged && t > 0) gates_publish_regs(gl[cur ^ 1] + rt * 16 * GATE_KMAX, gv[rt], p.k, tid);
       float s[4];
       read_rowsum(psum[cur][rt], q, s);
 #pragma unroll
@@ -860,13 +962,28 @@ static hipError_t launch_stream(K kern, dim3 grid, size_t dyn, hipStream_t st, c
   if ((RTv) == 2) { constexpr int RT = 2; if constexpr (NC >= 4) { CALL; } } \
   else { constexpr int RT = 1; CALL; }
 
+// LDS-resident weights for the streaming kernels: everything must fit next to the operand buffers, the gate
+// stage and (BPTT with dL/dA) the per-wave shares.  RINGATTR_LDS_WEIGHTS=0 keeps the weights in L2 (tests).
+static bool weights_fit_lds(int NCv, int k, size_t other_dynamic) {
+  if (NCv > 2) return false;
+  const char* v = getenv("RINGATTR_LDS_WEIGHTS");
+  if (v && v[0] == '0') return false;
+  const size_t wb = NCv == 1 ? packed_weight_bytes<1>(k) : packed_weight_bytes<2>(k);
+  return wb + other_dynamic + 20 * 1024 <= 128 * 1024;   // 20 KiB: static LDS of these kernels, rounded up
+}
+
 hipError_t ring_launch_fwd(const RingFwdArgs& a, int NCv, hipStream_t st) {
   ProfScope prof(1, st);
   if (ring_uses_resident(a.N, a.k)) return ring_launch_fwd_res256(a, st);
   const int rt = stream_row_tiles(NCv, a.nbt, false);
   hipError_t e = hipErrorInvalidValue;
+  if (weights_fit_lds(NCv, a.k, 8 * 1024)) {
+    RING_DISPATCH_NC(NCv, RING_DISPATCH_ACT(a.act, if constexpr (NC <= 2)
+        e = launch_stream(ring_fwd_kernel<NC, ACT, 1, true>, dim3(a.nbt), stream_lds_bytes<NC, 1>() + packed_weight_bytes<NC>(a.k), st, a)));
+    return e;
+  }
   RING_DISPATCH_NC(NCv, RING_DISPATCH_ACT(a.act, RING_DISPATCH_RT(rt,
-      e = launch_stream(ring_fwd_kernel<NC, ACT, RT>, dim3((a.nbt + RT - 1) / RT),
+      e = launch_stream(ring_fwd_kernel<NC, ACT, RT, false>, dim3((a.nbt + RT - 1) / RT),
                         stream_lds_bytes<NC, RT>() + fwd_state_lds_bytes<NC, RT>(), st, a))));
   return e;
 }
@@ -888,28 +1005,35 @@ hipError_t ring_launch_rebuild(const RingFwdArgs& a, int NCv, hipStream_t st) {
   return e;
 }
 
+template <int NC, bool GA, int RT, bool WL>
+static hipError_t launch_bptt_stream(const RingBpttArgs& a, dim3 grid, size_t dyn, hipStream_t st) {
+  return a.loss_coef ? launch_stream(ring_bptt_kernel<NC, GA, RT, true, WL>, grid, dyn, st, a)
+                     : launch_stream(ring_bptt_kernel<NC, GA, RT, false, WL>, grid, dyn, st, a);
+}
+
 hipError_t ring_launch_bptt(const RingBpttArgs& a, int NCv, hipStream_t st) {
   ProfScope prof(3, st);
   hipError_t e = hipErrorInvalidValue;
-  const bool loss = a.loss_coef != nullptr;
+  // (the parentheses keep the commas of the template argument lists away from the dispatch macros)
   if (a.grad_A) {   // the generic kernel is the one that also produces dL/dA
     const size_t ga = (size_t)2 * a.k * 64 * sizeof(float);
-    if (loss) {
-      RING_DISPATCH_NC(NCv, e = launch_stream(ring_bptt_kernel<NC, true, 1, true>, dim3(a.nbt), stream_lds_bytes<NC, 1>() + ga, st, a));
+    if (weights_fit_lds(NCv, a.k, 8 * 1024 + ga)) {
+      RING_DISPATCH_NC(NCv, if constexpr (NC <= 2) (e = launch_bptt_stream<NC, true, 1, true>(
+          a, dim3(a.nbt), stream_lds_bytes<NC, 1>() + ga + packed_weight_bytes<NC>(a.k), st)));
     } else {
-      RING_DISPATCH_NC(NCv, e = launch_stream(ring_bptt_kernel<NC, true, 1, false>, dim3(a.nbt), stream_lds_bytes<NC, 1>() + ga, st, a));
+      RING_DISPATCH_NC(NCv, (e = launch_bptt_stream<NC, true, 1, false>(a, dim3(a.nbt), stream_lds_bytes<NC, 1>() + ga, st)));
     }
     return e;
   }
   if (ring_uses_resident(a.N, a.k)) return ring_launch_bptt_res256(a, st);
-  const int rt = stream_row_tiles(NCv, a.nbt, false);
-  if (loss) {
-    RING_DISPATCH_NC(NCv, RING_DISPATCH_RT(rt,
-        e = launch_stream(ring_bptt_kernel<NC, false, RT, true>, dim3((a.nbt + RT - 1) / RT), stream_lds_bytes<NC, RT>(), st, a)));
-  } else {
-    RING_DISPATCH_NC(NCv, RING_DISPATCH_RT(rt,
-        e = launch_stream(ring_bptt_kernel<NC, false, RT, false>, dim3((a.nbt + RT - 1) / RT), stream_lds_bytes<NC, RT>(), st, a)));
+  if (weights_fit_lds(NCv, a.k, 8 * 1024)) {
+    RING_DISPATCH_NC(NCv, if constexpr (NC <= 2) (e = launch_bptt_stream<NC, false, 1, true>(
+        a, dim3(a.nbt), stream_lds_bytes<NC, 1>() + packed_weight_bytes<NC>(a.k), st)));
+    return e;
   }
+  const int rt = stream_row_tiles(NCv, a.nbt, false);
+  RING_DISPATCH_NC(NCv, RING_DISPATCH_RT(rt, (e = launch_bptt_stream<NC, false, RT, false>(
+      a, dim3((a.nbt + RT - 1) / RT), stream_lds_bytes<NC, RT>(), st))));
   return e;
 }
 
