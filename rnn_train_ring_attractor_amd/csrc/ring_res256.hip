@@ -356,6 +356,18 @@ __device__ __forceinline__ f32x4 async_load16(const void* ptr) {
   return v;
 }
 
+// The same load addressed as a wave-uniform base (scalar registers) plus a 32-bit per-lane byte offset plus an
+// immediate: the per-step address arithmetic then runs on the scalar unit and costs the vector ALU nothing.
+template <int IMM>
+__device__ __forceinline__ f32x4 async_load16_s(const void* uniform_base, unsigned lane_off) {
+  f32x4 v;
+  asm volatile(".Lring_async_load_%=:\n\tglobal_load_dwordx4 %0, %1, %2 offset:%3"
+               : "=&v"(v)
+               : "v"(lane_off), "s"(uniform_base), "n"(IMM)
+               : "memory");
+  return v;
+}
+
 template <int K, bool LOSS>
 __device__ __forceinline__ void bptt_stage_wait(BpttStage& s) {
   if constexpr (LOSS) {
@@ -379,16 +391,30 @@ __device__ __forceinline__ void bptt_stage_load(const RingBpttArgs& p, int t, in
   const _Float16* drec = p.dfrag + side_offset<R_NC>(t, p.nbt, bt, w, lane);
   const float* rows = LOSS ? p.hist : p.grad_out;
   if constexpr (FULL) {
-    const float* grow = rows + ((size_t)t * p.B + b0) * p.N + i0;
-#pragma unroll
-    for (int e = 0; e < 4; ++e) s.G[e] = async_load16(grow + (size_t)e * p.N);
-    s.D[0] = async_load16(drec);
-    s.D[1] = async_load16(drec + 8);
+    // FULL: N == 256 and whole batch tiles, so row e of the lane's four sits e KiB after row 0
+    const int q = lane >> 4, n = lane & 15;
+    const int ws = __builtin_amdgcn_readfirstlane(w);
+    const float* gtile = rows + ((size_t)t * p.B + 16 * bt) * 256;                      // uniform: the tile's 16 rows
+    const unsigned goff = (unsigned)((4 * q * 256 + 16 * R_NC * ws + R_NC * n) * sizeof(float));
+    s.G[0] = async_load16_s<0>(gtile, goff);
+    s.G[1] = async_load16_s<1024>(gtile, goff);
+    s.G[2] = async_load16_s<2048>(gtile, goff);
+    s.G[3] = async_load16_s<3072>(gtile, goff);
+    const _Float16* dtile = p.dfrag + side_offset<R_NC>(t, p.nbt, bt, ws, 0);           // uniform: the wave's record block
+    const unsigned doff = (unsigned)lane * (4 * R_NC * sizeof(_Float16));
+    s.D[0] = async_load16_s<0>(dtile, doff);
+    s.D[1] = async_load16_s<16>(dtile, doff);
     if constexpr (LOSS) {
-      const ring_f32x4* crow = p.loss_coef + (size_t)t * p.B + b0;
-#pragma unroll
-      for (int e = 0; e < 4; ++e) s.C[e] = async_load16(crow + e);
+      const ring_f32x4* ctile = p.loss_coef + (size_t)t * p.B + 16 * bt;                  // uniform: the tile's 16 records
+      const unsigned coff = (unsigned)(4 * q) * sizeof(ring_f32x4);
+      s.C[0] = async_load16_s<0>(ctile, coff);
+      s.C[1] = async_load16_s<16>(ctile, coff);
+      s.C[2] = async_load16_s<32>(ctile, coff);
+      s.C[3] = async_load16_s<48>(ctile, coff);
     }
+    (void)drec;
+    (void)b0;
+    (void)i0;
   } else {
     float G[4][R_NC];
     rows_load<R_NC>(rows + (size_t)t * p.B * p.N, p.N, p.B, b0, i0, G);
@@ -430,6 +456,7 @@ __global__ __launch_bounds__(256) void ring_bptt_res256_kernel(RingBpttArgs p) {
   const int i0 = 16 * R_NC * w + R_NC * n;
   const int N = p.N, B = p.B, T = p.T;
   const float oma = 1.f - p.alpha, J0 = p.J0;   // alpha rides in the saved F' record, J1 in the packed Wo fragments
+  const int wu = __builtin_amdgcn_readfirstlane(w);   // the wave index as a scalar, for address arithmetic
 
   bf16x8 wreg[2][R_NC][R_KCH];
   bf16x8* wl = wlds + (size_t)w * R_NC * R_KCH * 64 + lane;
@@ -504,12 +531,21 @@ __global__ __launch_bounds__(256) void ring_bptt_res256_kernel(RingBpttArgs p) {
             go = fmaf(kc, cs[c], fmaf(ks, sn[c], sb));
           }
           G[e][c] = go + carry[e][c];
-          g[e][c] = stage_dact(S, e, c) * G[e][c];
+          g[e][c] = __builtin_fmaf(stage_dact(S, e, c), G[e][c], 0.f);   // one mixed-precision FMA: the fp16 record is an operand as it is
         }
       }
       bf16x8* xb = xbuf + cur * R_XSLOTS;
       write_operand<R_NC>(xb, g, w, q, n);
-      pair_store<R_NC>(p.gfrag, t, p.nbt, bt, w, lane, g);
+      {
+        // pair_store with the address split into a wave-uniform base and the lane's slot: tile w*NC + c is c KiB on
+        char* gt = reinterpret_cast<char*>(p.gfrag + pair_offset<R_NC>(t, p.nbt, bt, wu * R_NC, 0));
+        const unsigned goff = (unsigned)lane * 16u;
+#pragma unroll
+        for (int c = 0; c < R_NC; ++c) {
+          const bf16x4 pk = {(__bf16)g[0][c], (__bf16)g[1][c], (__bf16)g[2][c], (__bf16)g[3][c]};
+          *reinterpret_cast<bf16x4*>(gt + c * 1024 + goff) = pk;
+        }
+      }
       bptt_stage_load<FULL, LOSS>(p, t - R_BPTT_DEPTH, bt, w, lane, b0, i0, S);
       lds_barrier();
 
