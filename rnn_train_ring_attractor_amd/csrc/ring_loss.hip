@@ -90,11 +90,14 @@ __global__ __launch_bounds__(256) void ring_loss_stats_kernel(const float* __res
   RowLanes<NCH> ph;
   ph.init(N, lane);
   const long rows = (long)T * B;
-  // two rows per trip, so that two row loads are in flight per wave
+  // two rows per trip, so that two row loads are in flight per wave.  The sweep runs from the last row to the
+  // first: the forward kernel has just written the history in time order, so its tail is what the memory-side
+  // cache still holds.
   const long stride = (long)gridDim.x * L_ROWS_PER_BLOCK;
-  for (long row = (long)blockIdx.x * L_ROWS_PER_BLOCK + wv; row < rows; row += 2 * stride) {
-    const long row2 = row + stride;
-    const bool has2 = row2 < rows;
+  for (long it = (long)blockIdx.x * L_ROWS_PER_BLOCK + wv; it < rows; it += 2 * stride) {
+    const long row = rows - 1 - it;
+    const long row2 = row - stride;
+    const bool has2 = row2 >= 0;
     float v[2][NCH][4];
     row_load<NCH, VEC>(hist + row * N, N, lane, v[0]);
     row_load<NCH, VEC>(hist + (has2 ? row2 : row) * N, N, lane, v[1]);
