@@ -358,10 +358,12 @@ __device__ __forceinline__ f32x4 async_load16(const void* ptr) {
 
 // The same load addressed as a wave-uniform base (scalar registers) plus a 32-bit per-lane byte offset plus an
 // immediate: the per-step address arithmetic then runs on the scalar unit and costs the vector ALU nothing.
+// Non-temporal: grad_output and the saved record are read exactly once, and what should stay in the caches
+// is the operand copy this kernel writes for the weight-gradient kernel that follows.
 template <int IMM>
 __device__ __forceinline__ f32x4 async_load16_s(const void* uniform_base, unsigned lane_off) {
   f32x4 v;
-  asm volatile(".Lring_async_load_%=:\n\tglobal_load_dwordx4 %0, %1, %2 offset:%3"
+  asm volatile(".Lring_async_load_%=:\n\tglobal_load_dwordx4 %0, %1, %2 offset:%3 nt"
                : "=&v"(v)
                : "v"(lane_off), "s"(uniform_base), "n"(IMM)
                : "memory");
