@@ -36,12 +36,21 @@ struct Tile {
 // of landing 8-way on the same ones.
 constexpr int XG = 17;
 
-// Contraction order of the pipelined NC = 4 kernels: positions 0..127 hold, wave by wave, the neurons
-// of column tiles 0,1 ("early" pair) and positions 128..255 those of tiles 2,3 ("late" pair), so a
-// wave's tile pair lands in one K chunk: position 128*h + 32*w + 2*n + cc <-> neuron 64*w + 4*n + 2*h + cc.
+// Neuron ownership of the pipelined NC = 4 forward.  Its eight waves (w = 0..3, h = 0 "early" / 1 "late") each
+// own two column tiles; tile cc, column n of wave (w,h) is neuron 64*w + 32*h + 2*n + cc, so the 16 lanes of an
+// MFMA row group hold 32 consecutive neurons and a history store writes whole 128-byte lines.  The contraction
+// index follows the same order, early waves first: position 128*h + 32*w + 2*n + cc <-> that neuron, which puts
+// a wave's tile pair into one K chunk.  (The saved buffers keep the common tile order; see split_common_slot.)
 __host__ __device__ __forceinline__ int split_k_neuron(int kappa) {
   const int h = kappa >> 7, s = kappa & 127;
-  return 64 * (s >> 5) + 4 * ((s & 31) >> 1) + 2 * h + (s & 1);
+  return 64 * (s >> 5) + 32 * h + (s & 31);
+}
+
+// Where the common tile order (tile c, column n <-> neuron 64*w + 4*n + c) keeps neuron 64*w + 32*h + 2*n + cc:
+// column 8*h + n/2 of tile 2*(n%2) + cc.
+__host__ __device__ __forceinline__ void split_common_slot(int h, int n, int cc, int& tile, int& col) {
+  tile = 2 * (n & 1) + cc;
+  col = 8 * h + (n >> 1);
 }
 
 // D = A(16x32 bf16) * B(32x16 bf16) + C(16x16 fp32).  Lane (q,n): A row n, B column n, both with

@@ -14,8 +14,8 @@
 //   contraction indices 32kc+8q .. +7.  transposed = 0: value = W[col][contr] (forward, re = W r);
 //   transposed = 1: value = W[contr][col] (backward, g @ W).
 //   scale0 multiplies matrix 0 (Wo) before rounding: kernels that fold J1 into the weights pass J1.
-//   split_k = 1 (NC = 4 only): contraction position kappa stands for neuron split_k_neuron(kappa), the
-//   order the pipelined weight-resident kernels keep their operand tile in.
+//   split_k = 1 (NC = 4 only): contraction position kappa stands for neuron split_k_neuron(kappa) and output
+//   column n of tile c for neuron 64*w + 32*(c/2) + 2*n + c%2: the pipelined weight-resident forward's order.
 // ------------------------------------------------------------------------------------------------
 __device__ __forceinline__ bf16x8 pack_fragment(const float* __restrict__ Wo, const float* __restrict__ Wa, size_t u,
                                                 int N, int NC, int transposed, int split_k, float scale0) {
@@ -29,7 +29,8 @@ __device__ __forceinline__ bf16x8 pack_fragment(const float* __restrict__ Wo, co
   const int w = (int)(v & 3);
   const int mm = (int)(v >> 2);
   const int q = lane >> 4, n = lane & 15;
-  const int col = 16 * NC * w + NC * n + c;
+  // split_k: the output columns follow the pipelined forward's ownership as well (tile c = 2*h + cc of wave w)
+  const int col = split_k ? 64 * w + 32 * (c >> 1) + 2 * n + (c & 1) : 16 * NC * w + NC * n + c;
   const int k0 = 32 * kc + 8 * q;
   const float* W = (mm == 0) ? Wo : Wa + (size_t)(mm - 1) * N * N;
   bf16x8 pk;

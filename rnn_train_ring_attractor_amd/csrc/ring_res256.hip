@@ -79,7 +79,8 @@ __device__ __forceinline__ void load_resident(const bf16x8* Wp, bf16x8* wl, bf16
 // is several hundred of them.  So the workgroup runs EIGHT waves, two per SIMD, in two roles that
 // are half a step out of phase: while one wave of a SIMD is in its vector-ALU epilogue the other one
 // feeds the matrix pipe.  Wave (w, h), w = 0..3, h = 0/1, owns column tiles 2h and 2h+1 of neuron
-// group w (neurons 64w + 4n + 2h + {0,1}); h = 0 is the "early" role E, h = 1 the "late" role L.  The
+// group w (neurons 64w + 32h + 2n + {0,1}: a row group's 16 lanes cover 32 consecutive neurons, so a history
+// store fills whole cache lines); h = 0 is the "early" role E, h = 1 the "late" role L.  The
 // contraction index is ordered so that K chunks 0..3 hold the E neurons and 4..7 the L neurons
 // (split_k_neuron), and the step t (r_t -> r_{t+1}) is
 //      barrier A_t   (r^E_t visible)
@@ -134,7 +135,9 @@ __global__ __launch_bounds__(512) void ring_fwd_res256_kernel(RingFwdArgs p) {
   const int tid = threadIdx.x, w8 = tid >> 6, h = w8 >> 2, w = w8 & 3, lane = tid & 63, q = lane >> 4, n = lane & 15;
   const int bt = blockIdx.x;
   const int b0 = 16 * bt + 4 * q;
-  const int i0 = 16 * R_NC * w + R_NC * n + 2 * h;
+  const int i0 = 64 * w + 32 * h + 2 * n;         // this lane's two neurons: i0, i0 + 1 (one per tile)
+  // their slots in the common tile order of the saved buffers: tile ct0 + cc, lane lc (same row group q)
+  const int ct0 = 2 * (n & 1), lc = (lane & 48) | (8 * h + (n >> 1));
   const int N = p.N, B = p.B, T = p.T;
   const float oma = 1.f - p.alpha, alpha = p.alpha, J0 = p.J0, J1 = p.J1;
   constexpr int HK = R_KCH / 2;
@@ -159,7 +162,7 @@ __global__ __launch_bounds__(512) void ring_fwd_res256_kernel(RingFwdArgs p) {
 #pragma unroll
     for (int cc = 0; cc < 2; ++cc) {
       bf16x4 pk = {(__bf16)r[0][cc], (__bf16)r[1][cc], (__bf16)r[2][cc], (__bf16)r[3][cc]};
-      *reinterpret_cast<bf16x4*>(p.rfrag + pair_offset<R_NC>(t, p.nbt, bt, w * R_NC + 2 * h + cc, lane)) = pk;
+      *reinterpret_cast<bf16x4*>(p.rfrag + pair_offset<R_NC>(t, p.nbt, bt, w * R_NC + ct0 + cc, lc)) = pk;
     }
   };
   write_half(h ? xL : xE, r, w, q, n);
@@ -169,7 +172,7 @@ __global__ __launch_bounds__(512) void ring_fwd_res256_kernel(RingFwdArgs p) {
       const bf16x4 z = {(__bf16)0.f, (__bf16)0.f, (__bf16)0.f, (__bf16)0.f};
 #pragma unroll
       for (int cc = 0; cc < 2; ++cc)
-        *reinterpret_cast<bf16x4*>(p.rfrag + pair_offset<R_NC>(T, p.nbt, bt, w * R_NC + 2 * h + cc, lane)) = z;
+        *reinterpret_cast<bf16x4*>(p.rfrag + pair_offset<R_NC>(T, p.nbt, bt, w * R_NC + ct0 + cc, lc)) = z;
     }
   }
   GateStage gs;
@@ -207,14 +210,14 @@ __global__ __launch_bounds__(512) void ring_fwd_res256_kernel(RingFwdArgs p) {
     } else if (slot < 6) {
       if (SAVE) {
         const int cc = slot - 4;
-        _Float16* drec = p.dfrag + side_offset<R_NC>(t, p.nbt, bt, w, lane) + 8 * h + 4 * cc;
+        _Float16* drec = p.dfrag + side_offset<R_NC>(t, p.nbt, bt, w, lc) + 4 * (ct0 + cc);
         const f16x4 pk = {(_Float16)d[0][cc], (_Float16)d[1][cc], (_Float16)d[2][cc], (_Float16)d[3][cc]};
         *reinterpret_cast<f16x4*>(drec) = pk;
       }
     } else if (SAVE) {
       const int cc = slot - 6;   // r after step t is the operand of step t+1
       bf16x4 pk = {(__bf16)r[0][cc], (__bf16)r[1][cc], (__bf16)r[2][cc], (__bf16)r[3][cc]};
-      *reinterpret_cast<bf16x4*>(p.rfrag + pair_offset<R_NC>(t + 1, p.nbt, bt, w * R_NC + 2 * h + cc, lane)) = pk;
+      *reinterpret_cast<bf16x4*>(p.rfrag + pair_offset<R_NC>(t + 1, p.nbt, bt, w * R_NC + ct0 + cc, lc)) = pk;
     }
     __builtin_amdgcn_sched_barrier(0);
   };
