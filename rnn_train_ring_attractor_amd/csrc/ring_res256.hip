@@ -448,8 +448,12 @@ __device__ __forceinline__ float stage_dact(const BpttStage& s, int e, int c) {
 // LOSS: grad_output is not read; it is formed per element from the state history and the loss head's row
 // coefficients,  up * (kc cos(phi_i) + ks sin(phi_i) + beta sign(r_i)),  phi_i = 2 pi i / N,
 // up = upstream / (T * B)  (what ring_loss_grad_kernel would have written to HBM for this kernel to read back).
-template <bool FULL, bool LOSS>
+// MERGE (needs FULL and an even T): the operand copy of g pairs time steps 2j and 2j+1 in one 16-byte slot per
+// lane; the kernel walks down through 2j+1 and 2j in one trip of its unrolled loop, keeps the first in registers
+// and writes both with one 16-byte store per tile (whole cache lines, half as many store instructions).
+template <bool FULL, bool LOSS, bool MERGE>
 __global__ __launch_bounds__(256) void ring_bptt_res256_kernel(RingBpttArgs p) {
+  static_assert(!MERGE || (FULL && R_BPTT_DEPTH == 2), "merged pair stores need the unmasked two-step loop");
   extern __shared__ __attribute__((aligned(16))) char smem[];
   bf16x8* wlds = reinterpret_cast<bf16x8*>(smem);
   bf16x8* xbuf = wlds + R_WLDS_SLOTS;
@@ -503,6 +507,7 @@ __global__ __launch_bounds__(256) void ring_bptt_res256_kernel(RingBpttArgs p) {
   for (int u = 0; u < R_KCH / 2; ++u) w0[0][u] = wl[u * 64];
   // (the first lds_barrier inside the loop also publishes the gates)
 
+  bf16x4 held[R_NC];   // MERGE: the odd step's bf16 g, waiting for its even partner
   for (int u0 = 0; u0 < T; u0 += R_BPTT_DEPTH) {
 #pragma unroll
     for (int half = 0; half < R_BPTT_DEPTH; ++half) {
@@ -516,7 +521,15 @@ __global__ __launch_bounds__(256) void ring_bptt_res256_kernel(RingBpttArgs p) {
       // stage's six loads.  The counter is in order, so "at most 10 * (depth - 1) outstanding" means this
       // stage landed; a smaller number would also wait for later loads and for store acknowledgements.
       // (with the loss head fused in a stage has four more loads: 14 per step)
-      if constexpr (FULL) bptt_stage_wait<(LOSS ? 14 : 10) * (R_BPTT_DEPTH - 1), LOSS>(S);
+      // With merged pair stores the four stores all sit in the second step of a trip: the first step's stage
+      // sees them and the other stage's loads behind it, the second step's stage only the other stage's loads.
+      if constexpr (MERGE) {
+        constexpr int LOADS = LOSS ? 10 : 6;
+        if (half == 0) bptt_stage_wait<LOADS + 4, LOSS>(S);
+        else bptt_stage_wait<LOADS, LOSS>(S);
+      } else if constexpr (FULL) {
+        bptt_stage_wait<(LOSS ? 14 : 10) * (R_BPTT_DEPTH - 1), LOSS>(S);
+      }
 
       float G[4][R_NC], g[4][R_NC];
 #pragma unroll
@@ -548,7 +561,16 @@ __global__ __launch_bounds__(256) void ring_bptt_res256_kernel(RingBpttArgs p) {
 #pragma unroll
         for (int c = 0; c < R_NC; ++c) {
           const bf16x4 pk = {(__bf16)g[0][c], (__bf16)g[1][c], (__bf16)g[2][c], (__bf16)g[3][c]};
-          *reinterpret_cast<bf16x4*>(gt + c * 1024 + goff) = pk;
+          if constexpr (MERGE) {
+            if (half == 0) {
+              held[c] = pk;            // t is odd here (T even): the slot's second half, written with the first
+            } else {
+              const bf16x8 both = __builtin_shufflevector(pk, held[c], 0, 1, 2, 3, 4, 5, 6, 7);
+              *reinterpret_cast<bf16x8*>(gt + c * 1024 + goff) = both;
+            }
+          } else {
+            *reinterpret_cast<bf16x4*>(gt + c * 1024 + goff) = pk;
+          }
         }
       }
       bptt_stage_load<FULL, LOSS>(p, t - R_BPTT_DEPTH, bt, w, lane, b0, i0, S);
@@ -642,9 +664,9 @@ hipError_t ring_launch_fwd_res256(const RingFwdArgs& a, hipStream_t st) {
   }
 }
 
-template <bool FULL, bool LOSS>
+template <bool FULL, bool LOSS, bool MERGE>
 static hipError_t launch_bptt_variant(const RingBpttArgs& a, hipStream_t st) {
-  auto kern = ring_bptt_res256_kernel<FULL, LOSS>;
+  auto kern = ring_bptt_res256_kernel<FULL, LOSS, MERGE>;
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                                      (int)R_LDS_BYTES);
   if (e != hipSuccess) return e;
@@ -654,6 +676,11 @@ static hipError_t launch_bptt_variant(const RingBpttArgs& a, hipStream_t st) {
 
 hipError_t ring_launch_bptt_res256(const RingBpttArgs& a, hipStream_t st) {
   const bool full = (a.N == 256) && (a.B % 16 == 0);
-  if (a.loss_coef) return full ? launch_bptt_variant<true, true>(a, st) : launch_bptt_variant<false, true>(a, st);
-  return full ? launch_bptt_variant<true, false>(a, st) : launch_bptt_variant<false, false>(a, st);
+  const bool merge = full && (a.T % 2 == 0);
+  if (a.loss_coef) {
+    if (merge) return launch_bptt_variant<true, true, true>(a, st);
+    return full ? launch_bptt_variant<true, true, false>(a, st) : launch_bptt_variant<false, true, false>(a, st);
+  }
+  if (merge) return launch_bptt_variant<true, false, true>(a, st);
+  return full ? launch_bptt_variant<true, false, false>(a, st) : launch_bptt_variant<false, false, false>(a, st);
 }

@@ -238,13 +238,15 @@ def test_silent_action_channels_are_compacted(driven, gpu_device, monkeypatch):
         assert O.cosine(outs["1"][1][c], ref["grad_Wa"][c]) >= GRAD_COS
 
 
+@pytest.mark.parametrize("B", [17, 32], ids=["ragged_batch", "whole_tiles"])
 @pytest.mark.parametrize("T", [1, 2, 3, 32, 33, 64, 65])
-def test_sequence_length_edges_of_the_resident_kernels(T, gpu_device):
-    """Sequence lengths around the kernels' internal boundaries (first/last step peeling, paired time steps,
-    gate chunks of 32 steps) with a ragged batch, forward and backward."""
+def test_sequence_length_edges_of_the_resident_kernels(T, B, gpu_device):
+    """Sequence lengths around the kernels' internal boundaries (first/last step peeling, paired time steps and
+    their merged stores at even lengths, gate chunks of 32 steps) with a ragged batch (masked kernels) and with
+    whole batch tiles (unmasked kernels), forward and backward."""
     from rnn_train_ring_attractor_amd import ring_rnn_cuda_func
-    B, k, N = 17, 2, 256
-    print(f"[case] sequence edge T={T}", flush=True)
+    k, N = 2, 256
+    print(f"[case] sequence edge T={T} B={B}", flush=True)
     p = make_problem(50 + T, B, T, k, N)
     Wa = _t(p["Wa"], gpu_device).requires_grad_(True)
     Wo = _t(p["Wo"], gpu_device).requires_grad_(True)
