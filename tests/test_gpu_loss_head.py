@@ -121,3 +121,30 @@ def test_time_loop_and_loss_as_one_operator(B, T, k, N, act, own, streaming, wei
     for got, key in ((f[4], "grad_Wo"), (f[5], "grad_Wa"), (f[6], "grad_r_init")):
         assert O.cosine(got, ref[key]) >= 0.999, key
         assert O.max_rel_err(got, ref[key]) <= 2e-2, key
+
+
+@pytest.mark.parametrize("B,T,k,N,act", [(24, 8, 2, 120, "tanh"), (20, 6, 2, 256, "gelu"), (18, 5, 3, 300, "silu")],
+                         ids=["n120", "n256", "n300_k3"])
+def test_one_operator_also_returns_the_action_signal_gradient(B, T, k, N, act, gpu_device):
+    """dL/d action_signal and dL/d r_init through ring_rnn_loss_func (loss gradient formed inside the BPTT kernel
+    that also produces dL/dA) against ring_rnn_cuda_func + ring_loss_pair."""
+    from rnn_train_ring_attractor_amd import ring_loss_pair, ring_rnn_cuda_func, ring_rnn_loss_func
+    from tests.ring_cases import make_problem
+    print(f"[case] one operator with grad_A B={B} T={T} k={k} N={N} {act}", flush=True)
+    p = make_problem(500 + N, B, T, k, N, action="dense")
+    t = lambda x: torch.tensor(np.ascontiguousarray(x), device=gpu_device)
+    angle = t((np.random.default_rng(9).random((B, T)) * 2 * np.pi).astype(np.float32))
+    res = {}
+    for fused in (True, False):
+        A, r0 = t(p["A"]).requires_grad_(True), t(p["r0"]).requires_grad_(True)
+        Wa, Wo = t(p["Wa"]).requires_grad_(True), t(p["Wo"]).requires_grad_(True)
+        if fused:
+            total = ring_rnn_loss_func(A, Wa, -0.1, 0.1, Wo, r0, 0.15, act, angle, 0.2)[0]
+        else:
+            total = ring_loss_pair(ring_rnn_cuda_func(A, Wa, -0.1, 0.1, Wo, r0, 0.15, act), angle, 0.2)[0]
+        total.backward()
+        torch.cuda.synchronize()
+        res[fused] = [x.grad.cpu().numpy() for x in (A, r0, Wa, Wo)]
+    for a, b in zip(res[True], res[False]):
+        assert np.isfinite(a).all() and np.abs(b).max() > 0
+        assert O.max_rel_err(a, b) <= 2e-3 and O.cosine(a, b) >= 0.99999
