@@ -82,11 +82,13 @@ RINGATTR_API int ringattr_fwd(const void* A, const void* Wa, float J0, float J1,
  * grad_A [B,T,k] and grad_r_init [B,N] are optional outputs (NULL = skip), written
  * rather than accumulated; the reference returns None for both
  * (cpp/ring_rnn_cuda.py:144).  Asking for grad_A (a_dim <= 48) adds one read of
- * bump_history and runs the BPTT on the weight-streaming kernel for every N. */
+ * bump_history and runs the BPTT on the weight-streaming kernel for every N.
+ * accumulate != 0: grad_Wa / grad_Wo are added to, as in the reference, whose caller zeroes them first
+ * (cpp/ring_rnn_cuda.py:98-99); accumulate == 0: they are overwritten and need no zeroing. */
 RINGATTR_API int ringattr_bwd(const void* grad_output, const void* A, const void* Wa, float J0, float J1,
                  const void* Wo, const void* bump_history, const void* r_init,
                  void* grad_Wa, void* grad_Wo, float alpha,
-                 int N, int a_dim, int seq_len, int batch_size, int activation_type,
+                 int N, int a_dim, int seq_len, int batch_size, int activation_type, int accumulate,
                  const void* saved, void* grad_A, void* grad_r_init,
                  void* workspace, size_t workspace_bytes, void* stream);
 
@@ -120,7 +122,7 @@ RINGATTR_API int ringattr_loss_bwd(const void* bump_history, const void* target_
 RINGATTR_API int ringattr_bwd_loss(const void* loss_workspace, const void* upstream, const void* A, const void* Wa,
                       float J0, float J1, const void* Wo, const void* bump_history, const void* r_init,
                       void* grad_Wa, void* grad_Wo, float alpha,
-                      int N, int a_dim, int seq_len, int batch_size, int activation_type,
+                      int N, int a_dim, int seq_len, int batch_size, int activation_type, int accumulate,
                       const void* saved, void* grad_A, void* grad_r_init,
                       void* workspace, size_t workspace_bytes, void* stream);
 

@@ -30,7 +30,7 @@ PROTOTYPES = {
     "ringattr_fwd": (c_int, [c_void_p, c_void_p, c_float, c_float, c_void_p, c_void_p, c_void_p, c_float,
                              c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_size_t, c_void_p]),
     "ringattr_bwd": (c_int, [c_void_p, c_void_p, c_void_p, c_float, c_float, c_void_p, c_void_p, c_void_p,
-                             c_void_p, c_void_p, c_float, c_int, c_int, c_int, c_int, c_int,
+                             c_void_p, c_void_p, c_float, c_int, c_int, c_int, c_int, c_int, c_int,
                              c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
     "ringattr_loss_workspace_bytes": (c_size_t, [c_int] * 3),
     "ringattr_loss_fwd": (c_int, [c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_int, c_int, c_int,
@@ -38,7 +38,7 @@ PROTOTYPES = {
     "ringattr_loss_bwd": (c_int, [c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_int, c_int, c_int,
                                   c_void_p, c_size_t, c_void_p]),
     "ringattr_bwd_loss": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_float, c_void_p, c_void_p, c_void_p,
-                                  c_void_p, c_void_p, c_float, c_int, c_int, c_int, c_int, c_int,
+                                  c_void_p, c_void_p, c_float, c_int, c_int, c_int, c_int, c_int, c_int,
                                   c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
     "ringattr_profile_enable": (c_int, [c_int]),
     "ringattr_profile_read": (c_int, [ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_longlong)]),

@@ -790,7 +790,7 @@ __global__ __launch_bounds__(256) void ring_dw_kernel(RingDwArgs p) {
 }
 
 // Fixed-order sum of the K-split partials, undoing the tile permutation, accumulated into the
-// caller's grad_Wo / grad_Wa (which the caller zeroed, cpp/ring_rnn_cuda.py:98-99).
+// caller's grad_Wo / grad_Wa (which the caller zeroed, cpp/ring_rnn_cuda.py:98-99) or written over them.
 __global__ __launch_bounds__(256) void ring_dw_reduce_kernel(RingDwArgs p, int NC) {
   const int NT = 4 * NC;
   const size_t per_z = (size_t)(p.k + 1) * NT * NT * 64;
@@ -821,7 +821,10 @@ __global__ __launch_bounds__(256) void ring_dw_reduce_kernel(RingDwArgs p, int N
 #pragma unroll
   for (int e = 0; e < 4; ++e) {
     const int i = 16 * NC * (it / NC) + NC * (4 * q + e) + (it % NC);
-    if (i < p.N) out[(size_t)i * p.N + j] += scale * s[e];
+    if (i < p.N) {
+      float* o = out + (size_t)i * p.N + j;
+      *o = p.accumulate ? *o + scale * s[e] : scale * s[e];
+    }
   }
 }
 

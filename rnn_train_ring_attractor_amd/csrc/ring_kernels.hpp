@@ -43,6 +43,7 @@ struct RingDwArgs {
   float* grad_Wo;        // [N,N], accumulated into
   float* grad_Wa;        // [k,N,N], accumulated into
   float J1;
+  int accumulate;        // non-zero: += into grad_Wo / grad_Wa (the caller zeroed them); zero: overwrite
   int N, k, T, B, nbt, nz;
 };
 

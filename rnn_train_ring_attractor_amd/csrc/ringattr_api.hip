@@ -156,36 +156,37 @@ int ringattr_fwd(const void* A, const void* Wa, float J0, float J1, const void* 
 static int bwd_impl(const char* who, const void* grad_output, const void* loss_workspace, const void* upstream, const void* A,
                     const void* Wa, float J0, float J1, const void* Wo, const void* bump_history, const void* r_init,
                     void* grad_Wa, void* grad_Wo, float alpha, int N, int a_dim, int seq_len, int batch_size,
-                    int activation_type, const void* saved, void* grad_A, void* grad_r_init, void* workspace,
-                    size_t workspace_bytes, void* stream);
+                    int activation_type, int accumulate, const void* saved, void* grad_A, void* grad_r_init,
+                    void* workspace, size_t workspace_bytes, void* stream);
 
 int ringattr_bwd(const void* grad_output, const void* A, const void* Wa, float J0, float J1, const void* Wo,
                  const void* bump_history, const void* r_init, void* grad_Wa, void* grad_Wo, float alpha, int N,
-                 int a_dim, int seq_len, int batch_size, int activation_type, const void* saved, void* grad_A,
-                 void* grad_r_init, void* workspace, size_t workspace_bytes, void* stream) {
+                 int a_dim, int seq_len, int batch_size, int activation_type, int accumulate, const void* saved,
+                 void* grad_A, void* grad_r_init, void* workspace, size_t workspace_bytes, void* stream) {
   if (!grad_output) return fail(RINGATTR_ERR_INVALID, "ringattr_bwd: null tensor pointer");
   return bwd_impl("ringattr_bwd", grad_output, nullptr, nullptr, A, Wa, J0, J1, Wo, bump_history, r_init, grad_Wa, grad_Wo,
-                  alpha, N, a_dim, seq_len, batch_size, activation_type, saved, grad_A, grad_r_init, workspace,
+                  alpha, N, a_dim, seq_len, batch_size, activation_type, accumulate, saved, grad_A, grad_r_init, workspace,
                   workspace_bytes, stream);
 }
 
 int ringattr_bwd_loss(const void* loss_workspace, const void* upstream, const void* A, const void* Wa, float J0, float J1,
                       const void* Wo, const void* bump_history, const void* r_init, void* grad_Wa, void* grad_Wo,
-                      float alpha, int N, int a_dim, int seq_len, int batch_size, int activation_type, const void* saved,
-                      void* grad_A, void* grad_r_init, void* workspace, size_t workspace_bytes, void* stream) {
+                      float alpha, int N, int a_dim, int seq_len, int batch_size, int activation_type, int accumulate,
+                      const void* saved, void* grad_A, void* grad_r_init, void* workspace, size_t workspace_bytes,
+                      void* stream) {
   if (!loss_workspace) return fail(RINGATTR_ERR_INVALID, "ringattr_bwd_loss: null loss workspace");
   if (!aligned16(loss_workspace)) return fail(RINGATTR_ERR_INVALID, "ringattr_bwd_loss: every pointer must be 16-byte aligned");
   if (N > 1024) return fail(RINGATTR_ERR_INVALID, "the loss head supports N <= 1024 (got %d)", N);
   return bwd_impl("ringattr_bwd_loss", nullptr, loss_workspace, upstream, A, Wa, J0, J1, Wo, bump_history, r_init, grad_Wa,
-                  grad_Wo, alpha, N, a_dim, seq_len, batch_size, activation_type, saved, grad_A, grad_r_init, workspace,
-                  workspace_bytes, stream);
+                  grad_Wo, alpha, N, a_dim, seq_len, batch_size, activation_type, accumulate, saved, grad_A, grad_r_init,
+                  workspace, workspace_bytes, stream);
 }
 
 static int bwd_impl(const char* who, const void* grad_output, const void* loss_workspace, const void* upstream, const void* A,
                     const void* Wa, float J0, float J1, const void* Wo, const void* bump_history, const void* r_init,
                     void* grad_Wa, void* grad_Wo, float alpha, int N, int a_dim, int seq_len, int batch_size,
-                    int activation_type, const void* saved, void* grad_A, void* grad_r_init, void* workspace,
-                    size_t workspace_bytes, void* stream) {
+                    int activation_type, int accumulate, const void* saved, void* grad_A, void* grad_r_init,
+                    void* workspace, size_t workspace_bytes, void* stream) {
   Geo g;
   int rc = make_geo(N, a_dim, seq_len, batch_size, g);
   if (rc) return rc;
@@ -291,6 +292,7 @@ static int bwd_impl(const char* who, const void* grad_output, const void* loss_w
   d.grad_Wo = (float*)grad_Wo;
   d.grad_Wa = (float*)grad_Wa;
   d.J1 = J1;
+  d.accumulate = accumulate;
   d.N = N;
   d.k = a_dim;
   d.T = seq_len;
@@ -397,7 +399,7 @@ void bwd_cuda(void* grad_output, void* A, void* Wa, float J0, float J1, void* Wo
     return;
   }
   if (ringattr_bwd(grad_output, A, Wa, J0, J1, Wo, bump_history, r_init, grad_Wa, grad_Wo, alpha, N, a_dim, seq_len,
-                   batch_size, activation_type, nullptr, nullptr, nullptr, ws, need, nullptr) != RINGATTR_OK)
+                   batch_size, activation_type, /*accumulate=*/1, nullptr, nullptr, nullptr, ws, need, nullptr) != RINGATTR_OK)
     fprintf(stderr, "bwd_cuda: %s\n", ringattr_last_error());
   (void)hipStreamSynchronize(nullptr);
   (void)hipFree(ws);

@@ -129,13 +129,13 @@ class RingRnnLossFunc(Function):
     @staticmethod
     def backward(ctx, grad_total, _grad_parts, _grad_hist):
         A, Wa, Wo, hist, r0, saved, lws = ctx.saved_tensors
-        grad_Wa, grad_Wo = torch.zeros_like(Wa), torch.zeros_like(Wo)
+        grad_Wa, grad_Wo = torch.empty_like(Wa), torch.empty_like(Wo)    # written, not accumulated into
         grad_A = torch.empty_like(A) if ctx.needs_input_grad[0] else None
         grad_r0 = torch.empty_like(r0) if ctx.needs_input_grad[5] else None
         up = grad_total.to(torch.float32).reshape(1).contiguous()
         bwd_cuda.bwd(grad_output=None, A=A, Wa=Wa, J0=ctx.J0, J1=ctx.J1, Wo=Wo, bump_history=hist, r_init=r0,
                      grad_Wa=grad_Wa, grad_Wo=grad_Wo, alpha=ctx.alpha, activation_type=ctx.act, saved=saved,
-                     grad_A=grad_A, grad_r_init=grad_r0, loss_workspace=lws, loss_upstream=up)
+                     grad_A=grad_A, grad_r_init=grad_r0, loss_workspace=lws, loss_upstream=up, accumulate=False)
         return grad_A, grad_Wa, None, None, grad_Wo, grad_r0, None, None, None, None, None
 
 

@@ -87,8 +87,8 @@ class RingRnnCudaFunc(Function):
     @staticmethod
     def backward(ctx, grad_output):
         action_signal, Wa, Wo, bump_history, r_init, saved = ctx.saved_tensors
-        grad_Wa = torch.zeros_like(Wa)
-        grad_Wo = torch.zeros_like(Wo)
+        grad_Wa = torch.empty_like(Wa)      # written, not accumulated into: no zero-fill launches
+        grad_Wo = torch.empty_like(Wo)
         # The reference returns None for action_signal and r_init (cpp/ring_rnn_cuda.py:144); here they get their
         # gradients when the caller asked for them (gain networks in front of the op need dL/d action_signal).
         grad_A = torch.empty_like(action_signal) if ctx.needs_input_grad[0] else None
@@ -96,5 +96,5 @@ class RingRnnCudaFunc(Function):
         bwd_cuda.bwd(grad_output=grad_output.contiguous(), A=action_signal, Wa=Wa, J0=ctx.J0, J1=ctx.J1, Wo=Wo,
                      bump_history=bump_history, r_init=r_init, grad_Wa=grad_Wa, grad_Wo=grad_Wo,
                      alpha=ctx.alpha, activation_type=ctx.activation_type, saved=saved, grad_A=grad_A,
-                     grad_r_init=grad_r0)
+                     grad_r_init=grad_r0, accumulate=False)
         return grad_A, grad_Wa, None, None, grad_Wo, grad_r0, None, None

@@ -130,7 +130,10 @@ class _Bwd:
     def bwd(grad_output, A, Wa, J0, J1, Wo, bump_history, re_history=None, r_init=None, grad_Wa=None, grad_Wo=None,
             alpha=None, activation_type=None, grad_r=None, W_eff_temp=None, grad_re_temp=None,
             grad_W_eff_temp_bf16=None, A_t_temp_bf16=None, grad_re_temp_T=None, cublas_handle=None,
-            saved=None, grad_r_init=None, grad_A=None, stream=None, loss_workspace=None, loss_upstream=None):
+            saved=None, grad_r_init=None, grad_A=None, stream=None, loss_workspace=None, loss_upstream=None,
+            accumulate=True):
+        # accumulate=True adds into grad_Wa / grad_Wo as the reference does (its caller zeroes them,
+        # cpp/ring_rnn_cuda.py:98-99); False overwrites them, so they may be uninitialised.
         # loss_workspace (what the fused loss head's forward filled for this bump_history) in place of grad_output:
         # the gradient of the loss pair is then formed inside the backward, scaled by loss_upstream (1-element tensor)
         if (grad_output is None) == (loss_workspace is None):
@@ -184,7 +187,7 @@ class _Bwd:
                 ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
                 rc = lib.ringattr_bwd_loss(_ptr(loss_workspace), _ptr(loss_upstream), _ptr(A), _ptr(Wa), J0, J1, _ptr(Wo),
                                            _ptr(bump_history), _ptr(r_init), _ptr(grad_Wa), _ptr(grad_Wo), alpha, N, k, T,
-                                           B, act, _ptr(saved), _ptr(grad_A), _ptr(grad_r_init), _ptr(ws), ws_bytes,
+                                           B, act, 1 if accumulate else 0, _ptr(saved), _ptr(grad_A), _ptr(grad_r_init), _ptr(ws), ws_bytes,
                                            _stream_ptr(stream, dev))
             _lib.check(rc)
             return None
@@ -195,7 +198,7 @@ class _Bwd:
             ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
             rc = lib.ringattr_bwd(_ptr(grad_output), _ptr(A), _ptr(Wa), J0, J1, _ptr(Wo), _ptr(bump_history),
                                   _ptr(r_init), _ptr(grad_Wa), _ptr(grad_Wo), alpha, N, k, T, B, act,
-                                  _ptr(saved), _ptr(grad_A), _ptr(grad_r_init), _ptr(ws), ws_bytes,
+                                  1 if accumulate else 0, _ptr(saved), _ptr(grad_A), _ptr(grad_r_init), _ptr(ws), ws_bytes,
                                   _stream_ptr(stream, dev))
         _lib.check(rc)
         return None

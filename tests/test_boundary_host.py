@@ -60,7 +60,7 @@ def test_c_abi_rejects_bad_arguments_with_codes_not_exit():
     bad_shape = list(ok_args)
     bad_shape[9] = 0                                                    # a_dim
     assert lib.ringattr_fwd(*bad_shape, 0, None, p, 1 << 20, None) == 1
-    bwd_args = [p, p, p, 0.0, 1.0, p, p, p, p, p, 0.15, 64, 2, 4, 16, 0]
+    bwd_args = [p, p, p, 0.0, 1.0, p, p, p, p, p, 0.15, 64, 2, 4, 16, 0, 1]
     assert lib.ringattr_bwd(*bwd_args, None, None, None, p, 16, None) == 2
     wide = list(bwd_args)
     wide[12] = 64                                                       # a_dim beyond what the grad_A path stages in LDS

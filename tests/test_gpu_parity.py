@@ -230,6 +230,18 @@ def test_gradients_accumulate_and_are_deterministic(gpu_device):
     # history, the saved path took them over the bf16 operand copy: a difference at operand-rounding level.
     assert O.max_rel_err((outs[0][0] - 1.0).cpu().numpy(), Wa.grad.cpu().numpy()) <= MODEL_TOL
     assert O.max_rel_err((outs[0][1] - 2.0).cpu().numpy(), Wo.grad.cpu().numpy()) <= MODEL_TOL
+    # accumulate=False: the buffers are written, whatever they held (here NaN), to exactly the accumulated sums
+    gWa = torch.full_like(Wa, float("nan"))
+    gWo = torch.full_like(Wo, float("nan"))
+    bwd_cuda.bwd(grad_output=G, A=_dev(p["A"], gpu_device), Wa=Wa.detach(), J0=-0.1, J1=0.1, Wo=Wo.detach(),
+                 bump_history=hist.detach(), r_init=_dev(p["r0"], gpu_device), grad_Wa=gWa, grad_Wo=gWo,
+                 alpha=0.15, activation_type=1, accumulate=False)
+    zWa, zWo = torch.zeros_like(Wa), torch.zeros_like(Wo)
+    bwd_cuda.bwd(grad_output=G, A=_dev(p["A"], gpu_device), Wa=Wa.detach(), J0=-0.1, J1=0.1, Wo=Wo.detach(),
+                 bump_history=hist.detach(), r_init=_dev(p["r0"], gpu_device), grad_Wa=zWa, grad_Wo=zWo,
+                 alpha=0.15, activation_type=1)
+    torch.cuda.synchronize()
+    assert torch.equal(gWa, zWa) and torch.equal(gWo, zWo)
 
 
 def test_alpha_zero_and_zero_weights_closed_forms(gpu_device):
