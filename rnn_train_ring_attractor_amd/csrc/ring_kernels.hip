@@ -1050,15 +1050,17 @@ hipError_t ring_launch_dw(const RingDwArgs& a, int NCv, hipStream_t st) {
   {
   ProfScope prof(4, st);
   if (ring_dw_tiled_applicable(NCv)) {
-    (void)ring_launch_dw_tiled(a, NCv, st);
-  } else if (NCv == 1) {
-    hipLaunchKernelGGL((ring_dw_kernel<1, 4>), dim3(blocks), dim3(256), 0, st, a);
+    e = ring_launch_dw_tiled(a, NCv, st);   // every group's launch status, first failure wins
   } else {
-    RING_DISPATCH_NC(NCv, if constexpr (NC >= 2) hipLaunchKernelGGL((ring_dw_kernel<NC, 8>), dim3(blocks), dim3(256), 0, st, a));
+    if (NCv == 1) {
+      hipLaunchKernelGGL((ring_dw_kernel<1, 4>), dim3(blocks), dim3(256), 0, st, a);
+    } else {
+      RING_DISPATCH_NC(NCv, if constexpr (NC >= 2) hipLaunchKernelGGL((ring_dw_kernel<NC, 8>), dim3(blocks), dim3(256), 0, st, a));
+    }
+    e = hipGetLastError();
   }
-  e = hipGetLastError();
   }
-  if (e != hipSuccess) return e;
+  if (e != hipSuccess) return e;   // the reduction must not sum partials that were never written
   const size_t per_z = (size_t)(a.k + 1) * NT * NT * 64;
   ProfScope prof(5, st);
   hipLaunchKernelGGL(ring_dw_reduce_kernel, dim3((unsigned)((per_z + 255) / 256)), dim3(256), 0, st, a, NCv);

@@ -93,7 +93,7 @@ class RingRnnLossFunc(Function):
 
     @staticmethod
     def forward(ctx, action_signal, Wa, J0, J1, Wo, r_init, alpha, activation_name, target_angle, bump_weight,
-                target_amplitude):
+                target_amplitude, grad_mode=None):
         from .ring_rnn_cuda import _activation_id
         act = _activation_id(activation_name)
         B, T, k = action_signal.shape
@@ -107,7 +107,9 @@ class RingRnnLossFunc(Function):
             amp = target_amplitude.reshape(-1).contiguous()
             _check("target_amplitude", amp, (B,), dev)
         hist = torch.empty(T, B, N, device=dev, dtype=A.dtype)
-        needs_grad = any(ctx.needs_input_grad[i] for i in (0, 1, 4, 5))
+        # autograd switches gradient mode off in here and needs_input_grad stays True under no_grad(): the wrapper says
+        needs_grad = grad_mode is not False and any(ctx.needs_input_grad[i] for i in (0, 1, 4, 5))
+        ctx.extra_inputs = 0 if grad_mode is None else 1
         saved = torch.empty(saved_nbytes(N, k, T, B), dtype=torch.uint8, device=dev) if needs_grad else None
         fwd_cuda.fwd(A=A, Wa=Wa_c, J0=J0, J1=J1, Wo=Wo_c, r_init=r0, bump_history=hist, alpha=alpha,
                      activation_type=act, saved=saved)
@@ -136,7 +138,7 @@ class RingRnnLossFunc(Function):
         bwd_cuda.bwd(grad_output=None, A=A, Wa=Wa, J0=ctx.J0, J1=ctx.J1, Wo=Wo, bump_history=hist, r_init=r0,
                      grad_Wa=grad_Wa, grad_Wo=grad_Wo, alpha=ctx.alpha, activation_type=ctx.act, saved=saved,
                      grad_A=grad_A, grad_r_init=grad_r0, loss_workspace=lws, loss_upstream=up, accumulate=False)
-        return grad_A, grad_Wa, None, None, grad_Wo, grad_r0, None, None, None, None, None
+        return (grad_A, grad_Wa, None, None, grad_Wo, grad_r0, None, None, None, None, None) + (None,) * ctx.extra_inputs
 
 
 def ring_rnn_loss_func(action_signal, Wa, J0, J1, Wo, r_init, alpha, activation, target_angle, bump_weight=0.2,
@@ -150,5 +152,5 @@ def ring_rnn_loss_func(action_signal, Wa, J0, J1, Wo, r_init, alpha, activation,
     if compact is not None:
         action_signal, Wa = compact
     total, parts, hist = RingRnnLossFunc.apply(action_signal, Wa, J0, J1, Wo, r_init, alpha, activation, target_angle,
-                                               bump_weight, target_amplitude)
+                                               bump_weight, target_amplitude, torch.is_grad_enabled())
     return total, parts[1], parts[2], hist

@@ -28,7 +28,9 @@ def ring_rnn_cuda_func(action_signal, Wa, J0, J1, Wo, r_init, alpha, activation=
     compact = _silent_channel_view(action_signal, Wa)
     if compact is not None:
         action_signal, Wa = compact
-    return RingRnnCudaFunc.apply(action_signal, Wa, J0, J1, Wo, r_init, alpha, activation)
+    # Autograd switches gradient mode off inside Function.forward, and needs_input_grad stays True under
+    # torch.no_grad(): the wrapper is the place that knows whether a backward can follow.
+    return RingRnnCudaFunc.apply(action_signal, Wa, J0, J1, Wo, r_init, alpha, activation, torch.is_grad_enabled())
 
 
 def _silent_channel_view(action_signal, Wa):
@@ -63,7 +65,7 @@ def _silent_channel_view(action_signal, Wa):
 
 class RingRnnCudaFunc(Function):
     @staticmethod
-    def forward(ctx, action_signal, Wa, J0, J1, Wo, r_init, alpha, activation_name):
+    def forward(ctx, action_signal, Wa, J0, J1, Wo, r_init, alpha, activation_name, grad_mode=None):
         activation_type = _activation_id(activation_name)
         batch_size, seq_len, a_dim = action_signal.shape
         N = Wa.shape[1]
@@ -72,7 +74,9 @@ class RingRnnCudaFunc(Function):
         bump_history = torch.empty(seq_len, batch_size, N, device=action_signal.device, dtype=action_signal.dtype)
 
         # F'(re) and the bf16 operand copy of r_prev are only worth writing when a backward will follow
-        needs_grad = any(ctx.needs_input_grad[i] for i in (0, 1, 4, 5))
+        # (grad_mode is None when apply() is called with the reference's eight arguments)
+        needs_grad = grad_mode is not False and any(ctx.needs_input_grad[i] for i in (0, 1, 4, 5))
+        ctx.extra_inputs = 0 if grad_mode is None else 1
         saved = None
         if needs_grad:
             saved = torch.empty(saved_nbytes(N, a_dim, seq_len, batch_size), dtype=torch.uint8,
@@ -97,4 +101,4 @@ class RingRnnCudaFunc(Function):
                      bump_history=bump_history, r_init=r_init, grad_Wa=grad_Wa, grad_Wo=grad_Wo,
                      alpha=ctx.alpha, activation_type=ctx.activation_type, saved=saved, grad_A=grad_A,
                      grad_r_init=grad_r0, accumulate=False)
-        return grad_A, grad_Wa, None, None, grad_Wo, grad_r0, None, None
+        return (grad_A, grad_Wa, None, None, grad_Wo, grad_r0, None, None) + (None,) * ctx.extra_inputs
