@@ -74,6 +74,21 @@ RINGATTR_API int ringattr_fwd(const void* A, const void* Wa, float J0, float J1,
                  int N, int a_dim, int seq_len, int batch_size, int activation_type,
                  void* saved, void* workspace, size_t workspace_bytes, void* stream);
 
+/* ringattr_fwd for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same arguments and results as
+ * ringattr_fwd without the workspace pair: the packed bf16 weights go into a fixed array of
+ * RINGATTR_NOALLOC_SCRATCH_BYTES that lives inside the library's code object on every GPU it runs on (held until
+ * the process ends).  The call allocates and frees nothing.  Shapes whose packed weights
+ * ((1 + a_dim) * NPAD^2 * 2 bytes, NPAD = N rounded up to the kernel's tiling) exceed the array are rejected with
+ * RINGATTR_ERR_WORKSPACE.  All calls on one GPU share that GPU's array: calls that overlap in time on one GPU
+ * (different streams, different threads) race on it; calls on one stream are ordered and safe.  The device that
+ * owns the tensors must be current.  `saved` may be NULL or a caller buffer of ringattr_saved_bytes. */
+#define RINGATTR_NOALLOC_SCRATCH_BYTES (4u << 20)
+RINGATTR_API int ringattr_fwd_noalloc(const void* A, const void* Wa, float J0, float J1, const void* Wo,
+                 const void* r_init, void* bump_history, float alpha,
+                 int N, int a_dim, int seq_len, int batch_size, int activation_type,
+                 void* saved, void* stream);
+
 /* Reverse-time BPTT + weight gradients.
  * Replaces bwd_cuda (cpp/bwd.cu:4-52) and cpp/bwd.cpp:34-99.
  * `saved` may be NULL: the saved record is then recomputed, from bump_history

@@ -6,8 +6,15 @@
 #include <stdio.h>
 #include <string.h>
 
+#include <mutex>
+
 #include "ring_kernels.hpp"
 #include "ringattr.h"
+
+// Fixed device-side scratch of ringattr_fwd_noalloc: every GPU the library runs on holds its own copy of this array
+// until the process ends.  In host code the name below is only a handle for hipGetSymbolAddress; the address the
+// kernels receive is the per-device pointer that call returns (noalloc_scratch()).
+static __device__ __align__(256) unsigned char scratch[RINGATTR_NOALLOC_SCRATCH_BYTES];
 
 namespace {
 
@@ -79,11 +86,33 @@ int hip_fail(hipError_t e, const char* what) {
   return fail(RINGATTR_ERR_HIP, "%s: %s", what, hipGetErrorString(e));
 }
 
+// Device address of `scratch` on the current device, looked up once per device.
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mu;
+void* g_scratch_ptr[kMaxDevices] = {};
+
+int noalloc_scratch(void** out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return hip_fail(e, "hipGetDevice");
+  if (dev < 0 || dev >= kMaxDevices) return fail(RINGATTR_ERR_INVALID, "device index %d out of range", dev);
+  std::lock_guard<std::mutex> lk(g_scratch_mu);
+  if (!g_scratch_ptr[dev]) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return hip_fail(e, "hipGetSymbolAddress(scratch)");
+    if (!p) return fail(RINGATTR_ERR_HIP, "hipGetSymbolAddress(scratch) returned a null address");
+    g_scratch_ptr[dev] = p;
+  }
+  *out = g_scratch_ptr[dev];
+  return RINGATTR_OK;
+}
+
 }  // namespace
 
 extern "C" {
 
-int ringattr_version(void) { return 1000; }
+int ringattr_version(void) { return 1001; }
 
 const char* ringattr_last_error(void) { return g_err; }
 
@@ -150,6 +179,28 @@ int ringattr_fwd(const void* A, const void* Wa, float J0, float J1, const void* 
   e = ring_launch_fwd(a, g.NC, st);
   if (e != hipSuccess) return hip_fail(e, "forward launch");
   return RINGATTR_OK;
+}
+
+int ringattr_fwd_noalloc(const void* A, const void* Wa, float J0, float J1, const void* Wo, const void* r_init,
+                         void* bump_history, float alpha, int N, int a_dim, int seq_len, int batch_size,
+                         int activation_type, void* saved, void* stream) {
+  Geo g;
+  int rc = make_geo(N, a_dim, seq_len, batch_size, g);
+  if (rc) return rc;
+  if (g.wpack_bytes > (size_t)RINGATTR_NOALLOC_SCRATCH_BYTES)
+    return fail(RINGATTR_ERR_WORKSPACE,
+                "ringattr_fwd_noalloc: N = %d with a_dim = %d needs %zu bytes of packed weights, the built-in scratch "
+                "holds %zu; use ringattr_fwd with a caller workspace",
+                N, a_dim, g.wpack_bytes, (size_t)RINGATTR_NOALLOC_SCRATCH_BYTES);
+  if ((rc = check_act(activation_type))) return rc;
+  if (!A || !Wa || !Wo || !r_init || !bump_history)
+    return fail(RINGATTR_ERR_INVALID, "ringattr_fwd_noalloc: null tensor pointer");
+  void* ws = nullptr;
+  if ((rc = noalloc_scratch(&ws))) return rc;
+  // Every byte of the packed-weight area this call reads is rewritten by its own packing launch, so nothing of an
+  // earlier call's contents survives into the result; calls that overlap on one GPU would race on the array.
+  return ringattr_fwd(A, Wa, J0, J1, Wo, r_init, bump_history, alpha, N, a_dim, seq_len, batch_size, activation_type,
+                      saved, ws, (size_t)RINGATTR_NOALLOC_SCRATCH_BYTES, stream);
 }
 
 // grad_output != null: plain backward.  Otherwise loss_workspace (filled by ringattr_loss_fwd) describes grad_output.

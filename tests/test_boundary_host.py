@@ -67,6 +67,10 @@ def test_c_abi_rejects_bad_arguments_with_codes_not_exit():
     assert lib.ringattr_bwd(*wide, None, p, None, p, 1 << 30, None) == 1 and "grad_A" in _lib.last_error()
     assert lib.ringattr_bwd(*bwd_args, None, p + 4, None, p, 1 << 30, None) == 1 and "aligned" in _lib.last_error()
     assert lib.ringattr_profile_read(None, None) == 1
+    # the entry point with the built-in scratch rejects shapes whose packed weights exceed it, before any GPU call
+    assert lib.ringattr_fwd_noalloc(p, p, 0.0, 1.0, p, p, p, 0.15, 512, 8, 4, 16, 0, None, None) == 2
+    assert "built-in scratch" in _lib.last_error()
+    assert lib.ringattr_fwd_noalloc(p, p, 0.0, 1.0, p, p, p, 0.15, 64, 2, 4, 16, 9, None, None) == 1
     with pytest.raises(ValueError):
         _lib.check(1)
     with pytest.raises(RuntimeError):
