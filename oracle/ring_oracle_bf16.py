@@ -47,10 +47,12 @@ def round_u8_dact(x):
 
 
 def forward_backward(A, Wa, J0, J1, Wo, r_init, alpha, activation_name, grad_output=None, rounding=True,
-                     rowsum_rounded=False, dact="fp16"):
+                     folded=False, dact="fp16"):
     """Returns dict(bump_history [T,B,N], and, when grad_output is given, grad_Wa, grad_Wo, grad_r_init).
-    rowsum_rounded: the J0 row sums run over the bf16 operand copy (the weight-resident kernels take them
-    from the matrix pipe) instead of the fp32 state.  dact: storage format of F', "fp16" or "u8"."""
+    folded: model of the weight-resident kernels, whose bf16 Wo operand is round(J1 * Wo + J0) (formed in fp32), so
+    that J0 * sum_j x_j + J1 * (x Wo^T) is one product over the bf16 operand copy of x; otherwise (the streaming
+    kernels) Wo is rounded alone, J1 is applied in fp32 and the J0 row sums run over the fp32 values.
+    dact: storage format of F', "fp16" or "u8"."""
     rb16 = round_bf16 if rounding else _identity
     rf16 = (round_u8_dact if dact == "u8" else round_fp16) if rounding else _identity
     A = np.asarray(A, np.float64)
@@ -60,13 +62,15 @@ def forward_backward(A, Wa, J0, J1, Wo, r_init, alpha, activation_name, grad_out
     B, T, k = A.shape
     N = Wo.shape[0]
     Wob, Wab = rb16(Wo), rb16(Wa)
+    if folded:   # fp32 fused multiply-add, then one rounding to bf16
+        Wof = rb16((Wo * float(np.float32(J1)) + float(np.float32(J0))).astype(np.float32))
     hist = np.empty((T, B, N))
     D = np.empty((T, B, N))
     R = np.empty((T, B, N))
     for t in range(T):
         rb = rb16(r)
         R[t] = rb
-        re = J0 * (rb if rowsum_rounded else r).sum(axis=1, keepdims=True) + J1 * (rb @ Wob.T)
+        re = rb @ Wof.T if folded else J0 * r.sum(axis=1, keepdims=True) + J1 * (rb @ Wob.T)
         for c in range(k):
             re = re + A[:, t, c:c + 1] * (rb @ Wab[c].T)
         D[t] = rf16(alpha * O.activation_derivative(re, activation_name))   # the kernels save alpha * F'
@@ -83,7 +87,10 @@ def forward_backward(A, Wa, J0, J1, Wo, r_init, alpha, activation_name, grad_out
         G = G_out[t] + carry
         g = D[t] * G
         gb = rb16(g)
-        carry = (1.0 - alpha) * G + J0 * (gb if rowsum_rounded else g).sum(axis=1, keepdims=True) + J1 * (gb @ Wob)
+        if folded:
+            carry = (1.0 - alpha) * G + gb @ Wof
+        else:
+            carry = (1.0 - alpha) * G + J0 * g.sum(axis=1, keepdims=True) + J1 * (gb @ Wob)
         for c in range(k):
             carry = carry + A[:, t, c:c + 1] * (gb @ Wab[c])
         grad_Wo += J1 * (gb.T @ R[t])

@@ -13,12 +13,14 @@
 //   out[mm][w][c][kc][lane][8]; lane (q,n) owns output column 16*NC*w + NC*n + c and the eight
 //   contraction indices 32kc+8q .. +7.  transposed = 0: value = W[col][contr] (forward, re = W r);
 //   transposed = 1: value = W[contr][col] (backward, g @ W).
-//   scale0 multiplies matrix 0 (Wo) before rounding: kernels that fold J1 into the weights pass J1.
+//   Matrix 0 (Wo) is stored as scale0 * Wo + shift0 (rounded once, after the fp32 sum): the weight-resident kernels
+//   pass (J1, J0), which turns  J0 * sum_j x_j + J1 * (x Wo^T)  into one product; the others pass (1, 0).  Padding
+//   stays zero.
 //   split_k = 1 (NC = 4 only): contraction position kappa stands for neuron split_k_neuron(kappa) and output
 //   column n of tile c for neuron 64*w + 32*(c/2) + 2*n + c%2: the pipelined weight-resident forward's order.
 // ------------------------------------------------------------------------------------------------
 __device__ __forceinline__ bf16x8 pack_fragment(const float* __restrict__ Wo, const float* __restrict__ Wa, size_t u,
-                                                int N, int NC, int transposed, int split_k, float scale0) {
+                                                int N, int NC, int transposed, int split_k, float scale0, float shift0) {
   const int KCH = 2 * NC;
   const int lane = (int)(u & 63);
   size_t v = u >> 6;
@@ -38,8 +40,11 @@ __device__ __forceinline__ bf16x8 pack_fragment(const float* __restrict__ Wo, co
   for (int x = 0; x < 8; ++x) {
     const int kk = split_k ? split_k_neuron(k0 + x) : k0 + x;
     float val = 0.f;
-    if (col < N && kk < N) val = transposed ? W[(size_t)kk * N + col] : W[(size_t)col * N + kk];
-    pk[x] = (__bf16)(mm == 0 ? val * scale0 : val);
+    if (col < N && kk < N) {
+      val = transposed ? W[(size_t)kk * N + col] : W[(size_t)col * N + kk];
+      if (mm == 0) val = fmaf(val, scale0, shift0);
+    }
+    pk[x] = (__bf16)val;
   }
   return pk;
 }
@@ -50,12 +55,13 @@ __global__ __launch_bounds__(256) void ring_pack_weights_kernel(const float* __r
                                                                 const float* __restrict__ Wa,
                                                                 bf16x8* __restrict__ out, bf16x8* __restrict__ out2, int N,
                                                                 int k, int NC, int transposed, int split_k, float scale0,
-                                                                int transposed2, int split_k2, float scale2) {
+                                                                float shift0, int transposed2, int split_k2, float scale2,
+                                                                float shift2) {
   const size_t total = (size_t)(1 + k) * 4 * NC * 2 * NC * 64;
   const size_t all = out2 ? 2 * total : total;
   for (size_t u = (size_t)blockIdx.x * blockDim.x + threadIdx.x; u < all; u += (size_t)gridDim.x * blockDim.x) {
-    if (u < total) out[u] = pack_fragment(Wo, Wa, u, N, NC, transposed, split_k, scale0);
-    else out2[u - total] = pack_fragment(Wo, Wa, u - total, N, NC, transposed2, split_k2, scale2);
+    if (u < total) out[u] = pack_fragment(Wo, Wa, u, N, NC, transposed, split_k, scale0, shift0);
+    else out2[u - total] = pack_fragment(Wo, Wa, u - total, N, NC, transposed2, split_k2, scale2, shift2);
   }
 }
 
@@ -909,20 +915,20 @@ hipError_t ring_profile_collect(double* ms, long long* launches) {
   }
 
 hipError_t ring_launch_pack2(const float* Wo, const float* Wa, int N, int k, int NC, void* out, int transposed,
-                             int split_k, float scale0, void* out2, int transposed2, int split_k2, float scale2,
-                             hipStream_t st) {
+                             int split_k, float scale0, float shift0, void* out2, int transposed2, int split_k2,
+                             float scale2, float shift2, hipStream_t st) {
   if ((split_k || (out2 && split_k2)) && NC != 4) return hipErrorInvalidValue;
   const size_t total = (size_t)(1 + k) * 4 * NC * 2 * NC * 64 * (out2 ? 2 : 1);
   const int blocks = (int)((total + 255) / 256 < 4096 ? (total + 255) / 256 : 4096);
   ProfScope prof(0, st);
   hipLaunchKernelGGL(ring_pack_weights_kernel, dim3(blocks), dim3(256), 0, st, Wo, Wa, (bf16x8*)out, (bf16x8*)out2, N, k,
-                     NC, transposed, split_k, scale0, transposed2, split_k2, scale2);
+                     NC, transposed, split_k, scale0, shift0, transposed2, split_k2, scale2, shift2);
   return hipGetLastError();
 }
 
 hipError_t ring_launch_pack(const float* Wo, const float* Wa, void* out, int N, int k, int NC, int transposed,
-                            int split_k, float scale0, hipStream_t st) {
-  return ring_launch_pack2(Wo, Wa, N, k, NC, out, transposed, split_k, scale0, nullptr, 0, 0, 1.f, st);
+                            int split_k, float scale0, float shift0, hipStream_t st) {
+  return ring_launch_pack2(Wo, Wa, N, k, NC, out, transposed, split_k, scale0, shift0, nullptr, 0, 0, 1.f, 0.f, st);
 }
 
 // RINGATTR_STREAMING=1 forces the generic weight-streaming kernels (used by tests to cross-check).

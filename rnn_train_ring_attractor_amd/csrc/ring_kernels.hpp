@@ -47,12 +47,13 @@ struct RingDwArgs {
   int N, k, T, B, nbt, nz;
 };
 
+// matrix 0 is packed as scale0 * Wo + shift0 (see ring_pack_weights_kernel)
 hipError_t ring_launch_pack(const float* Wo, const float* Wa, void* out, int N, int k, int NC, int transposed,
-                            int split_k, float scale0, hipStream_t st);
+                            int split_k, float scale0, float shift0, hipStream_t st);
 // two packed copies in one launch (out2 may be null)
 hipError_t ring_launch_pack2(const float* Wo, const float* Wa, int N, int k, int NC, void* out, int transposed,
-                             int split_k, float scale0, void* out2, int transposed2, int split_k2, float scale2,
-                             hipStream_t st);
+                             int split_k, float scale0, float shift0, void* out2, int transposed2, int split_k2,
+                             float scale2, float shift2, hipStream_t st);
 hipError_t ring_launch_fwd(const RingFwdArgs& a, int NC, hipStream_t st);
 hipError_t ring_launch_rebuild(const RingFwdArgs& a, int NC, hipStream_t st);
 hipError_t ring_launch_bptt(const RingBpttArgs& a, int NC, hipStream_t st);

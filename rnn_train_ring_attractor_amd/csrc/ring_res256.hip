@@ -89,7 +89,8 @@ __device__ __forceinline__ void load_resident(const bf16x8* Wp, bf16x8* wl, bf16
 //   E: tiles x K chunks 4..7, epilogue -> r^E_{t+1}   L: tiles x K chunks 0..7 -> pre-activations of step t
 // The E half of the operand tile is double-buffered by step parity (L still reads r^E_t while E
 // writes r^E_{t+1}); the L half is written and read in different intervals and needs one buffer.
-// Row sums for the J0 term come from the matrix pipe (r x ones).
+// The packed Wo slice holds J1 * Wo + J0 (ring_pack_weights_kernel), so the global-inhibition term J0 * sum_j r_j
+// and the J1 scale are part of the one product and cost neither row sums nor epilogue arithmetic.
 // Registers: 128 AGPRs hold the wave's slices of the two gated matrices, the slice of Wo sits in LDS.
 // ------------------------------------------------------------------------------------------------
 namespace {
@@ -139,15 +140,15 @@ __global__ __launch_bounds__(512) void ring_fwd_res256_kernel(RingFwdArgs p) {
   // their slots in the common tile order of the saved buffers: tile ct0 + cc, lane lc (same row group q)
   const int ct0 = 2 * (n & 1), lc = (lane & 48) | (8 * h + (n >> 1));
   const int N = p.N, B = p.B, T = p.T;
-  const float oma = 1.f - p.alpha, alpha = p.alpha, J0 = p.J0, J1 = p.J1;
+  const float oma = 1.f - p.alpha;
+  const ActScale asc = act_scale_make(p.alpha);
   constexpr int HK = R_KCH / 2;
+  // wave-uniform indices as scalars: store addresses then split into a scalar base and a per-lane constant
+  const int wu = __builtin_amdgcn_readfirstlane(w), hu = __builtin_amdgcn_readfirstlane(h);
 
   bf16x8 wreg[2][2][R_KCH];
   bf16x8* wl = wlds + (size_t)(w8 * 2 * R_KCH) * 64 + lane;
   load_resident8(reinterpret_cast<const bf16x8*>(p.Wpack), wl, wreg, w, h, lane);
-  bf16x8 ones;
-#pragma unroll
-  for (int x = 0; x < 8; ++x) ones[x] = (__bf16)1.0f;
 
   float r[4][2], okf[4][2], d[4][2];
 #pragma unroll
@@ -195,34 +196,41 @@ __global__ __launch_bounds__(512) void ring_fwd_res256_kernel(RingFwdArgs p) {
   // epilogue (the write path would throttle the wave for the whole burst while the matrix pipe
   // idles) but one at a time between the MFMA groups of the following contraction.  The values stay
   // in r[] and d[] until the next activation.  slot 0..3: history rows, 4..5: F', 6..7: operand copy.
+  // Lane-constant byte offsets of the three kinds of store; what varies with the step is wave-uniform and is
+  // added on the scalar unit (the unmasked variant addresses every store as scalar base + lane offset + immediate).
+  const unsigned hist_lane = (unsigned)((4 * q * 256 + 2 * n) * sizeof(float));           // + row e * 1 KiB
+  const unsigned d_lane = (unsigned)((lc * 4 * R_NC + 4 * ct0) * sizeof(_Float16));        // + tile cc * 8 B
+  const unsigned r_lane = (unsigned)((ct0 * 64 + lc) * 16);                                // + tile cc * 1 KiB
   auto emit_store = [&](int t, int slot) {
     __builtin_amdgcn_sched_barrier(0);
     if (slot < 4) {
       if (p.hist == nullptr) return;   // recompute of the saved record only: the history already exists
       const int e = slot;
-      float* dst = p.hist + ((size_t)t * B + b0 + e) * N + i0;
       if constexpr (FULL) {
-        *reinterpret_cast<f32x2*>(dst) = f32x2{r[e][0], r[e][1]};
+        char* base = reinterpret_cast<char*>(p.hist + ((size_t)t * B + 16 * bt) * 256 + 64 * wu + 32 * hu);
+        *reinterpret_cast<f32x2*>(base + hist_lane + e * 1024) = f32x2{r[e][0], r[e][1]};
       } else {
+        float* dst = p.hist + ((size_t)t * B + b0 + e) * N + i0;
         if (okf[e][0] != 0.f) dst[0] = r[e][0];
         if (okf[e][1] != 0.f) dst[1] = r[e][1];
       }
     } else if (slot < 6) {
       if (SAVE) {
         const int cc = slot - 4;
-        _Float16* drec = p.dfrag + side_offset<R_NC>(t, p.nbt, bt, w, lc) + 4 * (ct0 + cc);
+        char* base = reinterpret_cast<char*>(p.dfrag + side_offset<R_NC>(t, p.nbt, bt, wu, 0));
         const f16x4 pk = {(_Float16)d[0][cc], (_Float16)d[1][cc], (_Float16)d[2][cc], (_Float16)d[3][cc]};
-        *reinterpret_cast<f16x4*>(drec) = pk;
+        *reinterpret_cast<f16x4*>(base + d_lane + cc * 8) = pk;
       }
     } else if (SAVE) {
       const int cc = slot - 6;   // r after step t is the operand of step t+1
+      char* base = reinterpret_cast<char*>(p.rfrag + pair_offset<R_NC>(t + 1, p.nbt, bt, wu * R_NC, 0));
       bf16x4 pk = {(__bf16)r[0][cc], (__bf16)r[1][cc], (__bf16)r[2][cc], (__bf16)r[3][cc]};
-      *reinterpret_cast<bf16x4*>(p.rfrag + pair_offset<R_NC>(t + 1, p.nbt, bt, w * R_NC + ct0 + cc, lc)) = pk;
+      *reinterpret_cast<bf16x4*>(base + r_lane + cc * 1024) = pk;
     }
     __builtin_amdgcn_sched_barrier(0);
   };
 
-  f32x4 P[2][3], S;
+  f32x4 P[2][3];
   auto mfma_unit = [&](int f, const bf16x8 (&af)[HK]) {
     const int cc = (f >> 1) & 1, ph = f >> 2, j = f & 1, fn = (f + 1) & 7;
 #pragma unroll
@@ -244,29 +252,24 @@ __global__ __launch_bounds__(512) void ring_fwd_res256_kernel(RingFwdArgs p) {
     for (int u = 0; u < HK; ++u) af[u] = xrow[u * 4 * XG];
     if (ph == 0) {
       const f32x4 z = {0.f, 0.f, 0.f, 0.f};
-      S = z;
 #pragma unroll
       for (int cc = 0; cc < 2; ++cc) P[cc][0] = P[cc][1] = P[cc][2] = z;
     }
-#pragma unroll
-    for (int u = 0; u < HK; ++u) S = mfma16(af[u], ones, S);
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       if constexpr (decltype(emit)::value) emit_store(ts, 4 * ph + j);
       mfma_unit(4 * ph + j, af);
     }
   };
-  // x[e][cc] = J0*rowsum + J1*P0 + a0*P1 + a1*P2 with the gates of step t
+  // x[e][cc] = P0 + a0*P1 + a1*P2 with the gates of step t (P0 already holds J0*rowsum + J1*(Wo r))
   auto preactivation = [&](int t, float (&x)[4][2]) {
     const f32x2* gb = gbuf + (((t / R_GCH) & 1) * R_GCH + t % R_GCH) * 16 + 4 * q;
-    const f32x4 js = S * J0;
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
       const f32x2 gate = gb[e];
 #pragma unroll
       for (int cc = 0; cc < 2; ++cc) {
-        float v = fmaf(J1, P[cc][0][e], js[e]);
-        v = fmaf(gate[0], P[cc][1][e], v);
+        const float v = fmaf(gate[0], P[cc][1][e], P[cc][0][e]);
         x[e][cc] = fmaf(gate[1], P[cc][2][e], v);
       }
     }
@@ -276,15 +279,15 @@ __global__ __launch_bounds__(512) void ring_fwd_res256_kernel(RingFwdArgs p) {
     for (int e = 0; e < 4; ++e)
 #pragma unroll
       for (int cc = 0; cc < 2; ++cc) {
-        float F, D;
-        act_fast<ACT>(x[e][cc], F, D);
-        float rn = fmaf(alpha, F, oma * r[e][cc]);
+        float aF, aD;
+        act_scaled<ACT>(x[e][cc], asc, aF, aD);
+        float rn = fmaf(oma, r[e][cc], aF);
         if constexpr (!FULL) {
           rn *= okf[e][cc];
-          D *= okf[e][cc];
+          aD *= okf[e][cc];
         }
         r[e][cc] = rn;
-        d[e][cc] = alpha * D;   // the saved record is alpha * F'(re)
+        d[e][cc] = aD;          // the saved record is alpha * F'(re)
       }
   };
   constexpr std::true_type with_stores{};
@@ -464,15 +467,12 @@ __global__ __launch_bounds__(256) void ring_bptt_res256_kernel(RingBpttArgs p) {
   const int b0 = 16 * bt + 4 * q;
   const int i0 = 16 * R_NC * w + R_NC * n;
   const int N = p.N, B = p.B, T = p.T;
-  const float oma = 1.f - p.alpha, J0 = p.J0;   // alpha rides in the saved F' record, J1 in the packed Wo fragments
+  const float oma = 1.f - p.alpha;   // alpha rides in the saved F' record, J0 and J1 in the packed Wo fragments
   const int wu = __builtin_amdgcn_readfirstlane(w);   // the wave index as a scalar, for address arithmetic
 
   bf16x8 wreg[2][R_NC][R_KCH];
   bf16x8* wl = wlds + (size_t)w * R_NC * R_KCH * 64 + lane;
   load_resident(reinterpret_cast<const bf16x8*>(p.Wpack), wl, wreg, w, lane);
-  bf16x8 ones;
-#pragma unroll
-  for (int x = 0; x < 8; ++x) ones[x] = (__bf16)1.0f;
 
   float carry[4][R_NC];
   float okf[4][R_NC];
@@ -579,11 +579,6 @@ __global__ __launch_bounds__(256) void ring_bptt_res256_kernel(RingBpttArgs p) {
       bf16x8 af[R_KCH];
 #pragma unroll
       for (int kc = 0; kc < R_KCH; ++kc) af[kc] = xb[(kc * 4 + q) * XG + n];
-      // J0 * (row sums of g) from the matrix pipe: g x ones puts every row's sum in all 16 columns
-      f32x4 js = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int kc = 0; kc < R_KCH; ++kc) js = mfma16(af[kc], ones, js);
-      js *= J0;
       f32x2 gate[4];
       {
         const f32x2* gb = gbuf + ((ci & 1) * R_GCH + l) * 16 + 4 * q;
@@ -592,8 +587,9 @@ __global__ __launch_bounds__(256) void ring_bptt_res256_kernel(RingBpttArgs p) {
       }
 #pragma unroll
       for (int c = 0; c < R_NC; ++c) {
-        // the ungated chain starts from the terms that need no product: (1 - alpha) * G + J0 * sum(g)
-        f32x4 P0 = {fmaf(oma, G[0][c], js[0]), fmaf(oma, G[1][c], js[1]), fmaf(oma, G[2][c], js[2]), fmaf(oma, G[3][c], js[3])};
+        // the ungated chain starts from the term that needs no product, (1 - alpha) * G; J0 * sum(g) comes with
+        // the product itself (the packed fragments hold J1 * Wo^T + J0)
+        f32x4 P0 = {oma * G[0][c], oma * G[1][c], oma * G[2][c], oma * G[3][c]};
         f32x4 P1 = {0.f, 0.f, 0.f, 0.f}, P2 = P1;
 #pragma unroll
         for (int h = 0; h < 2; ++h) {

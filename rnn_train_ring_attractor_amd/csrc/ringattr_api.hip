@@ -86,6 +86,31 @@ int hip_fail(hipError_t e, const char* what) {
   return fail(RINGATTR_ERR_HIP, "%s: %s", what, hipGetErrorString(e));
 }
 
+// Which kernel family filled a saved buffer: the transposed weight copy behind the saved activations has J0 and J1
+// folded into Wo for the weight-resident BPTT kernel and is plain for the streaming one.  The forward notes what it
+// wrote under the buffer's address; a backward that finds no matching note (another process state, a copied
+// buffer, RINGATTR_STREAMING changed in between) packs its own copy instead of trusting the one in the buffer.
+constexpr int kSavedNotes = 256;
+struct SavedNote { const void* ptr; int family; };   // family: 1 streaming, 2 weight-resident
+std::mutex g_saved_mu;
+SavedNote g_saved_notes[kSavedNotes] = {};
+int g_saved_next = 0;
+
+void saved_note_put(const void* ptr, int family) {
+  std::lock_guard<std::mutex> lk(g_saved_mu);
+  for (auto& n : g_saved_notes)
+    if (n.ptr == ptr) { n.family = family; return; }
+  g_saved_notes[g_saved_next] = SavedNote{ptr, family};
+  g_saved_next = (g_saved_next + 1) % kSavedNotes;
+}
+
+int saved_note_get(const void* ptr) {
+  std::lock_guard<std::mutex> lk(g_saved_mu);
+  for (const auto& n : g_saved_notes)
+    if (n.ptr == ptr) return n.family;
+  return 0;
+}
+
 // Device address of `scratch` on the current device, looked up once per device.
 constexpr int kMaxDevices = 64;
 std::mutex g_scratch_mu;
@@ -152,13 +177,15 @@ int ringattr_fwd(const void* A, const void* Wa, float J0, float J1, const void* 
                 workspace ? workspace_bytes : (size_t)0);
   hipStream_t st = static_cast<hipStream_t>(stream);
 
-  // With a saved buffer the same launch also writes the transposed copy the backward will need (J1
-  // folded into Wo for the weight-resident BPTT kernel) behind the saved activations.
+  // With a saved buffer the same launch also writes the transposed copy the backward will need behind the saved
+  // activations.  The weight-resident kernels take Wo as J1 * Wo + J0 in both copies.
   const int resident = ring_uses_resident(N, a_dim) ? 1 : 0;
   void* wpack_t = saved ? (char*)saved + g.side_bytes + g.pair_bytes : nullptr;
-  hipError_t e = ring_launch_pack2((const float*)Wo, (const float*)Wa, N, a_dim, g.NC, workspace, 0, resident, 1.f,
-                                   wpack_t, 1, 0, resident ? J1 : 1.f, st);
+  const float s0 = resident ? J1 : 1.f, h0 = resident ? J0 : 0.f;
+  hipError_t e = ring_launch_pack2((const float*)Wo, (const float*)Wa, N, a_dim, g.NC, workspace, 0, resident, s0, h0,
+                                   wpack_t, 1, 0, s0, h0, st);
   if (e != hipSuccess) return hip_fail(e, "pack weights");
+  if (saved) saved_note_put(saved, resident ? 2 : 1);
 
   RingFwdArgs a;
   a.A = (const float*)A;
@@ -275,7 +302,9 @@ static int bwd_impl(const char* who, const void* grad_output, const void* loss_w
     _Float16* d = (_Float16*)ws;
     ws += g.side_bytes;
     __bf16* r = (__bf16*)ws;
-    hipError_t e = ring_launch_pack((const float*)Wo, (const float*)Wa, wf, N, a_dim, g.NC, 0, ring_uses_resident(N, a_dim) ? 1 : 0, 1.f, st);
+    const bool res = ring_uses_resident(N, a_dim);
+    hipError_t e = ring_launch_pack((const float*)Wo, (const float*)Wa, wf, N, a_dim, g.NC, 0, res ? 1 : 0, res ? J1 : 1.f,
+                                    res ? J0 : 0.f, st);
     if (e != hipSuccess) return hip_fail(e, "pack weights");
     RingFwdArgs f;
     f.A = (const float*)A;
@@ -299,15 +328,16 @@ static int bwd_impl(const char* who, const void* grad_output, const void* loss_w
     rfrag = r;
   }
 
-  // the weight-resident BPTT kernel takes J1 folded into the transposed Wo fragments
+  // the weight-resident BPTT kernel takes J1 * Wo + J0 in the transposed Wo fragments
   const bool resident = ring_uses_resident(N, a_dim);
   const bool bptt_resident = resident && !grad_A;
   hipError_t e = hipSuccess;
-  if (saved && bptt_resident == resident) {
-    // the forward left the transposed copy (with the scale this BPTT kernel expects) behind the saved activations
+  if (saved && saved_note_get(saved) == (bptt_resident ? 2 : 1)) {
+    // the forward left the transposed copy, in the form this BPTT kernel expects, behind the saved activations
     wb = (char*)const_cast<void*>(saved) + g.side_bytes + g.pair_bytes;
   } else {
-    e = ring_launch_pack((const float*)Wo, (const float*)Wa, wb, N, a_dim, g.NC, 1, 0, bptt_resident ? J1 : 1.f, st);
+    e = ring_launch_pack((const float*)Wo, (const float*)Wa, wb, N, a_dim, g.NC, 1, 0, bptt_resident ? J1 : 1.f,
+                         bptt_resident ? J0 : 0.f, st);
     if (e != hipSuccess) return hip_fail(e, "pack transposed weights");
   }
 

@@ -26,10 +26,10 @@ MODEL_TOL = 5e-3        # HIP vs the rounding-aware CPU model (same operand roun
 ACTS = {"relu": 0, "gelu": 1, "tanh": 2, "silu": 3}
 
 
-def _rowsum_rounded(N, k, A=None):
+def _folded(N, k, A=None):
     """The weight-resident kernels (128 < N <= 256 and two action channels, or more of which at most two are ever
-    driven: the Python operator then runs on those two) take the J0 row sums over the bf16 operand copy of the
-    state, the generic ones over the fp32 state; the rounding model follows the kernel under test."""
+    driven: the Python operator then runs on those two) take Wo as the bf16 rounding of J1 * Wo + J0, the generic
+    ones round Wo alone and sum the J0 term in fp32; the rounding model follows the kernel under test."""
     if not (128 < N <= 256) or os.environ.get("RINGATTR_STREAMING") == "1":
         return False
     if k == 2:
@@ -90,7 +90,7 @@ def test_forward_trajectory_and_decoded_angle(case, gpu_device):
     err = O.max_rel_err(got, ref)
     assert err <= TRAJ_TOL, f"trajectory error {err}"
     model = OB.forward_backward(p["A"], p["Wa"], J0, J1, p["Wo"], p["r0"], 0.15, act,
-                                rowsum_rounded=_rowsum_rounded(N, k, p["A"]))["bump_history"]
+                                folded=_folded(N, k, p["A"]))["bump_history"]
     assert O.max_rel_err(got, model) <= MODEL_TOL
     # per-step error must not blow up along the sequence either
     for t in (0, T // 2, T - 1):
@@ -133,7 +133,7 @@ def test_backward_weight_gradients(case, gpu_device):
     ref_hist, _ = O.forward_dense(p["A"], p["Wa"], J0, J1, p["Wo"], p["r0"], 0.15, act)
     ref = O.backward_dense(p["G"], p["A"], p["Wa"], J0, J1, p["Wo"], ref_hist, p["r0"], 0.15, act)
     model = OB.forward_backward(p["A"], p["Wa"], J0, J1, p["Wo"], p["r0"], 0.15, act, p["G"],
-                                rowsum_rounded=_rowsum_rounded(N, k, p["A"]))
+                                folded=_folded(N, k, p["A"]))
     gWo, gWa = Wo.grad.cpu().numpy(), Wa.grad.cpu().numpy()
     assert np.isfinite(gWo).all() and np.isfinite(gWa).all()
     assert np.abs(ref["grad_Wo"]).max() > 0, "degenerate case: the reference gradient is identically zero"
