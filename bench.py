@@ -1,19 +1,24 @@
 """Headline benchmark: fused forward + BPTT of the ring-attractor time loop on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu]
-
-Defaults: K = 1000 timed steps after W = 200 warm-up steps (about one second of GPU time): the chip's clocks
-take some tens of milliseconds of sustained load to settle, and a step is well under a millisecond.
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu] [--prewarm-ms MS]
 
 One "step" = one forward + one backward of the operator over one synthetic batch at
 N=256, B=4096, T=120, k=2, gelu (inputs resident in HBM before the timed region).
-Prints ONE JSON line: sample-steps/s (B*T per fwd+bwd), the roofline of the slowest kernel from
-HIP events recorded on the launch stream inside the timed region, and a host-CPU baseline (torch
-port of the reference's per-sample-W_eff formulation) on a bounded sample of the same workload.
+
+Phases: an untimed PRE-WARM that always runs (steps of the same workload for at least --prewarm-ms of wall time: the
+chip's clocks take tens of milliseconds of sustained load to settle and a step is well under a millisecond; its
+length is reported under "prewarm"), then exactly --warmup untimed steps, then exactly --steps timed steps between
+two torch.cuda.synchronize().
+
+Prints ONE JSON line: sample-steps/s (B*T per fwd+bwd), the roofline of the slowest kernel from HIP events recorded
+on the launch stream inside the timed region, and host-CPU baselines (torch port of the reference's per-sample-W_eff
+formulation): the reference's own CPU configuration (N=120, B=64, T=120, tanh, fp32) exactly, and the benchmarked
+workload at a reduced batch.
 """
 import argparse
 import json
 import os
+import re
 import sys
 import time
 
@@ -24,31 +29,30 @@ if ROOT not in sys.path:
 PEAK_BF16_TFLOPS = 2500.0      # MI355X dense bf16 MFMA, TFLOP/s
 PEAK_HBM_GBS = 8000.0          # MI355X HBM3E, GB/s
 
-# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per dispatch, each scaled by what the
-# same counter reads for a 1 GiB device copy: x2.000 for FETCH_SIZE, x1.000 for WRITE_SIZE); the summary is
-# profiles/train_n256_b4096_t120_gelu_counters.md.  Counter runs cannot share a process with the timed region, so
-# the figures are carried here and refreshed whenever a kernel's memory behaviour changes.
-MEASURED_TRAFFIC_BYTES = {
-    "train_n256_b4096_t120_gelu": {"fwd": (6002 * 2.0 + 983679) * 1024, "bptt": (376734 * 2.0 + 245760) * 1024,
-                                   "dw": (256553 * 2.0 + 49152) * 1024},
-}
-
+HEADLINE = "train_n256_b4096_t120_gelu"
 WORKLOADS = {
     # the headline training shape (the default and the only workload the metric is quoted on)
-    "train_n256_b4096_t120_gelu": dict(N=256, B=4096, T=120, k=2, act="gelu", J0=-1.0 / 256, J1=1.0, mode="train"),
+    HEADLINE: dict(N=256, B=4096, T=120, k=2, act="gelu", J0=-1.0 / 256, J1=1.0, mode="train"),
     # the other benchmark shapes, for reference figures (run with --workload; pick --steps to taste)
     "train_n120_b64_t120_tanh": dict(N=120, B=64, T=120, k=2, act="tanh", J0=-1.0 / 120, J1=1.0, mode="train"),
     "infer_n256_b1024_t120_relu": dict(N=256, B=1024, T=120, k=2, act="relu", J0=-1.0 / 256, J1=1.0, mode="infer"),
     "train_n512_b8192_t512_tanh": dict(N=512, B=8192, T=512, k=2, act="tanh", J0=-1.0 / 512, J1=1.0, mode="train"),
+    # the general ring with gain networks: two 1 -> 16 -> 1 MLPs turn the angular velocity into the (L, R) gates and
+    # train through dL/d action_signal (model step: MLPs + time loop forward and backward, MLP gradients included)
+    "gain_n256_b4096_t240_relu": dict(N=256, B=4096, T=240, k=2, act="relu", J0=-1.0 / 256, J1=1.0, mode="gain"),
     # the reference training script's own defaults: 16 action channels of which two are driven (zero padding)
     "train_n256_b128_t100_k16pad_gelu": dict(N=256, B=128, T=100, k=16, act="gelu", J0=-0.1, J1=0.1, mode="train"),
 }
+# the shapes of the reference's published latency table (assets/REPORT.md:5-10): forward, B=256, T=20, 16 dense channels
+for _n in (128, 256, 384, 512, 1024, 2048):
+    WORKLOADS[f"report_fwd_n{_n}_b256_t20_k16"] = dict(N=_n, B=256, T=20, k=16, act="silu", J0=-0.1, J1=0.1, mode="infer",
+                                                      action="dense")
 
 
 def make_inputs(cfg, device):
     """Seeded synthetic inputs of the named shape, drawn on the host with the package's own data helpers:
     weights ~ N(0, 1/N); angular-velocity trials (10 % leading zeros, U(-0.1*pi, 0.1*pi), zero ratio in
-    {0.2, 0.5, 0.8}); L/R gates = relu(-/+av); Gaussian bump at each trial's initial angle."""
+    {0.2, 0.5, 0.8}); L/R gates = relu(-/+av); von Mises (kappa = 4) bump at each trial's initial angle."""
     import math
     import torch
     from rnn_train_ring_attractor_amd import host
@@ -57,10 +61,15 @@ def make_inputs(cfg, device):
     Wo = torch.randn(N, N) / math.sqrt(N)
     Wa = torch.randn(k, N, N) / math.sqrt(N)
     av, angle = host.generate_av_integration_data_ultra_fast(B, T)
-    A = host.av_to_action_signal(av) if k == 2 else host.av_to_action_signal_ND(av, k)
-    r0 = host.create_initial_bump(angle[:, 0], N)
+    if cfg.get("action") == "dense":
+        A = torch.rand(B, T, k) * 0.3 / k
+    else:
+        A = host.av_to_action_signal(av) if k == 2 else host.av_to_action_signal_ND(av, k)
+    pref = torch.arange(N, dtype=torch.float32) * (2 * math.pi / N)
+    r0 = torch.exp(4.0 * torch.cos(pref[None, :] - angle[:, :1]))
+    r0 = r0 / r0.norm(dim=1, keepdim=True)
     to = lambda x: x.float().contiguous().to(device)
-    return dict(A=to(A), Wa=to(Wa), Wo=to(Wo), r0=to(r0), angle=to(angle))
+    return dict(A=to(A), Wa=to(Wa), Wo=to(Wo), r0=to(r0), angle=to(angle), av=to(av))
 
 
 def loss_head_grad(hist, angle):
@@ -81,27 +90,63 @@ def loss_head_grad(hist, angle):
     return h.grad.contiguous()
 
 
-def cpu_baseline(cfg, sample_B, iters=8):
-    """Torch port of the reference formulation (W_eff per sample + bmm + autograd), fp32, host cores."""
+def host_cpu():
+    """(threads to use, CPU model string, logical CPUs visible).  Threads = OMP_NUM_THREADS when the environment
+    sets it (the GPU boxes export this job's CPU share there), otherwise every CPU this process may run on."""
+    model = "unknown"
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                model = line.split(":", 1)[1].strip()
+                break
+    except OSError:
+        pass
+    try:
+        visible = len(os.sched_getaffinity(0))
+    except AttributeError:
+        visible = os.cpu_count() or 1
+    threads = int(os.environ.get("OMP_NUM_THREADS", "0")) or visible
+    return threads, model, visible
+
+
+def cpu_baseline(N, B, T, k, act, J0, J1, budget_s, note):
+    """Torch port of the reference formulation (W_eff per sample + bmm + autograd), fp32, host cores: one warm-up,
+    then fwd+bwd iterations until `budget_s` seconds of work (at least 3)."""
     import torch
     from oracle import torch_port as TP
     from tests.ring_cases import make_problem
-    threads = int(os.environ.get("OMP_NUM_THREADS", "0")) or min(16, os.cpu_count() or 1)
+    threads, model, visible = host_cpu()
     torch.set_num_threads(threads)
-    p = make_problem(42, sample_B, cfg["T"], cfg["k"], cfg["N"])
+    p = make_problem(42, B, T, k, N, bump="vm")
     t = lambda x: torch.tensor(x)
-    args = (t(p["A"]), t(p["Wa"]), cfg["J0"], cfg["J1"], t(p["Wo"]), t(p["r0"]), 0.15, cfg["act"])
+    args = (t(p["A"]), t(p["Wa"]), J0, J1, t(p["Wo"]), t(p["r0"]), 0.15, act)
     G = t(p["G"])
     TP.fwd_bwd_autograd(*args, grad_output=G)          # warm-up
     ts = []
-    for _ in range(iters):
+    while len(ts) < 3 or (sum(ts) < budget_s and len(ts) < 200):
         t0 = time.perf_counter()
         TP.fwd_bwd_autograd(*args, grad_output=G)
         ts.append(time.perf_counter() - t0)
     mean = sum(ts) / len(ts)
-    return {"value": sample_B * cfg["T"] / mean, "unit": "sample-steps/s", "cores": threads, "kind": "port",
-            "sample": f"N={cfg['N']} B={sample_B} T={cfg['T']} {cfg['act']} fp32, {iters} fwd+bwd iters, "
-                      f"{mean * 1e3:.0f} ms each (full B={cfg['B']} would need B*N^2*4*T bytes of saved W_eff)"}
+    return {"value": B * T / mean, "unit": "sample-steps/s", "cores": threads, "cpu_model": model,
+            "logical_cpus_visible": visible, "kind": "port",
+            "sample": f"N={N} B={B} T={T} {act} fp32, {len(ts)} fwd+bwd iters, {mean * 1e3:.1f} ms each; {note}"}
+
+
+def measured_traffic(workload):
+    """HBM bytes per launch of each kernel, from the committed rocprofv3 counter summary of this workload
+    (profiles/<workload>_counters.md carries a line 'TRAFFIC_BYTES_PER_LAUNCH fwd=.. bptt=.. dw=..': FETCH_SIZE and
+    WRITE_SIZE per dispatch, each scaled by what the same counter reads for a 1 GiB device copy).  Counter runs cannot
+    share a process with the timed region, so the figure is read from there; None when no summary exists."""
+    path = os.path.join(ROOT, "profiles", f"{workload}_counters.md")
+    try:
+        text = open(path).read()
+    except OSError:
+        return None
+    m = re.search(r"^TRAFFIC_BYTES_PER_LAUNCH\s+(.*)$", text, re.M)
+    if not m:
+        return None
+    return {kv.split("=")[0]: float(kv.split("=")[1]) for kv in m.group(1).split()}
 
 
 def main():
@@ -109,8 +154,10 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=1000)
     ap.add_argument("--warmup", type=int, default=200)
-    ap.add_argument("--workload", default="train_n256_b4096_t120_gelu", choices=sorted(WORKLOADS))
-    ap.add_argument("--no-cpu", action="store_true", help="skip the host-CPU baseline leg")
+    ap.add_argument("--workload", default=HEADLINE, choices=sorted(WORKLOADS))
+    ap.add_argument("--prewarm-ms", type=float, default=500.0,
+                    help="untimed steps of the workload run for at least this long before --warmup (clock settling)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the host-CPU baseline legs")
     ap.add_argument("--cpu-sample-batch", type=int, default=128)
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run three 1 GiB device-to-device copies (known HBM traffic) for scaling rocprofv3's "
@@ -128,24 +175,55 @@ def main():
     cfg = WORKLOADS[args.workload]
     N, B, T, k = cfg["N"], cfg["B"], cfg["T"], cfg["k"]
     x = make_inputs(cfg, dev)
-    Wa = x["Wa"].requires_grad_(True)
-    Wo = x["Wo"].requires_grad_(True)
+    mode = cfg["mode"]
+    train = mode in ("train", "gain")
 
-    def fwd():
-        return ring_rnn_cuda_func(x["A"], Wa, cfg["J0"], cfg["J1"], Wo, x["r0"], 0.15, cfg["act"])
+    if mode == "gain":
+        from rnn_train_ring_attractor_amd import host
+        torch.manual_seed(7)
+        model = host.LeakyRingAttractor(N, activation=cfg["act"], initialization="random").to(dev)
+        model.J0, model.J1 = cfg["J0"], cfg["J1"]
+        params = [p for p in model.parameters() if p.requires_grad]
 
-    train = cfg["mode"] == "train"
-    if train:
+        def fwd():
+            return model.forward_history(x["av"], x["r0"])
+
         G = loss_head_grad(fwd(), x["angle"])
 
         def step():
-            Wa.grad = None
-            Wo.grad = None
+            for p in params:
+                p.grad = None
             fwd().backward(G)
     else:
-        def step():
-            with torch.no_grad():
-                fwd()
+        Wa, Wo = x["Wa"], x["Wo"]
+        if train:
+            Wa.requires_grad_(True)
+            Wo.requires_grad_(True)
+
+        def fwd():
+            return ring_rnn_cuda_func(x["A"], Wa, cfg["J0"], cfg["J1"], Wo, x["r0"], 0.15, cfg["act"])
+
+        if train:
+            G = loss_head_grad(fwd(), x["angle"])
+
+            def step():
+                Wa.grad = None
+                Wo.grad = None
+                fwd().backward(G)
+        else:
+            def step():
+                with torch.no_grad():
+                    fwd()
+
+    # untimed pre-warm: sustained load until the clocks have settled
+    t0 = time.perf_counter()
+    prewarm_steps = 0
+    while (time.perf_counter() - t0) * 1e3 < args.prewarm_ms:
+        for _ in range(10):
+            step()
+        prewarm_steps += 10
+        torch.cuda.synchronize()
+    prewarm_ms = (time.perf_counter() - t0) * 1e3
 
     for _ in range(args.warmup):
         step()
@@ -168,34 +246,46 @@ def main():
 
     ms_per_step = dt / args.steps * 1e3
     value = B * T / (dt / args.steps)
-    flops_third = 6.0 * N * N * B * T                      # per kernel: fwd, bptt and dW each contract 2*3*N^2 per sample-step
+    mats = 1 + k
+    flops_third = 2.0 * mats * N * N * B * T               # per kernel: fwd, bptt and dW each contract 2*(1+k)*N^2 per sample-step
     kern = {kname: (ms / max(cnt, 1)) for kname, (ms, cnt) in prof.items() if cnt}
     dominant = max(("fwd", "bptt", "dw") if train else ("fwd",), key=lambda n_: kern.get(n_, 0.0))
     dom_ms = kern[dominant]
     achieved = flops_third / (dom_ms * 1e-3) / 1e12
     bytes_per_ss = 12 * N + 8 * k                           # fp32 history write + r_prev/grad_output reads + A
+    traffic = measured_traffic(args.workload)
     out = {
         "metric": ("fwd+bwd sample-steps/s (B*T/s) at N=256,B=4096,T=120; % bf16 MFMA peak"
-                   if args.workload == "train_n256_b4096_t120_gelu" else
+                   if args.workload == HEADLINE else
                    f"{'fwd+bwd' if train else 'fwd'} sample-steps/s (B*T/s) at N={N},B={B},T={T}"),
         "value": value, "unit": "sample-steps/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
         "config": {"workload": args.workload, "N": N, "B": B, "T": T, "a_dim": k, "activation": cfg["act"],
-                   "mode": "forward + backward" if train else "forward only (no saved activations)",
+                   "mode": {"train": "forward + backward", "infer": "forward only (no saved activations)",
+                            "gain": "gain MLPs + forward + backward (MLP gradients through dL/d action_signal)"}[mode],
                    "grad_output": "gradient of the cos-sim + 0.2*bump-amplitude loss pair, precomputed" if train else None},
-        "pct_bf16_mfma_peak": 100.0 * ((18.0 if train else 6.0) * N * N * value) / (PEAK_BF16_TFLOPS * 1e12),
+        "prewarm": {"steps": prewarm_steps, "ms": prewarm_ms, "note": "untimed, before --warmup; clock settling"},
+        "pct_bf16_mfma_peak": 100.0 * ((3 if train else 1) * 2.0 * mats * N * N * value) / (PEAK_BF16_TFLOPS * 1e12),
         "algorithmic_hbm_gbs": (bytes_per_ss if train else 4 * N + 4 * k) * value / 1e9,
         "roofline": {"bound": "mfma", "kernel": dominant, "achieved": achieved, "peak": PEAK_BF16_TFLOPS,
                      "unit": "TFLOP/s", "frac": achieved / PEAK_BF16_TFLOPS,
-                     "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload, {}).get(dominant),
+                     "traffic": (traffic or {}).get(dominant),
                      "flops_per_launch": flops_third, "avg_launch_ms": dom_ms,
-                     "algorithmic_bytes_per_launch": {"fwd": (4 * N + 4 * k) * B * T, "bptt": (4 * N + 4 * k) * B * T,
-                                                      "dw": (4 * N + 4 * k) * B * T}[dominant]},
+                     "algorithmic_bytes_per_launch": (4 * N + 4 * k) * B * T},
         "kernel_ms": kern,
     }
+    if traffic:
+        out["traffic_bytes_per_launch"] = traffic
+        out["traffic_over_algorithmic"] = sum(traffic.values()) / (bytes_per_ss * B * T) if train else None
     if not args.no_cpu:
-        out["cpu_baseline"] = cpu_baseline(cfg, min(args.cpu_sample_batch, B))
+        # the reference's CPU configuration exactly (what cpu_baseline means), then this workload at a reduced batch
+        out["cpu_baseline"] = cpu_baseline(120, 64, 120, 2, "tanh", -1.0 / 120, 1.0, 8.0,
+                                           "the reference's CPU configuration (LeakyRingAttractor no-gain) at its full size")
+        sb = min(args.cpu_sample_batch, B)
+        out["cpu_baseline_workload"] = cpu_baseline(
+            N, sb, T, k, cfg["act"], cfg["J0"], cfg["J1"], 10.0,
+            f"this workload at batch {sb} of {B} (the full batch would need B*N^2*4*T bytes of saved W_eff)")
     print(json.dumps(out))
 
 

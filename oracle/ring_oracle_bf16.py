@@ -48,7 +48,7 @@ def round_u8_dact(x):
 
 def forward_backward(A, Wa, J0, J1, Wo, r_init, alpha, activation_name, grad_output=None, rounding=True,
                      folded=False, dact="fp16"):
-    """Returns dict(bump_history [T,B,N], and, when grad_output is given, grad_Wa, grad_Wo, grad_r_init).
+    """Returns dict(bump_history [T,B,N], and, when grad_output is given, grad_Wa, grad_Wo, grad_r_init, grad_A).
     folded: model of the weight-resident kernels, whose bf16 Wo operand is round(J1 * Wo + J0) (formed in fp32), so
     that J0 * sum_j x_j + J1 * (x Wo^T) is one product over the bf16 operand copy of x; otherwise (the streaming
     kernels) Wo is rounded alone, J1 is applied in fp32 and the J0 row sums run over the fp32 values.
@@ -67,9 +67,11 @@ def forward_backward(A, Wa, J0, J1, Wo, r_init, alpha, activation_name, grad_out
     hist = np.empty((T, B, N))
     D = np.empty((T, B, N))
     R = np.empty((T, B, N))
+    Rfull = np.empty((T, B, N))
     for t in range(T):
         rb = rb16(r)
         R[t] = rb
+        Rfull[t] = r
         re = rb @ Wof.T if folded else J0 * r.sum(axis=1, keepdims=True) + J1 * (rb @ Wob.T)
         for c in range(k):
             re = re + A[:, t, c:c + 1] * (rb @ Wab[c].T)
@@ -82,6 +84,7 @@ def forward_backward(A, Wa, J0, J1, Wo, r_init, alpha, activation_name, grad_out
     G_out = np.asarray(grad_output, np.float64)
     grad_Wo = np.zeros_like(Wo)
     grad_Wa = np.zeros_like(Wa)
+    grad_A = np.zeros((B, T, k))
     carry = np.zeros((B, N))
     for t in range(T - 1, -1, -1):
         G = G_out[t] + carry
@@ -92,9 +95,12 @@ def forward_backward(A, Wa, J0, J1, Wo, r_init, alpha, activation_name, grad_out
         else:
             carry = (1.0 - alpha) * G + J0 * g.sum(axis=1, keepdims=True) + J1 * (gb @ Wob)
         for c in range(k):
-            carry = carry + A[:, t, c:c + 1] * (gb @ Wab[c])
+            pc = gb @ Wab[c]
+            carry = carry + A[:, t, c:c + 1] * pc
+            # dL/dA: the per-matrix product dotted with r_prev (the weight-resident kernels read its bf16 copy)
+            grad_A[:, t, c] = (pc * (R[t] if folded else Rfull[t])).sum(axis=1)
         grad_Wo += J1 * (gb.T @ R[t])
         for c in range(k):
             grad_Wa[c] += rb16(A[:, t, c:c + 1] * gb).T @ R[t]
-    out.update(grad_Wo=grad_Wo, grad_Wa=grad_Wa, grad_r_init=carry)
+    out.update(grad_Wo=grad_Wo, grad_Wa=grad_Wa, grad_r_init=carry, grad_A=grad_A)
     return out

@@ -161,6 +161,18 @@ __device__ __forceinline__ float row16_sum(float v) {
   return v;
 }
 
+// The same sum with data-parallel-primitive adds (no LDS traffic): butterfly inside each row of 16 lanes.
+__device__ __forceinline__ float row16_sum_dpp(float v) {
+#define RING_DPP_ADD(CTRL) \
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, false))
+  RING_DPP_ADD(0xB1);    // quad_perm [1,0,3,2]
+  RING_DPP_ADD(0x4E);    // quad_perm [2,3,0,1]
+  RING_DPP_ADD(0x141);   // row_half_mirror
+  RING_DPP_ADD(0x140);   // row_mirror
+#undef RING_DPP_ADD
+  return v;
+}
+
 // LDS operand buffer: slot(kc,q,b) = (kc*4+q)*XG + b holds the 8 bf16 values
 // x[b][32kc+8q .. +7]; an MFMA A-operand read by lane (q,b) is slot(kc,q,b): each group of 16 lanes
 // reads 256 contiguous bytes.  This writes the lane's [4 rows][NC neurons] fp32 values as bf16.

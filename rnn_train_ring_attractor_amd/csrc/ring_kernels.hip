@@ -1025,7 +1025,7 @@ hipError_t ring_launch_bptt(const RingBpttArgs& a, int NCv, hipStream_t st) {
   ProfScope prof(3, st);
   hipError_t e = hipErrorInvalidValue;
   // (the parentheses keep the commas of the template argument lists away from the dispatch macros)
-  if (a.grad_A) {   // the generic kernel is the one that also produces dL/dA
+  if (a.grad_A && !ring_uses_resident(a.N, a.k)) {   // the streaming kernel's dL/dA variant
     const size_t ga = (size_t)2 * a.k * 64 * sizeof(float);
     if (weights_fit_lds(NCv, a.k, 8 * 1024 + ga)) {
       RING_DISPATCH_NC(NCv, if constexpr (NC <= 2) (e = launch_bptt_stream<NC, true, 1, true>(

@@ -22,9 +22,10 @@ struct RingBpttArgs {
   const float* grad_out; // [T,B,N]
   const _Float16* dfrag;
   __bf16* gfrag;         // bf16 g in tile order (output)
+  const __bf16* rfrag;   // bf16 r_prev in tile order (the forward's operand copy); read for grad_A by the weight-resident kernel
   float* grad_r_init;    // [B,N] or null
-  float* grad_A;         // [B,T,k] or null (written, not accumulated); needs hist and r_init
-  const float* hist;     // [T,B,N] state history (r_prev of step t is hist[t-1]); only read for grad_A
+  float* grad_A;         // [B,T,k] or null (written, not accumulated); needs hist and r_init (streaming kernel) or rfrag
+  const float* hist;     // [T,B,N] state history (r_prev of step t is hist[t-1]); read for grad_A and by the fused loss head
   const float* r_init;   // [B,N]
   // Loss head fused into the weight-resident BPTT kernel (null: grad_out is read).  loss_coef[t*B + b] holds the
   // row's (kc, ks, beta, -) as ring_loss_stats/rows/decode left them; the kernel then reads hist, not grad_out.

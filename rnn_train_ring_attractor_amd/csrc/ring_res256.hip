@@ -18,8 +18,9 @@ constexpr int R_KCH = 8;
 constexpr int R_WLDS_SLOTS = 4 * R_NC * R_KCH * 64;   // 16-byte slots of the LDS-resident matrix
 constexpr int R_XSLOTS = R_KCH * 4 * XG;
 constexpr int R_GCH = 32;                             // time steps of action gates staged per LDS chunk
-constexpr int R_BPTT_DEPTH = 2;                       // BPTT steps whose grad_output / F' loads are in flight
-constexpr size_t R_LDS_BYTES = (size_t)(R_WLDS_SLOTS + 2 * R_XSLOTS) * 16 + 2 * R_GCH * 16 * 8;   // BPTT layout
+constexpr int R_BPTT_DEPTH_MAX = 4;                   // BPTT steps whose grad_output / F' loads are in flight (template DEPTH <= this)
+constexpr size_t R_GA_BYTES = 2 * 2 * 4 * 16 * sizeof(float);   // dL/dA shares: [step parity][channel][wave][row]
+constexpr size_t R_LDS_BYTES = (size_t)(R_WLDS_SLOTS + 2 * R_XSLOTS) * 16 + 2 * R_GCH * 16 * 8 + R_GA_BYTES;   // BPTT layout
 
 // Action gates (A[b,t,0], A[b,t,1]) reach the lanes through LDS in chunks of R_GCH steps, so the
 // time loop issues no vector-memory load whose wait would also drain the history stores.
@@ -336,17 +337,19 @@ __global__ __launch_bounds__(512) void ring_fwd_res256_kernel(RingFwdArgs p) {
 
 // ------------------------------------------------------------------------------------------------
 // BPTT recurrence, transposed weights resident.  Same contract as ring_bptt_kernel<4> with k == 2.
-// grad_output and F' are prefetched R_BPTT_DEPTH steps ahead into register stages (loop unrolled to match).
+// grad_output and F' are prefetched DEPTH steps ahead into register stages (loop unrolled to match).
 // ------------------------------------------------------------------------------------------------
 namespace {
 
 // One step's inputs in flight: grad_output rows (4 x 16 B) and the saved F' record (2 x 16 B, fp16).  With the
 // loss head fused in (LOSS) the rows are those of the state history instead and C holds the four rows' loss
 // coefficients (kc, ks, beta, -), from which the kernel forms grad_output itself.
+// With dL/dA requested (GA), R holds the bf16 operand copy of r_prev for the lane's four neurons (4 rows each).
 struct BpttStage {
   f32x4 G[4];
   f32x4 D[2];
   f32x4 C[4];
+  f32x2 R[4];
 };
 
 // In the unmasked variant the loads of a stage are issued with inline assembly and waited for
@@ -376,9 +379,31 @@ __device__ __forceinline__ f32x4 async_load16_s(const void* uniform_base, unsign
   return v;
 }
 
-template <int K, bool LOSS>
+template <int IMM>
+__device__ __forceinline__ f32x2 async_load8_s(const void* uniform_base, unsigned lane_off) {
+  f32x2 v;
+  asm volatile(".Lring_async_load_%=:\n\tglobal_load_dwordx2 %0, %1, %2 offset:%3 nt"
+               : "=&v"(v)
+               : "v"(lane_off), "s"(uniform_base), "n"(IMM)
+               : "memory");
+  return v;
+}
+
+template <int K, bool LOSS, bool GA>
 __device__ __forceinline__ void bptt_stage_wait(BpttStage& s) {
-  if constexpr (LOSS) {
+  if constexpr (LOSS && GA) {
+    asm volatile(".Lring_async_wait_%=:\n\ts_waitcnt vmcnt(%14)"
+                 : "+v"(s.G[0]), "+v"(s.G[1]), "+v"(s.G[2]), "+v"(s.G[3]), "+v"(s.D[0]), "+v"(s.D[1]), "+v"(s.C[0]),
+                   "+v"(s.C[1]), "+v"(s.C[2]), "+v"(s.C[3]), "+v"(s.R[0]), "+v"(s.R[1]), "+v"(s.R[2]), "+v"(s.R[3])
+                 : "n"(K)
+                 : "memory");
+  } else if constexpr (GA) {
+    asm volatile(".Lring_async_wait_%=:\n\ts_waitcnt vmcnt(%10)"
+                 : "+v"(s.G[0]), "+v"(s.G[1]), "+v"(s.G[2]), "+v"(s.G[3]), "+v"(s.D[0]), "+v"(s.D[1]), "+v"(s.R[0]),
+                   "+v"(s.R[1]), "+v"(s.R[2]), "+v"(s.R[3])
+                 : "n"(K)
+                 : "memory");
+  } else if constexpr (LOSS) {
     asm volatile(".Lring_async_wait_%=:\n\ts_waitcnt vmcnt(%10)"
                  : "+v"(s.G[0]), "+v"(s.G[1]), "+v"(s.G[2]), "+v"(s.G[3]), "+v"(s.D[0]), "+v"(s.D[1]), "+v"(s.C[0]),
                    "+v"(s.C[1]), "+v"(s.C[2]), "+v"(s.C[3])
@@ -392,7 +417,7 @@ __device__ __forceinline__ void bptt_stage_wait(BpttStage& s) {
   }
 }
 
-template <bool FULL, bool LOSS>
+template <bool FULL, bool LOSS, bool GA>
 __device__ __forceinline__ void bptt_stage_load(const RingBpttArgs& p, int t, int bt, int w, int lane, int b0, int i0,
                                                 BpttStage& s) {
   if (t < 0) t = 0;   // redundant reload past the start of the sequence; never consumed
@@ -440,6 +465,28 @@ __device__ __forceinline__ void bptt_stage_load(const RingBpttArgs& p, int t, in
   }
 }
 
+// The r_prev part of a stage (dL/dA only).  It is consumed during the step's products, after the refill of the
+// rest of the stage has been issued, so it is refilled separately at the end of the step: a refill before its
+// last use would need a register copy of values that are still in flight.
+template <bool FULL>
+__device__ __forceinline__ void bptt_stage_load_r(const RingBpttArgs& p, int t, int bt, int w, int lane, BpttStage& s) {
+  if (t < 0) t = 0;
+  if constexpr (FULL) {
+    // the half (t % 2) of the pair slots of the wave's four tiles, 1 KiB apart
+    const int ws = __builtin_amdgcn_readfirstlane(w);
+    const __bf16* rtile = p.rfrag + pair_offset<R_NC>(t, p.nbt, bt, ws * R_NC, 0);       // uniform
+    const unsigned roff = (unsigned)lane * 16u;
+    s.R[0] = async_load8_s<0>(rtile, roff);
+    s.R[1] = async_load8_s<1024>(rtile, roff);
+    s.R[2] = async_load8_s<2048>(rtile, roff);
+    s.R[3] = async_load8_s<3072>(rtile, roff);
+  } else {
+#pragma unroll
+    for (int c = 0; c < R_NC; ++c)
+      s.R[c] = *reinterpret_cast<const f32x2*>(p.rfrag + pair_offset<R_NC>(t, p.nbt, bt, w * R_NC + c, lane));
+  }
+}
+
 // F' of neuron c, rows e = 0..3: the record is [c][e] in fp16.
 __device__ __forceinline__ float stage_dact(const BpttStage& s, int e, int c) {
   const f16x4 h = __builtin_bit_cast(f16x4, f32x2{s.D[c >> 1][2 * (c & 1)], s.D[c >> 1][2 * (c & 1) + 1]});
@@ -454,19 +501,34 @@ __device__ __forceinline__ float stage_dact(const BpttStage& s, int e, int c) {
 // MERGE (needs FULL and an even T): the operand copy of g pairs time steps 2j and 2j+1 in one 16-byte slot per
 // lane; the kernel walks down through 2j+1 and 2j in one trip of its unrolled loop, keeps the first in registers
 // and writes both with one 16-byte store per tile (whole cache lines, half as many store instructions).
-template <bool FULL, bool LOSS, bool MERGE>
+// DEPTH: steps whose inputs are in flight (register stages); even, so that a trip of the unrolled loop holds whole pairs.
+// GA: also write grad_A[b,t,c] = sum_j (g Wa[c])[j] * r_prev[j], c = 0, 1: the per-matrix products of the step are
+// dotted with the bf16 operand copy of r_prev (the forward's, read with the step's other inputs), summed over the
+// row group's 16 lanes with data-parallel adds, over the four waves through LDS in wave order, and written out
+// after the next step's barrier.
+template <bool FULL, bool LOSS, bool MERGE, int DEPTH, bool GA>
 __global__ __launch_bounds__(256) void ring_bptt_res256_kernel(RingBpttArgs p) {
-  static_assert(!MERGE || (FULL && R_BPTT_DEPTH == 2), "merged pair stores need the unmasked two-step loop");
+  static_assert(DEPTH % 2 == 0 && DEPTH <= R_BPTT_DEPTH_MAX, "the unrolled loop walks whole step pairs");
+  static_assert(!MERGE || FULL, "merged pair stores need the unmasked loop");
   extern __shared__ __attribute__((aligned(16))) char smem[];
   bf16x8* wlds = reinterpret_cast<bf16x8*>(smem);
   bf16x8* xbuf = wlds + R_WLDS_SLOTS;
   f32x2* gbuf = reinterpret_cast<f32x2*>(xbuf + 2 * R_XSLOTS);
+  float* gabuf = reinterpret_cast<float*>(gbuf + 2 * R_GCH * 16);   // [step parity][channel][wave][row]
 
   const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, q = lane >> 4, n = lane & 15;
   const int bt = blockIdx.x;
   const int b0 = 16 * bt + 4 * q;
   const int i0 = 16 * R_NC * w + R_NC * n;
   const int N = p.N, B = p.B, T = p.T;
+  // dL/dA of step t from the shares the four waves left in buffer `par` (call after a barrier that follows them)
+  auto flush_grad_A = [&](int t, int par) {
+    if (tid < 32) {
+      const int ch = tid >> 4, row = tid & 15, b = 16 * bt + row;
+      const float* sh = gabuf + (par * 2 + ch) * 64 + row;
+      if (b < B) p.grad_A[((size_t)b * T + t) * 2 + ch] = ((sh[0] + sh[16]) + sh[32]) + sh[48];
+    }
+  };
   const float oma = 1.f - p.alpha;   // alpha rides in the saved F' record, J0 and J1 in the packed Wo fragments
   const int wu = __builtin_amdgcn_readfirstlane(w);   // the wave index as a scalar, for address arithmetic
 
@@ -496,9 +558,12 @@ __global__ __launch_bounds__(256) void ring_bptt_res256_kernel(RingBpttArgs p) {
   }
 
   pair_zero_tail<R_NC>(p.gfrag, T, p.nbt, bt, w, lane);
-  BpttStage st[R_BPTT_DEPTH];
+  BpttStage st[DEPTH];
 #pragma unroll
-  for (int d = 0; d < R_BPTT_DEPTH; ++d) bptt_stage_load<FULL, LOSS>(p, T - 1 - d, bt, w, lane, b0, i0, st[d]);
+  for (int d = 0; d < DEPTH; ++d) {
+    bptt_stage_load<FULL, LOSS, GA>(p, T - 1 - d, bt, w, lane, b0, i0, st[d]);
+    if constexpr (GA) bptt_stage_load_r<FULL>(p, T - 1 - d, bt, w, lane, st[d]);
+  }
   GateStage gs;
   gates_fetch(p.A, T, B, bt, 0, -1, tid, gs);
   gates_publish(gbuf, tid, B, bt, gs);
@@ -508,28 +573,31 @@ __global__ __launch_bounds__(256) void ring_bptt_res256_kernel(RingBpttArgs p) {
   // (the first lds_barrier inside the loop also publishes the gates)
 
   bf16x4 held[R_NC];   // MERGE: the odd step's bf16 g, waiting for its even partner
-  for (int u0 = 0; u0 < T; u0 += R_BPTT_DEPTH) {
+  for (int u0 = 0; u0 < T; u0 += DEPTH) {
 #pragma unroll
-    for (int half = 0; half < R_BPTT_DEPTH; ++half) {
+    for (int half = 0; half < DEPTH; ++half) {
       const int u = u0 + half;
       if (u >= T) break;
       const int t = T - 1 - u;
       const int cur = u & 1, ci = u / R_GCH, l = u % R_GCH;
       if (l == 0 && (ci + 1) * R_GCH < T) gates_fetch(p.A, T, B, bt, ci + 1, -1, tid, gs);
       BpttStage& S = st[half];
-      // issued after this stage's six loads: per step since then, four operand-copy stores and another
-      // stage's six loads.  The counter is in order, so "at most 10 * (depth - 1) outstanding" means this
-      // stage landed; a smaller number would also wait for later loads and for store acknowledgements.
-      // (with the loss head fused in a stage has four more loads: 14 per step)
-      // With merged pair stores the four stores all sit in the second step of a trip: the first step's stage
-      // sees them and the other stage's loads behind it, the second step's stage only the other stage's loads.
+      // Issued after this stage's loads (six; ten with the loss head fused in), in order: per later step its
+      // operand-copy stores and then another stage's loads.  The counter is in order, so once no more than that
+      // many operations are outstanding this stage has landed; a smaller number would also wait for later loads
+      // and for store acknowledgements.  Unmerged, every step issues four stores.  With merged pair stores the
+      // four stores sit in the second step of each pair (odd `half`): the steps since this stage was loaded are
+      // half - DEPTH + 1 .. half - 1, of which DEPTH / 2 are odd when `half` is even and DEPTH / 2 - 1 otherwise.
+      // (with dL/dA: four more loads per stage, and the one store of the previous step's dL/dA, issued by some waves
+      // only, which makes the bound conservative for the others: it can only wait for more)
+      constexpr int LOADS = 6 + (LOSS ? 4 : 0) + (GA ? 4 : 0);
       if constexpr (MERGE) {
-        constexpr int LOADS = LOSS ? 10 : 6;
-        if (half == 0) bptt_stage_wait<LOADS + 4, LOSS>(S);
-        else bptt_stage_wait<LOADS, LOSS>(S);
+        if ((half & 1) == 0) bptt_stage_wait<LOADS * (DEPTH - 1) + 4 * (DEPTH / 2), LOSS, GA>(S);
+        else bptt_stage_wait<LOADS * (DEPTH - 1) + 4 * (DEPTH / 2 - 1), LOSS, GA>(S);
       } else if constexpr (FULL) {
-        bptt_stage_wait<(LOSS ? 14 : 10) * (R_BPTT_DEPTH - 1), LOSS>(S);
+        bptt_stage_wait<(LOADS + 4) * (DEPTH - 1), LOSS, GA>(S);
       }
+      // (the stage's r_prev part is issued last in a step, behind everything counted above, and used in place)
 
       float G[4][R_NC], g[4][R_NC];
 #pragma unroll
@@ -562,7 +630,7 @@ __global__ __launch_bounds__(256) void ring_bptt_res256_kernel(RingBpttArgs p) {
         for (int c = 0; c < R_NC; ++c) {
           const bf16x4 pk = {(__bf16)g[0][c], (__bf16)g[1][c], (__bf16)g[2][c], (__bf16)g[3][c]};
           if constexpr (MERGE) {
-            if (half == 0) {
+            if ((half & 1) == 0) {
               held[c] = pk;            // t is odd here (T even): the slot's second half, written with the first
             } else {
               const bf16x8 both = __builtin_shufflevector(pk, held[c], 0, 1, 2, 3, 4, 5, 6, 7);
@@ -573,8 +641,12 @@ __global__ __launch_bounds__(256) void ring_bptt_res256_kernel(RingBpttArgs p) {
           }
         }
       }
-      bptt_stage_load<FULL, LOSS>(p, t - R_BPTT_DEPTH, bt, w, lane, b0, i0, S);
+      bptt_stage_load<FULL, LOSS, GA>(p, t - DEPTH, bt, w, lane, b0, i0, S);
       lds_barrier();
+      if constexpr (GA) {
+        if (u > 0) flush_grad_A(t + 1, cur ^ 1);   // the previous step's shares are complete behind this barrier
+      }
+      float ga[2][4] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
 
       bf16x8 af[R_KCH];
 #pragma unroll
@@ -613,6 +685,27 @@ __global__ __launch_bounds__(256) void ring_bptt_res256_kernel(RingBpttArgs p) {
           if constexpr (!FULL) x *= okf[e][c];
           carry[e][c] = x;
         }
+        if constexpr (GA) {
+          const bf16x4 rp = __builtin_bit_cast(bf16x4, S.R[c]);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const float rv = (float)rp[e];
+            ga[0][e] = fmaf(P1[e], rv, ga[0][e]);
+            ga[1][e] = fmaf(P2[e], rv, ga[1][e]);
+          }
+        }
+      }
+      if constexpr (GA) {
+        // the other parity's buffer is being read by this step's flush; this one was read one step ago, before
+        // the barrier above
+#pragma unroll
+        for (int ch = 0; ch < 2; ++ch)
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const float tot = row16_sum_dpp(ga[ch][e]);
+            if (n == 0) gabuf[((cur * 2 + ch) * 4 + w) * 16 + 4 * q + e] = tot;
+          }
+        bptt_stage_load_r<FULL>(p, t - DEPTH, bt, w, lane, S);
       }
       // the next iteration overwrites the other operand buffer and, every R_GCH steps, the other
       // gate chunk; both were last read before the barrier above, so no second barrier is needed
@@ -623,7 +716,11 @@ __global__ __launch_bounds__(256) void ring_bptt_res256_kernel(RingBpttArgs p) {
   // while their destination registers are still reserved, before anything below reuses them
   if constexpr (FULL) {
 #pragma unroll
-    for (int d = 0; d < R_BPTT_DEPTH; ++d) bptt_stage_wait<0, LOSS>(st[d]);
+    for (int d = 0; d < DEPTH; ++d) bptt_stage_wait<0, LOSS, GA>(st[d]);
+  }
+  if constexpr (GA) {
+    lds_barrier();
+    flush_grad_A(0, (T - 1) & 1);
   }
   if (p.grad_r_init) rows_store<R_NC>(p.grad_r_init, N, B, b0, i0, carry);
 }
@@ -660,9 +757,9 @@ hipError_t ring_launch_fwd_res256(const RingFwdArgs& a, hipStream_t st) {
   }
 }
 
-template <bool FULL, bool LOSS, bool MERGE>
+template <bool FULL, bool LOSS, bool MERGE, int DEPTH, bool GA>
 static hipError_t launch_bptt_variant(const RingBpttArgs& a, hipStream_t st) {
-  auto kern = ring_bptt_res256_kernel<FULL, LOSS, MERGE>;
+  auto kern = ring_bptt_res256_kernel<FULL, LOSS, MERGE, DEPTH, GA>;
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                                      (int)R_LDS_BYTES);
   if (e != hipSuccess) return e;
@@ -670,13 +767,24 @@ static hipError_t launch_bptt_variant(const RingBpttArgs& a, hipStream_t st) {
   return hipGetLastError();
 }
 
-hipError_t ring_launch_bptt_res256(const RingBpttArgs& a, hipStream_t st) {
+// Two steps of inputs in flight.  (Four, which the unmasked kernel that reads grad_output has the registers for,
+// measured the same: the kernel does not wait for its loads.)
+template <bool GA>
+static hipError_t launch_bptt_ga(const RingBpttArgs& a, hipStream_t st) {
   const bool full = (a.N == 256) && (a.B % 16 == 0);
   const bool merge = full && (a.T % 2 == 0);
   if (a.loss_coef) {
-    if (merge) return launch_bptt_variant<true, true, true>(a, st);
-    return full ? launch_bptt_variant<true, true, false>(a, st) : launch_bptt_variant<false, true, false>(a, st);
+    if (merge) return launch_bptt_variant<true, true, true, 2, GA>(a, st);
+    return full ? launch_bptt_variant<true, true, false, 2, GA>(a, st) : launch_bptt_variant<false, true, false, 2, GA>(a, st);
   }
-  if (merge) return launch_bptt_variant<true, false, true>(a, st);
-  return full ? launch_bptt_variant<true, false, false>(a, st) : launch_bptt_variant<false, false, false>(a, st);
+  if (merge) return launch_bptt_variant<true, false, true, 2, GA>(a, st);
+  return full ? launch_bptt_variant<true, false, false, 2, GA>(a, st) : launch_bptt_variant<false, false, false, 2, GA>(a, st);
+}
+
+hipError_t ring_launch_bptt_res256(const RingBpttArgs& a, hipStream_t st) {
+  if (a.grad_A) {
+    if (!a.rfrag) return hipErrorInvalidValue;
+    return launch_bptt_ga<true>(a, st);
+  }
+  return launch_bptt_ga<false>(a, st);
 }

@@ -330,7 +330,7 @@ static int bwd_impl(const char* who, const void* grad_output, const void* loss_w
 
   // the weight-resident BPTT kernel takes J1 * Wo + J0 in the transposed Wo fragments
   const bool resident = ring_uses_resident(N, a_dim);
-  const bool bptt_resident = resident && !grad_A;
+  const bool bptt_resident = resident;
   hipError_t e = hipSuccess;
   if (saved && saved_note_get(saved) == (bptt_resident ? 2 : 1)) {
     // the forward left the transposed copy, in the form this BPTT kernel expects, behind the saved activations
@@ -347,6 +347,7 @@ static int bwd_impl(const char* who, const void* grad_output, const void* loss_w
   b.grad_out = (const float*)grad_output;
   b.dfrag = dfrag;
   b.gfrag = gfrag;
+  b.rfrag = rfrag;
   b.grad_r_init = (float*)grad_r_init;
   b.grad_A = (float*)grad_A;
   b.hist = (const float*)bump_history;

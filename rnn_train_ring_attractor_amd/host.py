@@ -240,14 +240,18 @@ class LeakyRingAttractor(nn.Module):
             left, right = self.gain_l_net(left) * left, self.gain_r_net(right) * right
         return torch.cat([left, right], dim=2)
 
-    def forward(self, av_signal, r_init=None):
+    def forward_history(self, av_signal, r_init=None):
+        """bump_history [T,B,N] as the operator returns it (gain networks, then the time loop; no read-out)."""
         from .ring_rnn_cuda import ring_rnn_cuda_func
         batch_size = av_signal.shape[0]
         if r_init is None:
             angle = torch.full((batch_size,), math.pi, device=self.Wo.device)
             r_init = create_initial_bump(angle, self.num_neurons, device=self.Wo.device)
-        bump = ring_rnn_cuda_func(action_signal=self.action_signal(av_signal), Wa=torch.stack([self.Wl, self.Wr]),
+        return ring_rnn_cuda_func(action_signal=self.action_signal(av_signal), Wa=torch.stack([self.Wl, self.Wr]),
                                   J0=self.J0, J1=self.J1, Wo=self.Wo, r_init=r_init, alpha=0.15,
-                                  activation=self.activation_name).permute(1, 0, 2)
+                                  activation=self.activation_name)
+
+    def forward(self, av_signal, r_init=None):
+        bump = self.forward_history(av_signal, r_init).permute(1, 0, 2)
         proj = bump @ self.W_delta7
         return proj / proj.max(dim=2, keepdim=True)[0], bump

@@ -47,11 +47,13 @@ def _kernel_body(asm, mangled):
     return asm[i:asm.index("s_endpgm", i)].split("\n")
 
 
+@pytest.mark.parametrize("ga", [0, 1], ids=["weights_only", "with_grad_A"])
 @pytest.mark.parametrize("merge", [0, 1], ids=["stores_per_step", "merged_pair_stores"])
 @pytest.mark.parametrize("loss", [0, 1], ids=["grad_output", "fused_loss"])
-def test_async_loads_are_not_touched_before_their_wait(res256_asm, loss, merge):
+def test_async_loads_are_not_touched_before_their_wait(res256_asm, loss, merge, ga):
     asm, _ = res256_asm
-    body = _kernel_body(asm, f"_Z23ring_bptt_res256_kernelILb1ELb{loss}ELb{merge}EEv12RingBpttArgs")
+    depth = 2                           # input stages in flight (the launcher's choice)
+    body = _kernel_body(asm, f"_Z23ring_bptt_res256_kernelILb1ELb{loss}ELb{merge}ELi{depth}ELb{ga}EEv12RingBpttArgs")
     fifo, loads, waits, tag = [], 0, 0, None
     for ln in body + body:                      # second pass models the loop back edge
         t = ln.strip()
@@ -64,7 +66,7 @@ def test_async_loads_are_not_touched_before_their_wait(res256_asm, loss, merge):
         if not t or t[0] in ";.":
             continue
         if tag == "load":
-            assert t.startswith("global_load_dwordx4"), t
+            assert t.startswith(("global_load_dwordx4", "global_load_dwordx2")), t
             fifo.append(_regs(t.split()[1].rstrip(",")))
             loads += 1
             tag = None

@@ -183,15 +183,18 @@ def test_backward_without_saved_buffer_rebuilds_it(case, gpu_device):
 
 
 @pytest.mark.parametrize("B,T,k,N,act,action", [(40, 24, 2, 120, "tanh", "lr"), (48, 20, 2, 256, "gelu", "lr"),
-                                                (21, 9, 3, 200, "silu", "dense"), (32, 12, 16, 64, "tanh", "spread")],
-                         ids=["n120", "n256", "ragged_k3", "k16"])
+                                                (21, 9, 3, 200, "silu", "dense"), (32, 12, 16, 64, "tanh", "spread"),
+                                                (32, 7, 2, 256, "tanh", "dense"), (37, 10, 2, 200, "silu", "dense"),
+                                                (64, 66, 2, 256, "relu", "lr")],
+                         ids=["n120", "n256", "ragged_k3", "k16", "n256_odd_T", "n200_ragged_resident", "n256_relu_T66"])
 def test_gradients_of_action_signal_and_initial_state(B, T, k, N, act, action, gpu_device):
     """dL/d action_signal and dL/d r_init, which the reference operator does not return (cpp/ring_rnn_cuda.py:144);
     pinned by the fp64 oracle, whose grad_A / grad_r_init are themselves checked by finite differences."""
     from rnn_train_ring_attractor_amd import ring_rnn_cuda_func
     print(f"[case] grad_A B={B} T={T} k={k} N={N} {act}", flush=True)
     p = _problem(400, B, T, k, N, action)
-    J0, J1 = -0.05, 0.4
+    # (relu with strong inhibition silences every neuron and all gradients are exactly zero: weak inhibition there)
+    J0, J1 = (-1.0 / N, 1.0) if act == "relu" else (-0.05, 0.4)
     A = _dev(p["A"], gpu_device).requires_grad_(True)
     r0 = _dev(p["r0"], gpu_device).requires_grad_(True)
     Wa = _dev(p["Wa"], gpu_device).requires_grad_(True)
@@ -201,12 +204,20 @@ def test_gradients_of_action_signal_and_initial_state(B, T, k, N, act, action, g
     torch.cuda.synchronize()
     ref_hist, _ = O.forward_dense(p["A"], p["Wa"], J0, J1, p["Wo"], p["r0"], 0.15, act)
     ref = O.backward_dense(p["G"], p["A"], p["Wa"], J0, J1, p["Wo"], ref_hist, p["r0"], 0.15, act)
+    model = OB.forward_backward(p["A"], p["Wa"], J0, J1, p["Wo"], p["r0"], 0.15, act, p["G"], folded=_folded(N, k))
     for name, got, want in (("grad_A", A.grad, ref["grad_A"]), ("grad_r_init", r0.grad, ref["grad_r_init"]),
                             ("grad_Wo", Wo.grad, ref["grad_Wo"]), ("grad_Wa", Wa.grad, ref["grad_Wa"])):
         got = got.cpu().numpy()
         assert got.shape == want.shape and np.isfinite(got).all(), name
-        assert O.cosine(got, want) >= GRAD_COS, name
-        assert O.max_rel_err(got, want) <= GRAD_TOL, name
+        assert np.abs(want).max() > 0, name
+        if act == "relu":
+            # per-sample gradients do not average the derivative flips at the kink (see the note at the top): the
+            # fp64 comparison is by cosine, the entry-wise bound is against the rounding-aware model
+            assert O.cosine(got, want) >= 0.995, name
+            assert O.max_rel_err(got, model[name]) <= GRAD_TOL, name
+        else:
+            assert O.cosine(got, want) >= GRAD_COS, name
+            assert O.max_rel_err(got, want) <= GRAD_TOL, name
 
 
 def test_gradients_accumulate_and_are_deterministic(gpu_device):

@@ -32,7 +32,7 @@ def test_without_rounding_it_is_the_fp64_oracle(act):
     hist, _ = O.forward_dense(p["A"], p["Wa"], -0.1, 0.1, p["Wo"], p["r0"], 0.15, act)
     ref = O.backward_dense(p["G"], p["A"], p["Wa"], -0.1, 0.1, p["Wo"], hist, p["r0"], 0.15, act)
     np.testing.assert_allclose(got["bump_history"], hist, rtol=0, atol=1e-13)
-    for key in ("grad_Wo", "grad_Wa", "grad_r_init"):
+    for key in ("grad_Wo", "grad_Wa", "grad_r_init", "grad_A"):
         np.testing.assert_allclose(got[key], ref[key], rtol=0, atol=1e-11, err_msg=key)
 
 
