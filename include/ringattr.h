@@ -141,6 +141,22 @@ RINGATTR_API int ringattr_bwd_loss(const void* loss_workspace, const void* upstr
                       const void* saved, void* grad_A, void* grad_r_init,
                       void* workspace, size_t workspace_bytes, void* stream);
 
+/* Gain networks of the action signal, forward and backward.  Replaces the per-channel nn.Sequential(Linear(1,h), GELU,
+ * Linear(h,1), Softplus) evaluation and its autograd in the reference models (train/train_ring_attractor.py:70-79,
+ * 136-146; train/train_general_ring_attractor.py:38-46, 99-109): per sample, step and channel c
+ *   A[b,t,c] = x * softplus(sum_j w2[c][j] * gelu(w1[c][j] * |x| + b1[c][j]) + b2[c]),   x = base_signal[b,t,c].
+ * The networks depend only on the input signal, so they run once for all (b, t) in front of the time loop.
+ *   base_signal, action_signal, grad_action_signal, grad_base_signal  [B,T,k] fp32
+ *   params, grad_params  [k][3*hidden + 1] fp32, per channel [w1 | b1 | w2 | b2]
+ * ringattr_gain_bwd overwrites grad_params with the sums over all B*T samples (fixed summation order: repeatable
+ * bit for bit) and, when grad_base_signal is not NULL, writes dL/d base_signal.  hidden <= 32, a_dim <= 64. */
+RINGATTR_API size_t ringattr_gain_workspace_bytes(int a_dim, int hidden, int seq_len, int batch_size);
+RINGATTR_API int ringattr_gain_fwd(const void* base_signal, const void* params, void* action_signal,
+                      int a_dim, int hidden, int seq_len, int batch_size, void* stream);
+RINGATTR_API int ringattr_gain_bwd(const void* base_signal, const void* params, const void* grad_action_signal,
+                      void* grad_params, void* grad_base_signal, int a_dim, int hidden, int seq_len, int batch_size,
+                      void* workspace, size_t workspace_bytes, void* stream);
+
 /* Per-kernel timing for benchmarks; no counterpart in the reference.  While enabled, every kernel
  * launch is bracketed by two HIP events recorded on the launch stream.  ringattr_profile_read waits
  * for the recorded events, adds their durations into ms[RINGATTR_NUM_KERNELS] and the launch counts

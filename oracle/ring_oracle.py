@@ -352,3 +352,45 @@ def loss_pair_rank2(bump_tbn, target_angle, bump_weight=0.2, target_amplitude=No
     beta = beta * bump_weight / rows
     grad = kc[..., None] * np.cos(phi) + ks[..., None] * np.sin(phi) + beta[..., None] * np.sign(r)
     return cos_loss + bump_weight * amp_loss, cos_loss, amp_loss, grad
+
+
+# ---------------------------------------------------------------------------------------------------
+# Gain networks of the action signal (train/train_ring_attractor.py:70-79, 136-146;
+# train/train_general_ring_attractor.py:38-46, 99-109): per channel c a network
+# Linear(1,h) -> GELU (exact erf) -> Linear(h,1) -> Softplus (beta 1, threshold 20) on |x|, and A = x * gain.
+# params[c] = [w1[0..h) | b1[0..h) | w2[0..h) | b2].
+# ---------------------------------------------------------------------------------------------------
+def _gain_internals(x, params):
+    x = np.asarray(x, np.float64)
+    params = np.asarray(params, np.float64)
+    h = (params.shape[1] - 1) // 3
+    w1, b1, w2, b2 = params[:, :h], params[:, h:2 * h], params[:, 2 * h:3 * h], params[:, 3 * h]
+    m = np.abs(x)
+    u = m[..., None] * w1 + b1                              # [B,T,k,h]
+    a = activation(u, "gelu")
+    z = (a * w2).sum(axis=-1) + b2                          # [B,T,k]
+    s = np.where(z > 20.0, z, np.log1p(np.exp(np.minimum(z, 20.0))))
+    ds = np.where(z > 20.0, 1.0, 1.0 / (1.0 + np.exp(-np.minimum(z, 20.0))))
+    return x, m, u, a, z, s, ds, w1, w2
+
+
+def gain_forward(x, params):
+    """[B,T,k] base signal, [k,3h+1] parameters -> [B,T,k] gated signal x * softplus(net(|x|))."""
+    x, _, _, _, _, s, _, _, _ = _gain_internals(x, params)
+    return x * s
+
+
+def gain_backward(x, params, grad_A):
+    """Returns (grad_params [k,3h+1], grad_x [B,T,k]) of sum(grad_A * gain_forward(x, params))."""
+    x, m, u, a, z, s, ds, w1, w2 = _gain_internals(x, params)
+    g = np.asarray(grad_A, np.float64)
+    dz = g * x * ds                                          # [B,T,k]
+    du = dz[..., None] * w2 * activation_derivative(u, "gelu")
+    gw2 = (dz[..., None] * a).sum(axis=(0, 1))
+    gb2 = dz.sum(axis=(0, 1))
+    gb1 = du.sum(axis=(0, 1))
+    gw1 = (du * m[..., None]).sum(axis=(0, 1))
+    grad_params = np.concatenate([gw1, gb1, gw2, gb2[:, None]], axis=1)
+    dm = (du * w1).sum(axis=-1)
+    grad_x = g * s + np.sign(x) * dm
+    return grad_params, grad_x

@@ -81,6 +81,12 @@ hipError_t ring_launch_loss_bwd(const float* hist, const float* angle, const flo
 // the per-row coefficients (kc, ks, beta, -) inside a workspace that ring_launch_loss_fwd filled
 const ring_f32x4* ring_loss_row_coefficients(const void* workspace);
 
+// Gain networks of the action signal (ring_gain.hip): params / grad_params are [k][3h+1] = [w1 | b1 | w2 | b2] per channel.
+size_t ring_gain_workspace_bytes(int k, int h, long samples);
+hipError_t ring_launch_gain_fwd(const float* x, const float* params, float* out, int k, int h, long samples, hipStream_t st);
+hipError_t ring_launch_gain_bwd(const float* x, const float* params, const float* grad_A, float* grad_params, float* grad_x,
+                                int k, int h, long samples, void* workspace, hipStream_t st);
+
 // Optional event bracketing of launches (benchmark support).
 void ring_profile_set(bool on);
 bool ring_profile_on();

@@ -435,6 +435,46 @@ int ringattr_loss_bwd(const void* bump_history, const void* target_angle, const 
   return RINGATTR_OK;
 }
 
+size_t ringattr_gain_workspace_bytes(int a_dim, int hidden, int seq_len, int batch_size) {
+  if (a_dim <= 0 || hidden <= 0 || seq_len <= 0 || batch_size <= 0) {
+    fail(RINGATTR_ERR_INVALID, "a_dim, hidden, seq_len, batch_size must be positive (got %d, %d, %d, %d)", a_dim, hidden,
+         seq_len, batch_size);
+    return 0;
+  }
+  if (hidden > 32 || a_dim > 64) {
+    fail(RINGATTR_ERR_INVALID, "the gain networks support hidden <= 32 and a_dim <= 64 (got %d, %d)", hidden, a_dim);
+    return 0;
+  }
+  return align_up(ring_gain_workspace_bytes(a_dim, hidden, (long)seq_len * batch_size));
+}
+
+int ringattr_gain_fwd(const void* base_signal, const void* params, void* action_signal, int a_dim, int hidden, int seq_len,
+                      int batch_size, void* stream) {
+  if (ringattr_gain_workspace_bytes(a_dim, hidden, seq_len, batch_size) == 0) return RINGATTR_ERR_INVALID;
+  if (!base_signal || !params || !action_signal) return fail(RINGATTR_ERR_INVALID, "ringattr_gain_fwd: null tensor pointer");
+  hipError_t e = ring_launch_gain_fwd((const float*)base_signal, (const float*)params, (float*)action_signal, a_dim, hidden,
+                                      (long)seq_len * batch_size, static_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return hip_fail(e, "gain network forward launch");
+  return RINGATTR_OK;
+}
+
+int ringattr_gain_bwd(const void* base_signal, const void* params, const void* grad_action_signal, void* grad_params,
+                      void* grad_base_signal, int a_dim, int hidden, int seq_len, int batch_size, void* workspace,
+                      size_t workspace_bytes, void* stream) {
+  const size_t need = ringattr_gain_workspace_bytes(a_dim, hidden, seq_len, batch_size);
+  if (need == 0) return RINGATTR_ERR_INVALID;
+  if (!base_signal || !params || !grad_action_signal || !grad_params)
+    return fail(RINGATTR_ERR_INVALID, "ringattr_gain_bwd: null tensor pointer");
+  if (!workspace || workspace_bytes < need)
+    return fail(RINGATTR_ERR_WORKSPACE, "ringattr_gain_bwd: workspace of %zu bytes needed, %zu given", need,
+                workspace ? workspace_bytes : (size_t)0);
+  hipError_t e = ring_launch_gain_bwd((const float*)base_signal, (const float*)params, (const float*)grad_action_signal,
+                                      (float*)grad_params, (float*)grad_base_signal, a_dim, hidden,
+                                      (long)seq_len * batch_size, workspace, static_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return hip_fail(e, "gain network backward launch");
+  return RINGATTR_OK;
+}
+
 int ringattr_profile_enable(int on) {
   ring_profile_set(on != 0);
   return RINGATTR_OK;

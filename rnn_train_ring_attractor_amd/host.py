@@ -234,11 +234,15 @@ class LeakyRingAttractor(nn.Module):
             raise ValueError(f"Unknown initialization type: {initialization}")
 
     def action_signal(self, av_signal):
-        """[B,T] angular velocity -> [B,T,2] gated (L, R) channels."""
+        """[B,T] angular velocity -> [B,T,2] gated (L, R) channels.  On the GPU both gain networks run as one HIP
+        operator (forward and backward); on the CPU (tests of the module itself) as the torch modules they are."""
         left, right = torch.relu(-av_signal).unsqueeze(2), torch.relu(av_signal).unsqueeze(2)
-        if self.gain_l_net is not None:
-            left, right = self.gain_l_net(left) * left, self.gain_r_net(right) * right
-        return torch.cat([left, right], dim=2)
+        if self.gain_l_net is None:
+            return torch.cat([left, right], dim=2)
+        if av_signal.is_cuda:
+            from .gain import pack_gain_nets, ring_gain_func
+            return ring_gain_func(torch.cat([left, right], dim=2), pack_gain_nets([self.gain_l_net, self.gain_r_net]))
+        return torch.cat([self.gain_l_net(left) * left, self.gain_r_net(right) * right], dim=2)
 
     def forward_history(self, av_signal, r_init=None):
         """bump_history [T,B,N] as the operator returns it (gain networks, then the time loop; no read-out)."""

@@ -301,6 +301,125 @@ def test_gain_network_model_trains_through_the_operator(gpu_device):
         assert O.max_rel_err(got, ref) <= 2e-2, n
 
 
+def _gain_model(N, act, dev, seed=5):
+    from rnn_train_ring_attractor_amd import host
+    torch.manual_seed(seed)
+    model = host.LeakyRingAttractor(N, activation=act, initialization="random")
+    model.J0, model.J1 = -1.0 / N, 1.0
+    return model.to(dev)
+
+
+def _gain_oracle(model, av, r0, G, act):
+    """fp64 oracle of the gain-network model on a batch slice: gates, trajectory, weight gradients and the
+    gain-network parameter gradients through dL/d action_signal."""
+    from rnn_train_ring_attractor_amd.gain import pack_gain_nets
+    c = lambda t: t.detach().cpu().numpy().astype(np.float64)
+    params = c(pack_gain_nets([model.gain_l_net, model.gain_r_net]))
+    base = np.stack([np.maximum(-c(av), 0.0), np.maximum(c(av), 0.0)], axis=2)
+    A = O.gain_forward(base, params)
+    Wa = np.stack([c(model.Wl), c(model.Wr)])
+    hist, _ = O.forward_dense(A, Wa, model.J0, model.J1, c(model.Wo), c(r0), 0.15, act)
+    g = O.backward_dense(c(G), A, Wa, model.J0, model.J1, c(model.Wo), hist, c(r0), 0.15, act)
+    gp, _ = O.gain_backward(base, params, g["grad_A"])
+    # the same with the kernels' operand rounding made explicit (weight-resident family): relu's derivative flips
+    model_g = OB.forward_backward(A, Wa, model.J0, model.J1, c(model.Wo), c(r0), 0.15, act, c(G), folded=True)
+    gp_model, _ = O.gain_backward(base, params, model_g["grad_A"])
+    return hist, g, gp, model_g, gp_model
+
+
+def test_gain_network_configuration_at_full_size(gpu_device):
+    """The general ring with gain networks at its benchmark size: N=256, B=4096, T=240, relu, two 1 -> 16 -> 1 gain
+    networks evaluated by the HIP gain operator, BPTT through the weight-resident kernel with dL/d action_signal.
+    A 64-row slice is checked against the fp64 oracle (trajectory, weight gradients, gain-network gradients); the
+    full size by bitwise repeatability, slice invariance and additivity over batch shards."""
+    from rnn_train_ring_attractor_amd import host
+    from rnn_train_ring_attractor_amd.gain import pack_gain_nets
+    print("[case] gain-network configuration N=256 B=4096 T=240 relu (full size)", flush=True)
+    N, B, T, act = 256, 4096, 240, "relu"
+    model = _gain_model(N, act, gpu_device)
+    torch.manual_seed(6)
+    av, angle = host.generate_av_integration_data_ultra_fast(B, T)
+    r0 = host.create_initial_bump(angle[:, 0], N)
+    av, r0 = av.to(gpu_device), r0.to(gpu_device)
+    G = torch.randn(T, B, N, device=gpu_device, generator=torch.Generator(device=gpu_device).manual_seed(8))
+    names = [n for n, _ in model.named_parameters()]
+
+    def run(rows):
+        model.zero_grad()
+        h = model.forward_history(av[rows].contiguous(), r0[rows].contiguous())
+        h.backward(G[:, rows].contiguous())
+        return h.detach(), {n: p.grad.clone() for n, p in model.named_parameters()}
+
+    full, again = run(slice(0, B)), run(slice(0, B))
+    assert torch.equal(full[0], again[0])
+    assert all(torch.equal(full[1][n], again[1][n]) for n in names)
+    assert all(torch.isfinite(full[1][n]).all() for n in names)
+    sl = slice(2048, 2112)
+    part = run(sl)
+    assert torch.equal(part[0], full[0][:, sl])
+    hist, g, gp, model_g, gp_model = _gain_oracle(model, av[sl], r0[sl], G[:, sl], act)
+    c = lambda t: t.cpu().numpy()
+    assert O.max_rel_err(c(part[0]), hist) <= TRAJ_TOL
+    # relu: the derivative flips at the kink (operands rounded to bf16) leave the cosine; entry-wise bounds are
+    # asserted at a realistic batch in test_relu_gradients_against_fp64_at_a_realistic_batch
+    assert O.cosine(c(part[1]["Wo"]), g["grad_Wo"]) >= GRAD_COS
+    assert O.cosine(c(part[1]["Wl"]), g["grad_Wa"][0]) >= GRAD_COS and O.cosine(c(part[1]["Wr"]), g["grad_Wa"][1]) >= GRAD_COS
+    h = 16
+    got_l = np.concatenate([c(part[1]["gain_l_net.0.weight"]).ravel(), c(part[1]["gain_l_net.0.bias"]).ravel(),
+                            c(part[1]["gain_l_net.2.weight"]).ravel(), c(part[1]["gain_l_net.2.bias"]).ravel()])
+    got_r = np.concatenate([c(part[1]["gain_r_net.0.weight"]).ravel(), c(part[1]["gain_r_net.0.bias"]).ravel(),
+                            c(part[1]["gain_r_net.2.weight"]).ravel(), c(part[1]["gain_r_net.2.bias"]).ravel()])
+    assert got_l.shape == (3 * h + 1,)
+    # per-sample dL/dA does not average relu's derivative flips: against fp64 the gain-network gradients are held to
+    # the cosine, entry-wise to the rounding-aware model (same operand rounding as the kernels)
+    for got, want, want_model in ((got_l, gp[0], gp_model[0]), (got_r, gp[1], gp_model[1])):
+        assert O.cosine(got, want) >= 0.995
+        assert O.max_rel_err(got, want_model) <= GRAD_TOL
+    assert O.max_rel_err(c(part[1]["Wo"]), model_g["grad_Wo"]) <= GRAD_TOL
+    assert O.max_rel_err(c(part[1]["Wl"]), model_g["grad_Wa"][0]) <= GRAD_TOL
+    lo, hi = run(slice(0, B // 2)), run(slice(B // 2, B))
+    for n in names:
+        assert O.max_rel_err(c(lo[1][n] + hi[1][n]), c(full[1][n])) <= 2e-4, n
+
+
+@pytest.mark.parametrize("weights", ["random", "perfect"])
+def test_relu_gradients_against_fp64_at_a_realistic_batch(weights, gpu_device):
+    """relu weight gradients against the fp64 oracle at B = 1024, T = 120 (122 880 samples per entry).  relu's
+    derivative is a step, and rounding the operands to bf16 moves pre-activations across it: with random weights
+    single entries differ from fp64 by 3-6 % even at this batch, with bump-sustaining weights (a few neurons carry
+    the gradient) by 7-9 %; the cosine holds everywhere (>= 0.9991 measured).  The CPU model that rounds the same
+    operands differs from fp64 by the same amounts and agrees with the kernels to 1e-2 and better, so the deviation
+    is the operand format's, not a kernel's.  The entry-wise 2e-2 bound is therefore asserted against that model;
+    against fp64 the test asserts what was measured on the MI355X (with head room) so that a regression shows."""
+    from rnn_train_ring_attractor_amd import ring_rnn_cuda_func
+    print(f"[case] relu gradients vs fp64 at N=256 B=1024 T=120, {weights} weights", flush=True)
+    B, T, k, N = 1024, 120, 2, 256
+    J0, J1 = -1.0 / N, 1.0
+    p = make_problem(31, B, T, k, N, weights=weights)
+    if weights == "perfect":                       # scaled so that the bump stays bounded under relu
+        p["Wa"], p["Wo"] = p["Wa"] / N, p["Wo"] / N
+    Wa = _t(p["Wa"], gpu_device).requires_grad_(True)
+    Wo = _t(p["Wo"], gpu_device).requires_grad_(True)
+    h = ring_rnn_cuda_func(_t(p["A"], gpu_device), Wa, J0, J1, Wo, _t(p["r0"], gpu_device), 0.15, "relu")
+    h.backward(_t(p["G"], gpu_device))
+    torch.cuda.synchronize()
+    ref, _ = O.forward_dense(p["A"], p["Wa"], J0, J1, p["Wo"], p["r0"], 0.15, "relu")
+    g = O.backward_dense(p["G"], p["A"], p["Wa"], J0, J1, p["Wo"], ref, p["r0"], 0.15, "relu")
+    model = OB.forward_backward(p["A"], p["Wa"], J0, J1, p["Wo"], p["r0"], 0.15, "relu", p["G"], folded=True)
+    gWo, gWa = Wo.grad.cpu().numpy(), Wa.grad.cpu().numpy()
+    e_wo, e_wa = O.max_rel_err(gWo, g["grad_Wo"]), O.max_rel_err(gWa, g["grad_Wa"])
+    c_wo, c_wa = O.cosine(gWo, g["grad_Wo"]), O.cosine(gWa, g["grad_Wa"])
+    m_wo, m_wa = O.max_rel_err(gWo, model["grad_Wo"]), O.max_rel_err(gWa, model["grad_Wa"])
+    mm_wo = O.max_rel_err(model["grad_Wo"], g["grad_Wo"])
+    print(f"[measured] relu {weights} B=1024 T=120: vs fp64 grad_Wo max-rel {e_wo:.3e} cos {c_wo:.6f}, grad_Wa max-rel "
+          f"{e_wa:.3e} cos {c_wa:.6f}; vs rounding model grad_Wo {m_wo:.3e} grad_Wa {m_wa:.3e}; rounding model vs fp64 "
+          f"grad_Wo {mm_wo:.3e}", flush=True)
+    assert O.max_rel_err(h.detach().cpu().numpy(), ref) <= TRAJ_TOL
+    assert c_wo >= GRAD_COS and c_wa >= GRAD_COS
+    assert m_wo <= GRAD_TOL and m_wa <= GRAD_TOL
+    assert e_wo <= 0.12 and e_wa <= 0.12
+
+
 def test_training_driver_reduces_loss(gpu_device):
     """The reference-style driver (same imports and call pattern) trains on the HIP operator."""
     import train_general_ring_no_gain as drv
