@@ -1,0 +1,344 @@
+// Kernels for wide rings: 512 < N <= 2048 (NC = NPAD / 64 in {16, 24, 32}).
+//
+// The persistent kernels keep a batch tile's whole state and all (1 + a_dim) products of a step in one workgroup's
+// registers and LDS; past N = 512 neither fits.  Here a time step is one launch (the host loops over t, as the
+// reference does for every N: cpp/kernels/fwd_1loop_tc_idx.cuh:265-277, bwd_mixed_precision_aggressive.cuh:563-672)
+// and the output neurons of a batch tile are split over workgroups: workgroup (bt, cb) owns batch rows 16*bt..+15
+// and the 16 column tiles 16*cb..16*cb+15 (256 neurons), wave v of it tiles 16*cb + 4*v .. +3.  Every workgroup
+// stages the tile's full operand row block (r_prev or g, all NPAD neurons, bf16) in LDS, streams its 256-column
+// slice of each packed weight matrix from L2 once, and contracts over the whole ring with MFMA.  At these widths a
+// step is 20 us and more, so the launch per step is noise, and the state travels between steps through the history
+// tensor (forward) or a small fp32 carry buffer (BPTT), both L2 resident.
+//
+// Layouts are the common ones with NC as a run-time number: weights [mm][tile][kc][lane][8] (ring_pack_weights_kernel),
+// operand copies for the weight-gradient kernel in paired tile order (pair_offset).  The saved derivative record is
+// private to this family: row-major fp16 [t][16*nbt][NPAD].
+#include "ring_common.hpp"
+#include "ring_kernels.hpp"
+
+namespace {
+
+constexpr int BN_GATE_KMAX = 64;
+constexpr int BN_KG = 4;   // K chunks per weight prefetch group
+
+__device__ __forceinline__ size_t pair_off_rt(int NC, int t, int nbt, int bt, int tile, int lane) {
+  return (((((size_t)(t >> 1) * nbt + bt) * (size_t)(4 * NC) + tile) * 64 + lane) * 2 + (t & 1)) * 4;
+}
+
+// slot of K position j (neuron), row b in the LDS operand buffer (see write_operand): 16-byte slots, groups padded to XG
+__device__ __forceinline__ int op_slot(int j, int b) { return ((j >> 5) * 4 + ((j >> 3) & 3)) * XG + b; }
+
+// Stage the batch tile's operand rows: v(row, j) for all j < NPAD as bf16 into xb, and the fp32 row sums into rs[16].
+// Thread (row = tid / 16, sub = tid % 16) walks its row in float4 groups 64 neurons apart.  F(b, j4, ok4) returns the
+// four fp32 values of neurons j4..j4+3 of batch row b (zero where masked).
+template <typename F>
+__device__ __forceinline__ void stage_rows(bf16x8* xb, float* rs, int NPAD, int tid, F&& value4) {
+  const int row = tid >> 4, sub = tid & 15;
+  float sum = 0.f;
+  char* base = reinterpret_cast<char*>(xb);
+  for (int j = 4 * sub; j < NPAD; j += 64) {
+    const f32x4 v = value4(row, j);
+    sum += (v[0] + v[1]) + (v[2] + v[3]);
+    const bf16x4 pk = {(__bf16)v[0], (__bf16)v[1], (__bf16)v[2], (__bf16)v[3]};
+    *reinterpret_cast<bf16x4*>(base + (size_t)op_slot(j, row) * 16 + (j & 7) * 2) = pk;
+  }
+  sum = row16_sum_dpp(sum);
+  if (sub == 0) rs[row] = sum;
+}
+
+// fp32 [rows][N] row-major, four consecutive neurons, masked
+__device__ __forceinline__ f32x4 load4_masked(const float* slab, int N, int B, int b, int j) {
+  f32x4 v = {0.f, 0.f, 0.f, 0.f};
+  if (b >= B || j >= N) return v;
+  const float* src = slab + (size_t)b * N + j;
+  if ((N & 3) == 0) return *reinterpret_cast<const f32x4*>(src);   // j is a multiple of 4, so j + 3 < N
+#pragma unroll
+  for (int x = 0; x < 4; ++x)
+    if (j + x < N) v[x] = src[x];
+  return v;
+}
+
+__device__ __forceinline__ void store4_masked(float* slab, int N, int B, int b, int j, f32x4 v) {
+  if (b >= B || j >= N) return;
+  float* dst = slab + (size_t)b * N + j;
+  if ((N & 3) == 0) {
+    *reinterpret_cast<f32x4*>(dst) = v;
+    return;
+  }
+#pragma unroll
+  for (int x = 0; x < 4; ++x)
+    if (j + x < N) dst[x] = v[x];
+}
+
+__device__ __forceinline__ void stage_gates(float* gl, const float* __restrict__ A, int k, int T, int B, int t, int bt, int tid) {
+  for (int idx = tid; idx < 16 * k; idx += 256) {
+    const int row = idx / k, c = idx - row * k, b = 16 * bt + row;
+    gl[row * BN_GATE_KMAX + c] = b < B ? A[((size_t)b * T + t) * k + c] : 0.f;
+  }
+}
+
+// bit c set <=> channel c has a non-zero gate in some of the 16 rows (same value in every lane)
+__device__ __forceinline__ unsigned long long active_channels(const float* gl, int k, int lane) {
+  unsigned long long m = 0;
+  for (int c0 = 0; c0 < k; c0 += 4) {
+    const int c = c0 + (lane >> 4);
+    const bool nz = c < k && gl[(lane & 15) * BN_GATE_KMAX + c] != 0.f;
+    const unsigned long long bal = __ballot(nz);
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      if ((bal >> (16 * j)) & 0xffffull) m |= 1ull << (c0 + j);
+  }
+  const unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)m), hi = __builtin_amdgcn_readfirstlane((unsigned)(m >> 32));
+  return ((unsigned long long)hi << 32) | lo;
+}
+
+// acc[cl][e] += sum_mm coef_mm[e] * (X @ W_mm)[row 4q+e][tile tg0 + cl], X from the LDS operand buffer (all KCH chunks),
+// W_mm streamed from the packed global copy.  coef_0 = J1, coef_{1+c} = gate of channel c; channels whose gate is
+// zero in all 16 rows are skipped when the gates are staged (a_dim <= BN_GATE_KMAX).
+__device__ __forceinline__ void wide_products(const bf16x8* xb, const bf16x8* __restrict__ Wp, const float* __restrict__ A,
+                                              const float* gl, bool staged, int k, int T, int B, int t, int b0, float J1,
+                                              int NC, int tg0, int lane, f32x4 (&acc)[4]) {
+  const int KCH = 2 * NC, q = lane >> 4, n = lane & 15;
+  const unsigned long long active = staged ? active_channels(gl, k, lane) : ~0ull;
+  for (int mm = 0; mm <= k; ++mm) {
+    if (mm > 0 && staged && !((active >> (mm - 1)) & 1ull)) continue;
+    float coef[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      if (mm == 0) coef[e] = J1;
+      else if (staged) coef[e] = gl[(4 * q + e) * BN_GATE_KMAX + (mm - 1)];
+      else coef[e] = (b0 + e < B) ? A[((size_t)(b0 + e) * T + t) * k + (mm - 1)] : 0.f;
+    }
+    f32x4 p[4];
+#pragma unroll
+    for (int cl = 0; cl < 4; ++cl) p[cl] = f32x4{0.f, 0.f, 0.f, 0.f};
+    // tile tg0 + cl, chunk kc: fragment ((mm * 4NC + tile) * KCH + kc) * 64 + lane
+    const bf16x8* wm = Wp + ((size_t)mm * 4 * NC + tg0) * KCH * 64 + lane;
+    bf16x8 wf[2][BN_KG][4];
+#pragma unroll
+    for (int u = 0; u < BN_KG; ++u)
+#pragma unroll
+      for (int cl = 0; cl < 4; ++cl) wf[0][u][cl] = wm[((size_t)cl * KCH + u) * 64];
+    const int ngroups = KCH / BN_KG;       // KCH = 2 NC is a multiple of 8
+    for (int g2 = 0; g2 < ngroups; g2 += 2) {
+#pragma unroll
+      for (int half = 0; half < 2; ++half) {
+        const int g = g2 + half;
+        const int gn = g + 1 < ngroups ? g + 1 : g;     // past the end: a re-read, unused
+#pragma unroll
+        for (int u = 0; u < BN_KG; ++u)
+#pragma unroll
+          for (int cl = 0; cl < 4; ++cl) wf[half ^ 1][u][cl] = wm[((size_t)cl * KCH + gn * BN_KG + u) * 64];
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int u = 0; u < BN_KG; ++u) {
+          const bf16x8 af = xb[((g * BN_KG + u) * 4 + q) * XG + n];
+#pragma unroll
+          for (int cl = 0; cl < 4; ++cl) p[cl] = mfma16(af, wf[half][u][cl], p[cl]);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+#pragma unroll
+    for (int cl = 0; cl < 4; ++cl)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) acc[cl][e] = fmaf(coef[e], p[cl][e], acc[cl][e]);
+  }
+}
+
+}  // namespace
+
+// One forward step (REBUILD = false: r_prev from r_init / hist[t-1], writes hist[t]) or the recomputation of the saved
+// record of every step at once from an existing history (REBUILD = true: grid.z = T, hist is only read).
+template <int ACT, bool REBUILD>
+__global__ __launch_bounds__(256) void ring_wide_fwd_kernel(RingFwdArgs p, int NC, int t_arg) {
+  extern __shared__ __attribute__((aligned(16))) char wide_lds[];
+  bf16x8* xb = reinterpret_cast<bf16x8*>(wide_lds);
+  __shared__ float rs[16];
+  __shared__ float gl[16 * BN_GATE_KMAX];
+  const int tid = threadIdx.x, wv = tid >> 6, lane = tid & 63, q = lane >> 4, n = lane & 15;
+  const int bt = blockIdx.x, cb = blockIdx.y, t = REBUILD ? (int)blockIdx.z : t_arg;
+  const int N = p.N, B = p.B, T = p.T, NPAD = 64 * NC;
+  const bool staged = p.k <= BN_GATE_KMAX;
+  const float* prev = (t == 0) ? p.r_init : p.hist + (size_t)(t - 1) * B * N;
+
+  stage_rows(xb, rs, NPAD, tid, [&](int row, int j) { return load4_masked(prev, N, B, 16 * bt + row, j); });
+  if (staged) stage_gates(gl, p.A, p.k, T, B, t, bt, tid);
+  lds_barrier();
+
+  const int tg0 = 16 * cb + 4 * wv;                       // this wave's first column tile
+  const int wg = tg0 / NC, c0 = tg0 % NC;                 // common tile order: tile = wg * NC + c
+  const int j0 = 16 * NC * wg + NC * n + c0;              // the lane's four consecutive neurons
+  const int b0 = 16 * bt + 4 * q;
+  f32x4 acc[4];
+#pragma unroll
+  for (int cl = 0; cl < 4; ++cl) acc[cl] = f32x4{0.f, 0.f, 0.f, 0.f};
+  wide_products(xb, (const bf16x8*)p.Wpack, p.A, gl, staged, p.k, T, B, t, b0, p.J1, NC, tg0, lane, acc);
+
+  const float oma = 1.f - p.alpha;
+  const size_t rows_pad = (size_t)16 * p.nbt;
+  bf16x4 rcopy[4];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const int b = b0 + e;
+    const f32x4 rp = load4_masked(prev, N, B, b, j0);
+    const float js = p.J0 * rs[4 * q + e];
+    f32x4 rn, dd;
+#pragma unroll
+    for (int cl = 0; cl < 4; ++cl) {
+      float F, D;
+      act_fast<ACT>(acc[cl][e] + js, F, D);
+      const bool ok = b < B && j0 + cl < N;
+      rn[cl] = ok ? fmaf(p.alpha, F, oma * rp[cl]) : 0.f;
+      dd[cl] = ok ? p.alpha * D : 0.f;
+      rcopy[cl][e] = (__bf16)rp[cl];
+    }
+    if (!REBUILD) store4_masked(p.hist + (size_t)t * B * N, N, B, b, j0, rn);
+    if (p.dfrag) {
+      const f16x4 pk = {(_Float16)dd[0], (_Float16)dd[1], (_Float16)dd[2], (_Float16)dd[3]};
+      *reinterpret_cast<f16x4*>(p.dfrag + ((size_t)t * rows_pad + 16 * bt + 4 * q + e) * NPAD + j0) = pk;
+    }
+  }
+  if (p.rfrag) {
+    // bf16 copy of this step's operand r_prev for the weight-gradient kernel (slot t of the paired buffer)
+#pragma unroll
+    for (int cl = 0; cl < 4; ++cl)
+      *reinterpret_cast<bf16x4*>(p.rfrag + pair_off_rt(NC, t, p.nbt, bt, tg0 + cl, lane)) = rcopy[cl];
+    if (t == T - 1 && (T & 1)) {
+      const bf16x4 z = {(__bf16)0.f, (__bf16)0.f, (__bf16)0.f, (__bf16)0.f};
+#pragma unroll
+      for (int cl = 0; cl < 4; ++cl) *reinterpret_cast<bf16x4*>(p.rfrag + pair_off_rt(NC, T, p.nbt, bt, tg0 + cl, lane)) = z;
+    }
+  }
+}
+
+// One BPTT step t: G = grad_output[t] + carry_in, g = (alpha F') * G (operand, all neurons, every workgroup of the batch
+// tile), carry_out = (1-alpha) G + J0 sum(g) + J1 (g Wo) + sum_c A_c (g Wa_c) for the workgroup's own 256 neurons.
+// carry_in == nullptr at the last time step (zero carry); at t == 0 the host points carry_out at grad_r_init or scratch.
+__global__ __launch_bounds__(256) void ring_wide_bptt_kernel(RingBpttArgs p, int NC, int t, const float* carry_in,
+                                                             float* carry_out) {
+  extern __shared__ __attribute__((aligned(16))) char wide_lds[];
+  bf16x8* xb = reinterpret_cast<bf16x8*>(wide_lds);
+  __shared__ float rs[16];
+  __shared__ float gl[16 * BN_GATE_KMAX];
+  const int tid = threadIdx.x, wv = tid >> 6, lane = tid & 63, q = lane >> 4, n = lane & 15;
+  const int bt = blockIdx.x, cb = blockIdx.y;
+  const int N = p.N, B = p.B, T = p.T, NPAD = 64 * NC;
+  const bool staged = p.k <= BN_GATE_KMAX;
+  const size_t rows_pad = (size_t)16 * p.nbt;
+  const float* gout = p.grad_out + (size_t)t * B * N;
+  const _Float16* drow = p.dfrag + (size_t)t * rows_pad * NPAD;
+
+  // g of (row, j..j+3): carry rows live in a padded [16*nbt][NPAD] buffer
+  auto g4 = [&](int row, int j, f32x4& G) {
+    const int b = 16 * bt + row;
+    G = load4_masked(gout, N, B, b, j);
+    if (carry_in) {
+      const f32x4 cin = *reinterpret_cast<const f32x4*>(carry_in + ((size_t)16 * bt + row) * NPAD + j);
+      G += cin;
+    }
+    const f16x4 d = *reinterpret_cast<const f16x4*>(drow + ((size_t)16 * bt + row) * NPAD + j);
+    return f32x4{(float)d[0] * G[0], (float)d[1] * G[1], (float)d[2] * G[2], (float)d[3] * G[3]};
+  };
+  stage_rows(xb, rs, NPAD, tid, [&](int row, int j) { f32x4 G; return g4(row, j, G); });
+  if (staged) stage_gates(gl, p.A, p.k, T, B, t, bt, tid);
+  lds_barrier();
+
+  const int tg0 = 16 * cb + 4 * wv;
+  const int wg = tg0 / NC, c0 = tg0 % NC;
+  const int j0 = 16 * NC * wg + NC * n + c0;
+  const int b0 = 16 * bt + 4 * q;
+  const float oma = 1.f - p.alpha;
+  f32x4 acc[4];
+  bf16x4 gcopy[4];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    f32x4 G;
+    const f32x4 g = g4(4 * q + e, j0, G);
+    const float js = p.J0 * rs[4 * q + e];
+#pragma unroll
+    for (int cl = 0; cl < 4; ++cl) {
+      acc[cl][e] = fmaf(oma, G[cl], js);
+      gcopy[cl][e] = (__bf16)g[cl];
+    }
+  }
+#pragma unroll
+  for (int cl = 0; cl < 4; ++cl)
+    *reinterpret_cast<bf16x4*>(p.gfrag + pair_off_rt(NC, t, p.nbt, bt, tg0 + cl, lane)) = gcopy[cl];
+  if (t == T - 1 && (T & 1)) {
+    const bf16x4 z = {(__bf16)0.f, (__bf16)0.f, (__bf16)0.f, (__bf16)0.f};
+#pragma unroll
+    for (int cl = 0; cl < 4; ++cl) *reinterpret_cast<bf16x4*>(p.gfrag + pair_off_rt(NC, T, p.nbt, bt, tg0 + cl, lane)) = z;
+  }
+  wide_products(xb, (const bf16x8*)p.Wpack, p.A, gl, staged, p.k, T, B, t, b0, p.J1, NC, tg0, lane, acc);
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const int b = b0 + e;
+    f32x4 out;
+#pragma unroll
+    for (int cl = 0; cl < 4; ++cl) out[cl] = (b < B && j0 + cl < N) ? acc[cl][e] : 0.f;
+    *reinterpret_cast<f32x4*>(carry_out + ((size_t)16 * bt + 4 * q + e) * NPAD + j0) = out;
+    if (t == 0 && p.grad_r_init) store4_masked(p.grad_r_init, N, B, b, j0, out);
+  }
+}
+
+// ------------------------------------------------------------------------------------------------
+// Launchers
+// ------------------------------------------------------------------------------------------------
+bool ring_wide_applicable(int NC) { return NC == 16 || NC == 24 || NC == 32; }
+
+size_t ring_wide_carry_bytes(int NC, int nbt) { return (size_t)2 * 16 * nbt * 64 * NC * sizeof(float); }
+
+static size_t wide_lds_bytes(int NC) { return (size_t)2 * NC * 4 * XG * sizeof(bf16x8); }
+
+template <typename K>
+static hipError_t wide_attr(K kern, size_t dyn) {
+  return hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)dyn);
+}
+
+template <int ACT>
+static hipError_t wide_fwd_act(const RingFwdArgs& a, int NC, bool rebuild, hipStream_t st) {
+  const size_t dyn = wide_lds_bytes(NC);
+  const unsigned ncb = (unsigned)(NC / 4);
+  if (rebuild) {
+    hipError_t e = wide_attr(ring_wide_fwd_kernel<ACT, true>, dyn);
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL((ring_wide_fwd_kernel<ACT, true>), dim3(a.nbt, ncb, a.T), dim3(256), dyn, st, a, NC, 0);
+    return hipGetLastError();
+  }
+  hipError_t e = wide_attr(ring_wide_fwd_kernel<ACT, false>, dyn);
+  if (e != hipSuccess) return e;
+  for (int t = 0; t < a.T; ++t) {
+    hipLaunchKernelGGL((ring_wide_fwd_kernel<ACT, false>), dim3(a.nbt, ncb), dim3(256), dyn, st, a, NC, t);
+    e = hipGetLastError();
+    if (e != hipSuccess) return e;
+  }
+  return hipSuccess;
+}
+
+hipError_t ring_launch_wide_fwd(const RingFwdArgs& a, int NC, bool rebuild, hipStream_t st) {
+  switch (a.act) {
+    case ACT_RELU: return wide_fwd_act<ACT_RELU>(a, NC, rebuild, st);
+    case ACT_GELU: return wide_fwd_act<ACT_GELU>(a, NC, rebuild, st);
+    case ACT_TANH: return wide_fwd_act<ACT_TANH>(a, NC, rebuild, st);
+    case ACT_SILU: return wide_fwd_act<ACT_SILU>(a, NC, rebuild, st);
+    default: return hipErrorInvalidValue;
+  }
+}
+
+// carry: 2 * 16 * nbt * NPAD floats of scratch (ring_wide_carry_bytes), used as two alternating buffers
+hipError_t ring_launch_wide_bptt(const RingBpttArgs& a, int NC, float* carry, hipStream_t st) {
+  const size_t dyn = wide_lds_bytes(NC);
+  hipError_t e = wide_attr(ring_wide_bptt_kernel, dyn);
+  if (e != hipSuccess) return e;
+  const size_t half = (size_t)16 * a.nbt * 64 * NC;
+  const unsigned ncb = (unsigned)(NC / 4);
+  for (int t = a.T - 1, u = 0; t >= 0; --t, ++u) {
+    const float* cin = (u == 0) ? nullptr : carry + (size_t)((u - 1) & 1) * half;
+    float* cout = carry + (size_t)(u & 1) * half;
+    hipLaunchKernelGGL(ring_wide_bptt_kernel, dim3(a.nbt, ncb), dim3(256), dyn, st, a, NC, t, cin, cout);
+    e = hipGetLastError();
+    if (e != hipSuccess) return e;
+  }
+  return hipSuccess;
+}

@@ -216,7 +216,7 @@ __global__ __launch_bounds__(256) void ring_dw_direct_kernel(RingDwArgs p, int m
   }
 }
 
-bool ring_dw_tiled_applicable(int NC) { return NC == 4 || NC == 8; }
+bool ring_dw_tiled_applicable(int NC) { return NC == 4 || NC == 8 || NC == 16 || NC == 24 || NC == 32; }
 
 // K splits: one workgroup per CU, a multiple of 8 when possible (XCD grouping).  One launch per
 // group of three matrices, so the grid of a launch does not depend on a_dim.
@@ -253,8 +253,15 @@ hipError_t ring_launch_dw_tiled(const RingDwArgs& a, int NC, hipStream_t st) {
   const unsigned blocks = (unsigned)(NB * NB * a.nz);
   const int nmg = (a.k + 3) / 3;
   for (int mg = 0; mg < nmg; ++mg) {
-    hipError_t e = NC == 4 ? launch_group<4>(a, mg, blocks, st)
-                           : (NC == 8 ? launch_group<8>(a, mg, blocks, st) : hipErrorInvalidValue);
+    hipError_t e = hipErrorInvalidValue;
+    switch (NC) {
+      case 4: e = launch_group<4>(a, mg, blocks, st); break;
+      case 8: e = launch_group<8>(a, mg, blocks, st); break;
+      case 16: e = launch_group<16>(a, mg, blocks, st); break;
+      case 24: e = launch_group<24>(a, mg, blocks, st); break;
+      case 32: e = launch_group<32>(a, mg, blocks, st); break;
+      default: break;
+    }
     if (e != hipSuccess) return e;
   }
   return hipSuccess;

@@ -984,6 +984,7 @@ static bool weights_fit_lds(int NCv, int k, size_t other_dynamic) {
 
 hipError_t ring_launch_fwd(const RingFwdArgs& a, int NCv, hipStream_t st) {
   ProfScope prof(1, st);
+  if (NCv > 8) return ring_launch_wide_fwd(a, NCv, false, st);
   if (ring_uses_resident(a.N, a.k)) return ring_launch_fwd_res256(a, st);
   const int rt = stream_row_tiles(NCv, a.nbt, false);
   hipError_t e = hipErrorInvalidValue;
@@ -1003,6 +1004,7 @@ hipError_t ring_launch_fwd(const RingFwdArgs& a, int NCv, hipStream_t st) {
 // numbers the forward would have saved, and no pass over the weights per (batch tile, step).
 hipError_t ring_launch_rebuild(const RingFwdArgs& a, int NCv, hipStream_t st) {
   ProfScope prof(2, st);
+  if (NCv > 8) return ring_launch_wide_fwd(a, NCv, true, st);
   if (ring_uses_resident(a.N, a.k)) {
     RingFwdArgs f = a;
     f.hist = nullptr;
@@ -1024,6 +1026,10 @@ static hipError_t launch_bptt_stream(const RingBpttArgs& a, dim3 grid, size_t dy
 hipError_t ring_launch_bptt(const RingBpttArgs& a, int NCv, hipStream_t st) {
   ProfScope prof(3, st);
   hipError_t e = hipErrorInvalidValue;
+  if (NCv > 8) {
+    if (a.grad_A || a.loss_coef || !a.wide_carry) return hipErrorInvalidValue;   // the C ABI rejects these before
+    return ring_launch_wide_bptt(a, NCv, a.wide_carry, st);
+  }
   // (the parentheses keep the commas of the template argument lists away from the dispatch macros)
   if (a.grad_A && !ring_uses_resident(a.N, a.k)) {   // the streaming kernel's dL/dA variant
     const size_t ga = (size_t)2 * a.k * 64 * sizeof(float);

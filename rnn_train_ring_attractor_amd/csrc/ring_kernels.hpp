@@ -32,6 +32,7 @@ struct RingBpttArgs {
   const ring_f32x4* loss_coef;
   const float* loss_upstream;   // one float on the device, or null for 1
   float loss_inv_rows;          // 1 / (T * B)
+  float* wide_carry;     // N > 512 only: 2 x [16*nbt][NPAD] fp32 scratch for the carried gradient between step launches
   float J0, J1, alpha;
   int N, k, T, B, nbt;
 };
@@ -66,7 +67,13 @@ bool ring_uses_resident(int N, int k);   // applicable and not disabled by RINGA
 hipError_t ring_launch_fwd_res256(const RingFwdArgs& a, hipStream_t st);
 hipError_t ring_launch_bptt_res256(const RingBpttArgs& a, hipStream_t st);
 
-// LDS-tiled weight-gradient contraction for NC in {4, 8} (ring_dw.hip).
+// Step-per-launch kernels for 512 < N <= 2048, NC in {16, 24, 32} (ring_bign.hip).
+bool ring_wide_applicable(int NC);
+size_t ring_wide_carry_bytes(int NC, int nbt);
+hipError_t ring_launch_wide_fwd(const RingFwdArgs& a, int NC, bool rebuild, hipStream_t st);
+hipError_t ring_launch_wide_bptt(const RingBpttArgs& a, int NC, float* carry, hipStream_t st);
+
+// LDS-tiled weight-gradient contraction for NC in {4, 8, 16, 24, 32} (ring_dw.hip).
 bool ring_dw_tiled_applicable(int NC);
 int ring_dw_tiled_nz(int NC, int k, long nchunk);
 hipError_t ring_launch_dw_tiled(const RingDwArgs& a, int NC, hipStream_t st);

@@ -38,11 +38,15 @@ struct Geo {
   size_t side_bytes;     // saved F' (fp16), [T,16*nbt,NPAD] in lane order
   size_t pair_bytes;     // one bf16 operand copy, time steps paired: [ceil(T/2)*2,16*nbt,NPAD]
   size_t partial_bytes;  // split-K partials of the weight gradient
+  size_t carry_bytes;    // N > 512: the carried gradient between the per-step BPTT launches
 };
 
-// Smallest supported neuron tiling with 64*NC >= N.
+// Smallest supported neuron tiling with 64*NC >= N: the persistent kernels up to N = 512, the step-per-launch
+// kernels (NPAD a multiple of 512) up to N = 2048.
 int pick_nc(int N) {
   for (int nc = 1; nc <= 8; nc *= 2)
+    if (64 * nc >= N) return nc;
+  for (int nc = 16; nc <= 32; nc += 8)
     if (64 * nc >= N) return nc;
   return 0;
 }
@@ -51,7 +55,7 @@ int make_geo(int N, int k, int T, int B, Geo& g) {
   if (N <= 0 || k <= 0 || T <= 0 || B <= 0)
     return fail(RINGATTR_ERR_INVALID, "N, a_dim, seq_len, batch_size must be positive (got %d, %d, %d, %d)", N, k, T, B);
   const int nc = pick_nc(N);
-  if (nc == 0) return fail(RINGATTR_ERR_INVALID, "N = %d exceeds the supported maximum of 512 neurons", N);
+  if (nc == 0) return fail(RINGATTR_ERR_INVALID, "N = %d exceeds the supported maximum of 2048 neurons", N);
   g.N = N;
   g.k = k;
   g.T = T;
@@ -72,6 +76,7 @@ int make_geo(int N, int k, int T, int B, Geo& g) {
   if (nz < 1) nz = 1;
   g.nz = ring_dw_tiled_applicable(nc) ? ring_dw_tiled_nz(nc, k, nchunk) : (int)nz;
   g.partial_bytes = align_up((size_t)g.nz * (1 + k) * g.NPAD * g.NPAD * 4);
+  g.carry_bytes = nc > 8 ? align_up(ring_wide_carry_bytes(nc, g.nbt)) : 0;
   return RINGATTR_OK;
 }
 
@@ -156,7 +161,7 @@ size_t ringattr_fwd_workspace_bytes(int N, int a_dim, int seq_len, int batch_siz
 size_t ringattr_bwd_workspace_bytes(int N, int a_dim, int seq_len, int batch_size, int have_saved) {
   Geo g;
   if (make_geo(N, a_dim, seq_len, batch_size, g) != RINGATTR_OK) return 0;
-  size_t s = g.wpack_bytes + g.pair_bytes + g.partial_bytes;
+  size_t s = g.wpack_bytes + g.pair_bytes + g.partial_bytes + g.carry_bytes;
   if (!have_saved) s += g.wpack_bytes + g.side_bytes + g.pair_bytes;
   return s;
 }
@@ -273,6 +278,8 @@ static int bwd_impl(const char* who, const void* grad_output, const void* loss_w
     return fail(RINGATTR_ERR_INVALID, "%s: null tensor pointer", who);
   if (grad_A && (size_t)2 * a_dim * 64 * sizeof(float) > 24 * 1024)
     return fail(RINGATTR_ERR_INVALID, "%s: grad_A is supported for a_dim <= 48 (got %d)", who, a_dim);
+  if (g.NC > 8 && (grad_A || loss_workspace))
+    return fail(RINGATTR_ERR_INVALID, "%s: grad_A and the fused loss backward are supported for N <= 512 (got %d)", who, N);
   if (!aligned16(grad_output) || !aligned16(A) || !aligned16(Wa) || !aligned16(Wo) || !aligned16(bump_history) ||
       !aligned16(r_init) || !aligned16(grad_Wa) || !aligned16(grad_Wo) || !aligned16(saved) ||
       !aligned16(grad_r_init) || !aligned16(grad_A) || !aligned16(workspace))
@@ -290,6 +297,8 @@ static int bwd_impl(const char* who, const void* grad_output, const void* loss_w
   ws += g.pair_bytes;
   ring_f32x4* partial = (ring_f32x4*)ws;
   ws += g.partial_bytes;
+  float* carry = g.carry_bytes ? (float*)ws : nullptr;
+  ws += g.carry_bytes;
 
   const _Float16* dfrag;
   const __bf16* rfrag;
@@ -352,6 +361,7 @@ static int bwd_impl(const char* who, const void* grad_output, const void* loss_w
   b.grad_A = (float*)grad_A;
   b.hist = (const float*)bump_history;
   b.r_init = (const float*)r_init;
+  b.wide_carry = carry;
   b.loss_coef = loss_workspace ? ring_loss_row_coefficients(loss_workspace) : nullptr;
   b.loss_upstream = (const float*)upstream;
   b.loss_inv_rows = 1.f / ((float)seq_len * (float)batch_size);

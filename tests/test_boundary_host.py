@@ -43,7 +43,9 @@ def test_size_queries():
     # padding: N=120 -> 128 neurons, B=64 -> 4 batch tiles; odd T rounds the paired buffer up
     assert lib.ringattr_saved_bytes(120, 2, 7, 64) == (7 + 8) * 64 * 128 * 2 + 3 * 128 * 128 * 2
     assert lib.ringattr_saved_bytes(0, 2, 7, 64) == 0 and "positive" in _lib.last_error()
-    assert lib.ringattr_saved_bytes(513, 2, 7, 64) == 0 and "512" in _lib.last_error()
+    # 512 < N <= 2048 pads to a multiple of 512 neurons (step-per-launch kernels); beyond that nothing runs
+    assert lib.ringattr_saved_bytes(513, 2, 8, 64) == 2 * 8 * 64 * 1024 * 2 + 3 * 1024 * 1024 * 2
+    assert lib.ringattr_saved_bytes(2049, 2, 7, 64) == 0 and "2048" in _lib.last_error()
 
 
 def test_c_abi_rejects_bad_arguments_with_codes_not_exit():

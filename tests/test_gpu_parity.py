@@ -55,6 +55,11 @@ CASES = [
     ("n512_k16_pad",   32,   6, 16, 512, "gelu", -0.1, 0.1, "lr"),        # zero-padded channels, widest tiling
     ("k70_wide_action", 20,  4, 70,  96, "tanh", -0.1, 0.1, "dense"),     # more channels than the LDS gate stage holds
     ("n300_k5_spread", 48,   5,  5, 300, "silu", -0.05, 0.2, "spread"),   # widest tiling, several matrix groups
+    # wide rings (step-per-launch kernels, NPAD a multiple of 512): the reference's published widths
+    ("n1024_gelu",     48,   6,  2, 1024, "gelu", -1 / 1024, 1.0, "lr"),
+    ("n2048_k3_tanh",  20,   4,  3, 2048, "tanh", -0.01, 0.1, "dense"),
+    ("n700_k16_pad",   32,   5, 16, 700, "silu", -0.05, 0.2, "lr"),       # ragged width, zero-padded channels
+    ("n1500_relu",     17,   3,  2, 1500, "relu", -1 / 1500, 1.0, "dense"),
 ]
 
 
@@ -154,7 +159,7 @@ def test_backward_weight_gradients(case, gpu_device):
             assert np.abs(gWa[c]).max() == 0.0
 
 
-@pytest.mark.parametrize("case", [CASES[0], CASES[3], CASES[5], CASES[9]], ids=lambda c: c[0])
+@pytest.mark.parametrize("case", [CASES[0], CASES[3], CASES[5], CASES[9], CASES[15], CASES[17]], ids=lambda c: c[0])
 def test_backward_without_saved_buffer_rebuilds_it(case, gpu_device):
     """bwd_cuda.bwd called the way the reference operator calls it (dummy re_history, reference workspaces
     absent): F'(re) is rebuilt from bump_history; the result agrees with the saved-buffer path to fp32
