@@ -70,6 +70,32 @@ __device__ __forceinline__ void store4_masked(float* slab, int N, int B, int b, 
     if (j + x < N) dst[x] = v[x];
 }
 
+// V consecutive neurons (V in {1, 2, 4}) of one batch row as a zero-padded f32x4
+template <int V>
+__device__ __forceinline__ f32x4 loadv_masked(const float* slab, int N, int B, int b, int j) {
+  if constexpr (V == 4) return load4_masked(slab, N, B, b, j);
+  f32x4 v = {0.f, 0.f, 0.f, 0.f};
+  if (b >= B) return v;
+  const float* src = slab + (size_t)b * N + j;
+#pragma unroll
+  for (int x = 0; x < V; ++x)
+    if (j + x < N) v[x] = src[x];
+  return v;
+}
+
+template <int V>
+__device__ __forceinline__ void storev_masked(float* slab, int N, int B, int b, int j, f32x4 v) {
+  if constexpr (V == 4) {
+    store4_masked(slab, N, B, b, j, v);
+    return;
+  }
+  if (b >= B) return;
+  float* dst = slab + (size_t)b * N + j;
+#pragma unroll
+  for (int x = 0; x < V; ++x)
+    if (j + x < N) dst[x] = v[x];
+}
+
 __device__ __forceinline__ void stage_gates(float* gl, const float* __restrict__ A, int k, int T, int B, int t, int bt, int tid) {
   for (int idx = tid; idx < 16 * k; idx += 256) {
     const int row = idx / k, c = idx - row * k, b = 16 * bt + row;
@@ -95,9 +121,11 @@ __device__ __forceinline__ unsigned long long active_channels(const float* gl, i
 // acc[cl][e] += sum_mm coef_mm[e] * (X @ W_mm)[row 4q+e][tile tg0 + cl], X from the LDS operand buffer (all KCH chunks),
 // W_mm streamed from the packed global copy.  coef_0 = J1, coef_{1+c} = gate of channel c; channels whose gate is
 // zero in all 16 rows are skipped when the gates are staged (a_dim <= BN_GATE_KMAX).
+// TPW: column tiles per wave (a workgroup owns 4 * TPW tiles).
+template <int TPW>
 __device__ __forceinline__ void wide_products(const bf16x8* xb, const bf16x8* __restrict__ Wp, const float* __restrict__ A,
                                               const float* gl, bool staged, int k, int T, int B, int t, int b0, float J1,
-                                              int NC, int tg0, int lane, f32x4 (&acc)[4]) {
+                                              int NC, int tg0, int lane, f32x4 (&acc)[TPW]) {
   const int KCH = 2 * NC, q = lane >> 4, n = lane & 15;
   const unsigned long long active = staged ? active_channels(gl, k, lane) : ~0ull;
   for (int mm = 0; mm <= k; ++mm) {
@@ -109,16 +137,16 @@ __device__ __forceinline__ void wide_products(const bf16x8* xb, const bf16x8* __
       else if (staged) coef[e] = gl[(4 * q + e) * BN_GATE_KMAX + (mm - 1)];
       else coef[e] = (b0 + e < B) ? A[((size_t)(b0 + e) * T + t) * k + (mm - 1)] : 0.f;
     }
-    f32x4 p[4];
+    f32x4 p[TPW];
 #pragma unroll
-    for (int cl = 0; cl < 4; ++cl) p[cl] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int cl = 0; cl < TPW; ++cl) p[cl] = f32x4{0.f, 0.f, 0.f, 0.f};
     // tile tg0 + cl, chunk kc: fragment ((mm * 4NC + tile) * KCH + kc) * 64 + lane
     const bf16x8* wm = Wp + ((size_t)mm * 4 * NC + tg0) * KCH * 64 + lane;
-    bf16x8 wf[2][BN_KG][4];
+    bf16x8 wf[2][BN_KG][TPW];
 #pragma unroll
     for (int u = 0; u < BN_KG; ++u)
 #pragma unroll
-      for (int cl = 0; cl < 4; ++cl) wf[0][u][cl] = wm[((size_t)cl * KCH + u) * 64];
+      for (int cl = 0; cl < TPW; ++cl) wf[0][u][cl] = wm[((size_t)cl * KCH + u) * 64];
     const int ngroups = KCH / BN_KG;       // KCH = 2 NC is a multiple of 8
     for (int g2 = 0; g2 < ngroups; g2 += 2) {
 #pragma unroll
@@ -128,19 +156,19 @@ __device__ __forceinline__ void wide_products(const bf16x8* xb, const bf16x8* __
 #pragma unroll
         for (int u = 0; u < BN_KG; ++u)
 #pragma unroll
-          for (int cl = 0; cl < 4; ++cl) wf[half ^ 1][u][cl] = wm[((size_t)cl * KCH + gn * BN_KG + u) * 64];
+          for (int cl = 0; cl < TPW; ++cl) wf[half ^ 1][u][cl] = wm[((size_t)cl * KCH + gn * BN_KG + u) * 64];
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int u = 0; u < BN_KG; ++u) {
           const bf16x8 af = xb[((g * BN_KG + u) * 4 + q) * XG + n];
 #pragma unroll
-          for (int cl = 0; cl < 4; ++cl) p[cl] = mfma16(af, wf[half][u][cl], p[cl]);
+          for (int cl = 0; cl < TPW; ++cl) p[cl] = mfma16(af, wf[half][u][cl], p[cl]);
         }
         __builtin_amdgcn_sched_barrier(0);
       }
     }
 #pragma unroll
-    for (int cl = 0; cl < 4; ++cl)
+    for (int cl = 0; cl < TPW; ++cl)
 #pragma unroll
       for (int e = 0; e < 4; ++e) acc[cl][e] = fmaf(coef[e], p[cl][e], acc[cl][e]);
   }
@@ -150,7 +178,9 @@ __device__ __forceinline__ void wide_products(const bf16x8* xb, const bf16x8* __
 
 // One forward step (REBUILD = false: r_prev from r_init / hist[t-1], writes hist[t]) or the recomputation of the saved
 // record of every step at once from an existing history (REBUILD = true: grid.z = T, hist is only read).
-template <int ACT, bool REBUILD>
+// TPW column tiles per wave: a workgroup owns 64 * TPW neurons.  Wide rings use 4; narrower rings with few batch
+// tiles use fewer so that the step still spreads over the device (forward without saved record only).
+template <int ACT, bool REBUILD, int TPW>
 __global__ __launch_bounds__(256) void ring_wide_fwd_kernel(RingFwdArgs p, int NC, int t_arg) {
   extern __shared__ __attribute__((aligned(16))) char wide_lds[];
   bf16x8* xb = reinterpret_cast<bf16x8*>(wide_lds);
@@ -166,26 +196,26 @@ __global__ __launch_bounds__(256) void ring_wide_fwd_kernel(RingFwdArgs p, int N
   if (staged) stage_gates(gl, p.A, p.k, T, B, t, bt, tid);
   lds_barrier();
 
-  const int tg0 = 16 * cb + 4 * wv;                       // this wave's first column tile
+  const int tg0 = 4 * TPW * cb + TPW * wv;                // this wave's first column tile
   const int wg = tg0 / NC, c0 = tg0 % NC;                 // common tile order: tile = wg * NC + c
-  const int j0 = 16 * NC * wg + NC * n + c0;              // the lane's four consecutive neurons
+  const int j0 = 16 * NC * wg + NC * n + c0;              // the lane's TPW consecutive neurons
   const int b0 = 16 * bt + 4 * q;
-  f32x4 acc[4];
+  f32x4 acc[TPW];
 #pragma unroll
-  for (int cl = 0; cl < 4; ++cl) acc[cl] = f32x4{0.f, 0.f, 0.f, 0.f};
-  wide_products(xb, (const bf16x8*)p.Wpack, p.A, gl, staged, p.k, T, B, t, b0, p.J1, NC, tg0, lane, acc);
+  for (int cl = 0; cl < TPW; ++cl) acc[cl] = f32x4{0.f, 0.f, 0.f, 0.f};
+  wide_products<TPW>(xb, (const bf16x8*)p.Wpack, p.A, gl, staged, p.k, T, B, t, b0, p.J1, NC, tg0, lane, acc);
 
   const float oma = 1.f - p.alpha;
   const size_t rows_pad = (size_t)16 * p.nbt;
-  bf16x4 rcopy[4];
+  bf16x4 rcopy[TPW];
 #pragma unroll
   for (int e = 0; e < 4; ++e) {
     const int b = b0 + e;
-    const f32x4 rp = load4_masked(prev, N, B, b, j0);
+    const f32x4 rp = loadv_masked<TPW>(prev, N, B, b, j0);
     const float js = p.J0 * rs[4 * q + e];
-    f32x4 rn, dd;
+    f32x4 rn = {0.f, 0.f, 0.f, 0.f}, dd = rn;
 #pragma unroll
-    for (int cl = 0; cl < 4; ++cl) {
+    for (int cl = 0; cl < TPW; ++cl) {
       float F, D;
       act_fast<ACT>(acc[cl][e] + js, F, D);
       const bool ok = b < B && j0 + cl < N;
@@ -193,21 +223,22 @@ __global__ __launch_bounds__(256) void ring_wide_fwd_kernel(RingFwdArgs p, int N
       dd[cl] = ok ? p.alpha * D : 0.f;
       rcopy[cl][e] = (__bf16)rp[cl];
     }
-    if (!REBUILD) store4_masked(p.hist + (size_t)t * B * N, N, B, b, j0, rn);
+    if (!REBUILD) storev_masked<TPW>(p.hist + (size_t)t * B * N, N, B, b, j0, rn);
     if (p.dfrag) {
-      const f16x4 pk = {(_Float16)dd[0], (_Float16)dd[1], (_Float16)dd[2], (_Float16)dd[3]};
-      *reinterpret_cast<f16x4*>(p.dfrag + ((size_t)t * rows_pad + 16 * bt + 4 * q + e) * NPAD + j0) = pk;
+      _Float16* dst = p.dfrag + ((size_t)t * rows_pad + 16 * bt + 4 * q + e) * NPAD + j0;
+#pragma unroll
+      for (int cl = 0; cl < TPW; ++cl) dst[cl] = (_Float16)dd[cl];
     }
   }
   if (p.rfrag) {
     // bf16 copy of this step's operand r_prev for the weight-gradient kernel (slot t of the paired buffer)
 #pragma unroll
-    for (int cl = 0; cl < 4; ++cl)
+    for (int cl = 0; cl < TPW; ++cl)
       *reinterpret_cast<bf16x4*>(p.rfrag + pair_off_rt(NC, t, p.nbt, bt, tg0 + cl, lane)) = rcopy[cl];
     if (t == T - 1 && (T & 1)) {
       const bf16x4 z = {(__bf16)0.f, (__bf16)0.f, (__bf16)0.f, (__bf16)0.f};
 #pragma unroll
-      for (int cl = 0; cl < 4; ++cl) *reinterpret_cast<bf16x4*>(p.rfrag + pair_off_rt(NC, T, p.nbt, bt, tg0 + cl, lane)) = z;
+      for (int cl = 0; cl < TPW; ++cl) *reinterpret_cast<bf16x4*>(p.rfrag + pair_off_rt(NC, T, p.nbt, bt, tg0 + cl, lane)) = z;
     }
   }
 }
@@ -270,7 +301,7 @@ __global__ __launch_bounds__(256) void ring_wide_bptt_kernel(RingBpttArgs p, int
 #pragma unroll
     for (int cl = 0; cl < 4; ++cl) *reinterpret_cast<bf16x4*>(p.gfrag + pair_off_rt(NC, T, p.nbt, bt, tg0 + cl, lane)) = z;
   }
-  wide_products(xb, (const bf16x8*)p.Wpack, p.A, gl, staged, p.k, T, B, t, b0, p.J1, NC, tg0, lane, acc);
+  wide_products<4>(xb, (const bf16x8*)p.Wpack, p.A, gl, staged, p.k, T, B, t, b0, p.J1, NC, tg0, lane, acc);
 #pragma unroll
   for (int e = 0; e < 4; ++e) {
     const int b = b0 + e;
@@ -296,32 +327,41 @@ static hipError_t wide_attr(K kern, size_t dyn) {
   return hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)dyn);
 }
 
-template <int ACT>
-static hipError_t wide_fwd_act(const RingFwdArgs& a, int NC, bool rebuild, hipStream_t st) {
+template <int ACT, int TPW>
+static hipError_t wide_fwd_tpw(const RingFwdArgs& a, int NC, bool rebuild, hipStream_t st) {
   const size_t dyn = wide_lds_bytes(NC);
-  const unsigned ncb = (unsigned)(NC / 4);
+  const unsigned ncb = (unsigned)(NC / TPW);              // 4 NC tiles / (4 TPW per workgroup)
   if (rebuild) {
-    hipError_t e = wide_attr(ring_wide_fwd_kernel<ACT, true>, dyn);
+    hipError_t e = wide_attr(ring_wide_fwd_kernel<ACT, true, TPW>, dyn);
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL((ring_wide_fwd_kernel<ACT, true>), dim3(a.nbt, ncb, a.T), dim3(256), dyn, st, a, NC, 0);
+    hipLaunchKernelGGL((ring_wide_fwd_kernel<ACT, true, TPW>), dim3(a.nbt, ncb, a.T), dim3(256), dyn, st, a, NC, 0);
     return hipGetLastError();
   }
-  hipError_t e = wide_attr(ring_wide_fwd_kernel<ACT, false>, dyn);
+  hipError_t e = wide_attr(ring_wide_fwd_kernel<ACT, false, TPW>, dyn);
   if (e != hipSuccess) return e;
   for (int t = 0; t < a.T; ++t) {
-    hipLaunchKernelGGL((ring_wide_fwd_kernel<ACT, false>), dim3(a.nbt, ncb), dim3(256), dyn, st, a, NC, t);
+    hipLaunchKernelGGL((ring_wide_fwd_kernel<ACT, false, TPW>), dim3(a.nbt, ncb), dim3(256), dyn, st, a, NC, t);
     e = hipGetLastError();
     if (e != hipSuccess) return e;
   }
   return hipSuccess;
 }
 
-hipError_t ring_launch_wide_fwd(const RingFwdArgs& a, int NC, bool rebuild, hipStream_t st) {
+template <int ACT>
+static hipError_t wide_fwd_act(const RingFwdArgs& a, int NC, bool rebuild, int tpw, hipStream_t st) {
+  if (tpw == 1) return wide_fwd_tpw<ACT, 1>(a, NC, rebuild, st);
+  if (tpw == 2) return wide_fwd_tpw<ACT, 2>(a, NC, rebuild, st);
+  return wide_fwd_tpw<ACT, 4>(a, NC, rebuild, st);
+}
+
+// tpw = 4 whenever a saved record is written (the layout the BPTT and weight-gradient kernels of this family read)
+hipError_t ring_launch_wide_fwd(const RingFwdArgs& a, int NC, bool rebuild, int tpw, hipStream_t st) {
+  if (NC % 4 != 0 || (tpw != 1 && tpw != 2 && tpw != 4)) return hipErrorInvalidValue;
   switch (a.act) {
-    case ACT_RELU: return wide_fwd_act<ACT_RELU>(a, NC, rebuild, st);
-    case ACT_GELU: return wide_fwd_act<ACT_GELU>(a, NC, rebuild, st);
-    case ACT_TANH: return wide_fwd_act<ACT_TANH>(a, NC, rebuild, st);
-    case ACT_SILU: return wide_fwd_act<ACT_SILU>(a, NC, rebuild, st);
+    case ACT_RELU: return wide_fwd_act<ACT_RELU>(a, NC, rebuild, tpw, st);
+    case ACT_GELU: return wide_fwd_act<ACT_GELU>(a, NC, rebuild, tpw, st);
+    case ACT_TANH: return wide_fwd_act<ACT_TANH>(a, NC, rebuild, tpw, st);
+    case ACT_SILU: return wide_fwd_act<ACT_SILU>(a, NC, rebuild, tpw, st);
     default: return hipErrorInvalidValue;
   }
 }

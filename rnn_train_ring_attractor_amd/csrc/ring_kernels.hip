@@ -984,7 +984,18 @@ static bool weights_fit_lds(int NCv, int k, size_t other_dynamic) {
 
 hipError_t ring_launch_fwd(const RingFwdArgs& a, int NCv, hipStream_t st) {
   ProfScope prof(1, st);
-  if (NCv > 8) return ring_launch_wide_fwd(a, NCv, false, st);
+  if (NCv > 8) return ring_launch_wide_fwd(a, NCv, false, 4, st);
+  // A forward that keeps nothing for a backward, on few batch tiles, with weights too large to stay on chip: the
+  // persistent kernels would pull every weight byte through a handful of compute units once per step.  One launch per
+  // step with the output columns split over workgroups spreads that over the device (a launch costs a few
+  // microseconds, the step it replaces tens).  RINGATTR_SPLIT_FORWARD=0 keeps the persistent kernel (tests).
+  if (!a.dfrag && !a.rfrag && NCv >= 4 && a.nbt <= 64 && !ring_uses_resident(a.N, a.k)) {
+    const char* v = getenv("RINGATTR_SPLIT_FORWARD");
+    if (!(v && v[0] == '0')) {
+      const int tpw = a.nbt * NCv >= 512 ? 4 : (a.nbt * NCv >= 256 ? 2 : 1);   // aim at >= 128 workgroups
+      return ring_launch_wide_fwd(a, NCv, false, tpw, st);
+    }
+  }
   if (ring_uses_resident(a.N, a.k)) return ring_launch_fwd_res256(a, st);
   const int rt = stream_row_tiles(NCv, a.nbt, false);
   hipError_t e = hipErrorInvalidValue;
@@ -1004,7 +1015,7 @@ hipError_t ring_launch_fwd(const RingFwdArgs& a, int NCv, hipStream_t st) {
 // numbers the forward would have saved, and no pass over the weights per (batch tile, step).
 hipError_t ring_launch_rebuild(const RingFwdArgs& a, int NCv, hipStream_t st) {
   ProfScope prof(2, st);
-  if (NCv > 8) return ring_launch_wide_fwd(a, NCv, true, st);
+  if (NCv > 8) return ring_launch_wide_fwd(a, NCv, true, 4, st);
   if (ring_uses_resident(a.N, a.k)) {
     RingFwdArgs f = a;
     f.hist = nullptr;

@@ -70,7 +70,7 @@ hipError_t ring_launch_bptt_res256(const RingBpttArgs& a, hipStream_t st);
 // Step-per-launch kernels for 512 < N <= 2048, NC in {16, 24, 32} (ring_bign.hip).
 bool ring_wide_applicable(int NC);
 size_t ring_wide_carry_bytes(int NC, int nbt);
-hipError_t ring_launch_wide_fwd(const RingFwdArgs& a, int NC, bool rebuild, hipStream_t st);
+hipError_t ring_launch_wide_fwd(const RingFwdArgs& a, int NC, bool rebuild, int tiles_per_wave, hipStream_t st);
 hipError_t ring_launch_wide_bptt(const RingBpttArgs& a, int NC, float* carry, hipStream_t st);
 
 // LDS-tiled weight-gradient contraction for NC in {4, 8, 16, 24, 32} (ring_dw.hip).
