@@ -41,7 +41,8 @@ WORKLOADS = {
     # train through dL/d action_signal (model step: MLPs + time loop forward and backward, MLP gradients included)
     "gain_n256_b4096_t240_relu": dict(N=256, B=4096, T=240, k=2, act="relu", J0=-1.0 / 256, J1=1.0, mode="gain"),
     # the reference training script's own defaults: 16 action channels of which two are driven (zero padding)
-    "train_n256_b128_t100_k16pad_gelu": dict(N=256, B=128, T=100, k=16, act="gelu", J0=-0.1, J1=0.1, mode="train"),
+    "train_n256_b128_t100_k16pad_gelu": dict(N=256, B=128, T=100, k=16, act="gelu", J0=-0.1, J1=0.1, mode="train",
+                                             driven=(0, 1)),
 }
 # the shapes of the reference's published latency table (assets/REPORT.md:5-10): forward, B=256, T=20, 16 dense channels
 for _n in (128, 256, 384, 512, 1024, 2048):
@@ -201,7 +202,8 @@ def main():
             Wo.requires_grad_(True)
 
         def fwd():
-            return ring_rnn_cuda_func(x["A"], Wa, cfg["J0"], cfg["J1"], Wo, x["r0"], 0.15, cfg["act"])
+            return ring_rnn_cuda_func(x["A"], Wa, cfg["J0"], cfg["J1"], Wo, x["r0"], 0.15, cfg["act"],
+                                      driven_channels=cfg.get("driven"))
 
         if train:
             G = loss_head_grad(fwd(), x["angle"])

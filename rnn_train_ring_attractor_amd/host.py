@@ -77,6 +77,10 @@ def av_to_action_signal_ND(av_signal, action_dim=16, zero_padding=True):
         out = torch.zeros(*av_signal.shape, action_dim, device=av_signal.device, dtype=av_signal.dtype)
         out[:, :, 0] = torch.relu(-av_signal)
         out[:, :, 1] = torch.relu(av_signal)
+        if action_dim > 2:
+            # what this construction guarantees, for the operator: channels 2.. are identically zero
+            from .ring_rnn_cuda import DRIVEN_ATTR
+            setattr(out, DRIVEN_ATTR, (0, 1))
         return out
     scales = torch.linspace(-1, 1, action_dim, device=av_signal.device, dtype=av_signal.dtype)
     return torch.relu(av_signal.unsqueeze(-1) * scales)

@@ -142,13 +142,13 @@ class RingRnnLossFunc(Function):
 
 
 def ring_rnn_loss_func(action_signal, Wa, J0, J1, Wo, r_init, alpha, activation, target_angle, bump_weight=0.2,
-                       target_amplitude=None):
+                       target_amplitude=None, driven_channels=None):
     """`ring_rnn_cuda_func(...)` and `ring_loss_pair(...)` in one operator.
 
     Returns (total, cos_loss, amp_loss, bump_history); only `total` is differentiable (w.r.t. Wa, Wo and, when they
     require it, action_signal and r_init); bump_history [T,B,N] is returned detached for decoding and logging."""
     from .ring_rnn_cuda import _silent_channel_view
-    compact = _silent_channel_view(action_signal, Wa)
+    compact = _silent_channel_view(action_signal, Wa, driven_channels)
     if compact is not None:
         action_signal, Wa = compact
     total, parts, hist = RingRnnLossFunc.apply(action_signal, Wa, J0, J1, Wo, r_init, alpha, activation, target_angle,

@@ -19,13 +19,17 @@ def _activation_id(name):
     return _ACTIVATION_MAP[name]
 
 
-def ring_rnn_cuda_func(action_signal, Wa, J0, J1, Wo, r_init, alpha, activation='relu'):
+def ring_rnn_cuda_func(action_signal, Wa, J0, J1, Wo, r_init, alpha, activation='relu', driven_channels=None):
     """Ring RNN forward pass on the GPU.
 
     action_signal (B,T,k); Wa (k,N,N); J0, J1 scalars; Wo (N,N); r_init (B,N); alpha float;
     activation in {'relu','gelu','tanh','silu'}.  Returns bump_history (T,B,N).
+
+    driven_channels (optional, not in the reference): the caller's statement that every action channel outside this
+    list of at most two indices is identically zero (the training script's zero padding of (L, R) to a_dim = 16);
+    see `_silent_channel_view`.  Tensors made by `host.av_to_action_signal_ND(zero_padding=True)` carry it themselves.
     """
-    compact = _silent_channel_view(action_signal, Wa)
+    compact = _silent_channel_view(action_signal, Wa, driven_channels)
     if compact is not None:
         action_signal, Wa = compact
     # Autograd switches gradient mode off inside Function.forward, and needs_input_grad stays True under
@@ -33,16 +37,28 @@ def ring_rnn_cuda_func(action_signal, Wa, J0, J1, Wo, r_init, alpha, activation=
     return RingRnnCudaFunc.apply(action_signal, Wa, J0, J1, Wo, r_init, alpha, activation, torch.is_grad_enabled())
 
 
-def _silent_channel_view(action_signal, Wa):
+DRIVEN_ATTR = "_ring_driven_channels"     # set on zero-padded action signals by the host helper that builds them
+
+
+def _silent_channel_view(action_signal, Wa, driven_channels=None):
     """The training script pads the two driven action channels with zeros up to a_dim = 16
     (train_general_ring_no_gain.py:52-66 of the reference).  A channel that is zero for every sample and step
-    contributes nothing forward and has an exactly zero weight gradient, so when at most two channels are driven
-    and N fits the weight-resident kernels (128 < N <= 256), the operator runs on those two channels: the slices
-    below are ordinary differentiable indexing, autograd scatters the gradients back (zeros elsewhere).
-    Finding the driven channels reads the action signal back once per call (a small reduction and one
-    device-to-host copy); RINGATTR_COMPACT_CHANNELS=0 switches this off (e.g. under graph capture)."""
+    contributes nothing forward and has an exactly zero weight gradient, so when the caller states which (at most
+    two) channels are driven and N fits the weight-resident kernels (128 < N <= 256), the operator runs on those two:
+    the slices below are ordinary differentiable indexing, autograd scatters the gradients back (zeros elsewhere).
+
+    Nothing here reads the device back: which channels are driven comes from the caller (`driven_channels=`, or the
+    attribute the host helper leaves on the tensors it pads), so the call stays asynchronous and capturable.  The
+    statement is checked on the device: if a channel declared silent is not, the compacted action signal is
+    poisoned with NaN, which the kernels carry into every output instead of returning a plausible wrong result.
+    Without a statement the operator runs on all channels (the general kernels skip all-zero channels step by step).
+    RINGATTR_COMPACT_CHANNELS=0 switches the compaction off."""
     import os
     if os.environ.get("RINGATTR_COMPACT_CHANNELS", "1") == "0":
+        return None
+    if driven_channels is None:
+        driven_channels = getattr(action_signal, DRIVEN_ATTR, None)
+    if driven_channels is None:
         return None
     if action_signal.dim() != 3 or Wa.dim() != 3 or not action_signal.is_cuda:
         return None
@@ -51,16 +67,22 @@ def _silent_channel_view(action_signal, Wa):
         return None
     if action_signal.requires_grad:        # dL/dA of a silent channel is not zero: keep every channel
         return None
-    driven = torch.nonzero((action_signal != 0).flatten(0, 1).any(dim=0)).flatten().tolist()
-    if len(driven) > 2:
-        return None
+    driven = sorted(set(int(c) for c in driven_channels))
+    if len(driven) > 2 or any(c < 0 or c >= k for c in driven):
+        raise ValueError(f"driven_channels must name at most two channels in [0, {k}), got {list(driven_channels)}")
     for c in range(k):                     # fewer than two driven: fill up with silent ones (their gates are zero)
         if len(driven) == 2:
             break
         if c not in driven:
             driven.append(c)
-    idx = torch.tensor(sorted(driven), device=Wa.device)
-    return action_signal.index_select(2, idx), Wa.index_select(0, idx)
+    c0, c1 = sorted(driven)
+    # Everything below is enqueued work on device tensors indexed with Python integers: no index tensor is copied to
+    # the device (a host-to-device copy would wait for the stream) and nothing is read back.
+    nonzero = (action_signal != 0).flatten(0, 1).any(dim=0)                     # [k] on the device
+    violated = nonzero.sum() > (nonzero[c0].to(torch.int64) + nonzero[c1].to(torch.int64))
+    poison = torch.where(violated, torch.full((), float("nan"), device=Wa.device), torch.zeros((), device=Wa.device))
+    a2 = torch.stack([action_signal[:, :, c0], action_signal[:, :, c1]], dim=2) + poison
+    return a2, torch.stack([Wa[c0], Wa[c1]])
 
 
 class RingRnnCudaFunc(Function):

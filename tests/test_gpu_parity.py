@@ -27,15 +27,21 @@ ACTS = {"relu": 0, "gelu": 1, "tanh": 2, "silu": 3}
 
 
 def _folded(N, k, A=None):
-    """The weight-resident kernels (128 < N <= 256 and two action channels, or more of which at most two are ever
-    driven: the Python operator then runs on those two) take Wo as the bf16 rounding of J1 * Wo + J0, the generic
-    ones round Wo alone and sum the J0 term in fp32; the rounding model follows the kernel under test."""
+    """The weight-resident kernels (128 < N <= 256 and two action channels, or more of which the caller states that at
+    most two are driven: the Python operator then runs on those two) take Wo as the bf16 rounding of J1 * Wo + J0, the
+    generic ones round Wo alone and sum the J0 term in fp32; the rounding model follows the kernel under test."""
     if not (128 < N <= 256) or os.environ.get("RINGATTR_STREAMING") == "1":
         return False
     if k == 2:
         return True
-    driven = 0 if A is None else int((np.abs(A).reshape(-1, k).max(axis=0) > 0).sum())
-    return A is not None and driven <= 2 and os.environ.get("RINGATTR_COMPACT_CHANNELS", "1") != "0"
+    return _driven_hint(k, A) is not None and os.environ.get("RINGATTR_COMPACT_CHANNELS", "1") != "0"
+
+
+def _driven_hint(k, A):
+    """What a caller that zero-pads (L, R) to k channels knows and tells the operator: channels 0 and 1 are driven."""
+    if k <= 2 or A is None:
+        return None
+    return (0, 1) if np.abs(A[..., 2:]).max() == 0 else None
 
 
 CASES = [
@@ -77,7 +83,8 @@ def _run_op(p, J0, J1, act, device, requires_grad=True):
     A, r0 = _dev(p["A"], device), _dev(p["r0"], device)
     Wa = _dev(p["Wa"], device).requires_grad_(requires_grad)
     Wo = _dev(p["Wo"], device).requires_grad_(requires_grad)
-    hist = ring_rnn_cuda_func(action_signal=A, Wa=Wa, J0=J0, J1=J1, Wo=Wo, r_init=r0, alpha=0.15, activation=act)
+    hist = ring_rnn_cuda_func(action_signal=A, Wa=Wa, J0=J0, J1=J1, Wo=Wo, r_init=r0, alpha=0.15, activation=act,
+                              driven_channels=_driven_hint(p["A"].shape[2], p["A"]))
     return hist, Wa, Wo
 
 
