@@ -51,26 +51,20 @@ for _n in (128, 256, 384, 512, 1024, 2048):
 
 
 def make_inputs(cfg, device):
-    """Seeded synthetic inputs of the named shape, drawn on the host with the package's own data helpers:
-    weights ~ N(0, 1/N); angular-velocity trials (10 % leading zeros, U(-0.1*pi, 0.1*pi), zero ratio in
-    {0.2, 0.5, 0.8}); L/R gates = relu(-/+av); von Mises (kappa = 4) bump at each trial's initial angle."""
-    import math
+    """Seeded synthetic inputs of the named shape, generated on the device (nothing is staged from the host):
+    weights ~ N(0, 1/N) from torch's device generator; angular-velocity trials (10 % leading zeros,
+    U(-0.1*pi, 0.1*pi), zero ratio in {0.2, 0.5, 0.8}), L/R gates = relu(-/+av) and a von Mises (kappa = 4) bump at
+    each trial's initial angle from the library's input generator (ringattr_generate_inputs)."""
     import torch
-    from rnn_train_ring_attractor_amd import host
-    torch.manual_seed(42)
+    from rnn_train_ring_attractor_amd import generate_inputs
     N, B, T, k = cfg["N"], cfg["B"], cfg["T"], cfg["k"]
-    Wo = torch.randn(N, N) / math.sqrt(N)
-    Wa = torch.randn(k, N, N) / math.sqrt(N)
-    av, angle = host.generate_av_integration_data_ultra_fast(B, T)
+    gen = torch.Generator(device=device).manual_seed(42)
+    Wo = torch.randn(N, N, device=device, generator=gen) / N ** 0.5
+    Wa = torch.randn(k, N, N, device=device, generator=gen) / N ** 0.5
+    av, angle, A, r0 = generate_inputs(42, B, T, N, k, bump="vm", device=device)
     if cfg.get("action") == "dense":
-        A = torch.rand(B, T, k) * 0.3 / k
-    else:
-        A = host.av_to_action_signal(av) if k == 2 else host.av_to_action_signal_ND(av, k)
-    pref = torch.arange(N, dtype=torch.float32) * (2 * math.pi / N)
-    r0 = torch.exp(4.0 * torch.cos(pref[None, :] - angle[:, :1]))
-    r0 = r0 / r0.norm(dim=1, keepdim=True)
-    to = lambda x: x.float().contiguous().to(device)
-    return dict(A=to(A), Wa=to(Wa), Wo=to(Wo), r0=to(r0), angle=to(angle), av=to(av))
+        A = torch.rand(B, T, k, device=device, generator=gen) * (0.3 / k)
+    return dict(A=A, Wa=Wa, Wo=Wo, r0=r0, angle=angle, av=av)
 
 
 def loss_head_grad(hist, angle):

@@ -157,6 +157,33 @@ RINGATTR_API int ringattr_gain_bwd(const void* base_signal, const void* params, 
                       void* grad_params, void* grad_base_signal, int a_dim, int hidden, int seq_len, int batch_size,
                       void* workspace, size_t workspace_bytes, void* stream);
 
+/* Synthetic inputs generated on the device: angular-velocity trials, integrated angles, the action signal and the
+ * initial bump, written where the time loop reads them.  Replaces generate_av_integration_data_ultra_fast
+ * (utils/generate_av_integration_data.py:11-58), av_to_action_signal / av_to_action_signal_ND (root
+ * train_general_ring_no_gain.py:176-229) and create_initial_bump (train/train_ring_attractor.py:21-52).  Same
+ * distributions; the random stream is the library's own counter-based generator, a function of `seed` only
+ * (repeatable bit for bit, independent of launch geometry).
+ *   zero_ratios       HOST array of 1..8 floats (per trial one is picked uniformly)
+ *   spread_action     0: channels 0 / 1 = relu(-av) / relu(av), others zero; 1: relu(av * linspace(-1, 1, a_dim))
+ *   bump_kind, bump_param   0: Gaussian on the circular distance, width N / bump_param (the reference, 10);
+ *                           1: von Mises exp(kappa cos(phi_i - angle)), kappa = bump_param; both L2-normalised
+ *   av, angle [B,T]; action_signal [B,T,a_dim]; r_init [B,N] or NULL (all fp32 device pointers, outputs) */
+RINGATTR_API int ringattr_generate_inputs(unsigned long long seed, int N, int a_dim, int seq_len, int batch_size,
+                      float zero_padding_start_ratio, const float* zero_ratios, int n_zero_ratios, float max_av,
+                      int spread_action, int bump_kind, float bump_param,
+                      void* av, void* angle, void* action_signal, void* r_init, void* stream);
+
+/* Optimizer tail of a training step: torch.nn.utils.clip_grad_norm_(parameters, max_norm) followed by
+ * torch.optim.Adam.step() (root train_general_ring_no_gain.py:333-336), for up to 16 fp32 tensors in three launches.
+ * The gradient norm is summed in a fixed order (repeatable).  params / grads / exp_avg / exp_avg_sq are HOST arrays of
+ * n_tensors device pointers, numel a host array; grads are scaled in place by min(1, max_norm / (norm + 1e-6))
+ * (max_norm <= 0: no clipping), then m, v and the parameters are updated in place; `step` counts from 1.
+ * The workspace's last float receives the gradient norm before clipping. */
+RINGATTR_API size_t ringattr_clip_adam_workspace_bytes(int n_tensors, const size_t* numel);
+RINGATTR_API int ringattr_clip_adam(int n_tensors, void* const* params, void* const* grads, void* const* exp_avg,
+                      void* const* exp_avg_sq, const size_t* numel, float lr, float beta1, float beta2, float eps,
+                      float max_norm, int step, void* workspace, size_t workspace_bytes, void* stream);
+
 /* Per-kernel timing for benchmarks; no counterpart in the reference.  While enabled, every kernel
  * launch is bracketed by two HIP events recorded on the launch stream.  ringattr_profile_read waits
  * for the recorded events, adds their durations into ms[RINGATTR_NUM_KERNELS] and the launch counts

@@ -6,6 +6,7 @@ _EXPORTS = {
     "fwd_cuda": "rnn_cuda", "bwd_cuda": "rnn_cuda",
     "ring_loss_pair": "loss_head", "RingLossPair": "loss_head",
     "ring_rnn_loss_func": "loss_head", "RingRnnLossFunc": "loss_head",
+    "generate_inputs": "device_aux", "FusedClipAdam": "device_aux",
     "ring_gain_func": "gain", "RingGainFunc": "gain", "pack_gain_nets": "gain",
 }
 

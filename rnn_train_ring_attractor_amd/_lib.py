@@ -46,6 +46,13 @@ PROTOTYPES = {
     "ringattr_gain_fwd": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p]),
     "ringattr_gain_bwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
                                   c_void_p, c_size_t, c_void_p]),
+    "ringattr_generate_inputs": (c_int, [ctypes.c_ulonglong, c_int, c_int, c_int, c_int, c_float,
+                                         ctypes.POINTER(c_float), c_int, c_float, c_int, c_int, c_float,
+                                         c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
+    "ringattr_clip_adam_workspace_bytes": (c_size_t, [c_int, ctypes.POINTER(c_size_t)]),
+    "ringattr_clip_adam": (c_int, [c_int, ctypes.POINTER(c_void_p), ctypes.POINTER(c_void_p), ctypes.POINTER(c_void_p),
+                                   ctypes.POINTER(c_void_p), ctypes.POINTER(c_size_t), c_float, c_float, c_float,
+                                   c_float, c_float, c_int, c_void_p, c_size_t, c_void_p]),
     "ringattr_profile_enable": (c_int, [c_int]),
     "ringattr_profile_read": (c_int, [ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_longlong)]),
     "fwd_cuda": (None, [c_void_p, c_void_p, c_float, c_float, c_void_p, c_void_p, c_void_p, c_float,

@@ -1,0 +1,207 @@
+// Either side of the time loop, on the device: the synthetic input generator in front of it and the optimizer tail
+// behind it.
+//
+// Input generator (utils/generate_av_integration_data.py:11-58, root train_general_ring_no_gain.py:176-229,
+// train/train_ring_attractor.py:21-52 of the reference): angular-velocity trials, their integrated angle, the action
+// signal and the initial bump, written where the time loop reads them, so that a training or benchmark step stages
+// nothing from the host.  Per trial: the first int(T * start_ratio) steps are zero; of the remaining `rest` steps
+// exactly rest - floor(rest * zero_ratio) randomly placed ones carry U(-max_av, max_av) draws (zero_ratio picked
+// uniformly from a list); angle[0] = U(0, 2 pi), angle[t] = (angle[0] + sum_{s<t} av[s]) mod 2 pi.  The reference
+// draws a random permutation per trial (argsort of uniform keys) and keeps the first n positions; choosing each
+// position in turn with probability (still needed) / (still available) gives the same distribution over subsets
+// (selection sampling) in one sequential pass, which the running sum for the angle needs anyway.  The random stream
+// is this file's own counter-based generator (same distributions as the reference, not the same bits as torch's).
+//
+// Optimizer tail (root train_general_ring_no_gain.py:333-336: clip_grad_norm_(parameters, max_norm) then Adam.step()):
+// the squared gradient norm over all tensors in a fixed order (two launches), then one launch that scales the
+// gradients by min(1, max_norm / (norm + 1e-6)) and applies the Adam update to every tensor.
+#include "ring_common.hpp"
+#include "ring_kernels.hpp"
+
+namespace {
+
+// splitmix64 finaliser over (seed, stream, counter): stateless, so any element can be drawn independently
+__device__ __forceinline__ unsigned long long mix64(unsigned long long z) {
+  z += 0x9e3779b97f4a7c15ull;
+  z = (z ^ (z >> 30)) * 0xbf58476d1ce4e5b9ull;
+  z = (z ^ (z >> 27)) * 0x94d049bb133111ebull;
+  return z ^ (z >> 31);
+}
+
+__device__ __forceinline__ unsigned rand_u32(unsigned long long seed, unsigned stream, unsigned long long counter) {
+  return (unsigned)(mix64(mix64(seed ^ ((unsigned long long)stream << 56)) + counter) >> 32);
+}
+
+__device__ __forceinline__ float rand_unit(unsigned long long seed, unsigned stream, unsigned long long counter) {
+  return (float)(rand_u32(seed, stream, counter) >> 8) * (1.0f / 16777216.0f);   // [0, 1), 24 bits
+}
+
+}  // namespace
+
+// One thread per trial.  av [B,T], angle [B,T], action [B,T,k].
+__global__ __launch_bounds__(256) void ring_generate_trials_kernel(RingGenArgs p) {
+  const int b = blockIdx.x * blockDim.x + threadIdx.x;
+  if (b >= p.B) return;
+  const int T = p.T, k = p.k;
+  const int n0 = (int)((float)T * p.start_ratio);
+  const int rest = T - n0;
+  const float two_pi = 6.283185307179586f;
+  const float angle0 = rand_unit(p.seed, 0, (unsigned long long)b) * two_pi;
+  const int pick = (int)(rand_u32(p.seed, 1, (unsigned long long)b) % (unsigned)p.n_ratios);
+  int need = rest - (int)((float)rest * p.ratios[pick]);     // float32 product, truncated, as the reference
+  need = need < 0 ? 0 : (need > rest ? rest : need);
+  float run = 0.f;                                           // sum of av[s], s < t
+  float* av = p.av + (size_t)b * T;
+  float* ang = p.angle + (size_t)b * T;
+  float* act = p.action + (size_t)b * T * k;
+  for (int t = 0; t < T; ++t) {
+    float v = 0.f;
+    if (t >= n0) {
+      const int left = T - t;                                // positions still available, this one included
+      const unsigned long long c = (unsigned long long)b * T + t;
+      if (rand_unit(p.seed, 2, c) * (float)left < (float)need) {
+        v = (rand_unit(p.seed, 3, c) - 0.5f) * (2.f * p.max_av);
+        --need;
+      }
+    }
+    float a = angle0 + run;
+    a -= floorf(a / two_pi) * two_pi;                         // Python's %: result in [0, 2 pi)
+    if (t == 0) a = angle0;
+    av[t] = v;
+    ang[t] = a;
+    if (p.spread) {
+      for (int c = 0; c < k; ++c) {
+        const float scale = k > 1 ? -1.f + 2.f * (float)c / (float)(k - 1) : -1.f;   // linspace(-1, 1, k)
+        act[(size_t)t * k + c] = fmaxf(v * scale, 0.f);
+      }
+    } else {
+      for (int c = 0; c < k; ++c) act[(size_t)t * k + c] = c == 0 ? fmaxf(-v, 0.f) : (c == 1 ? fmaxf(v, 0.f) : 0.f);
+    }
+    run += v;
+  }
+}
+
+// One workgroup per trial: r_init[b][i] = bump(i; angle[b][0]) / its Euclidean norm.
+// kind 0: exp(-d^2 / (2 w^2)), d the circular distance in neuron units to angle * N / (2 pi), w = N / param
+// (train/train_ring_attractor.py:21-52); kind 1: von Mises, exp(param * cos(2 pi i / N - angle)).
+__global__ __launch_bounds__(256) void ring_generate_bump_kernel(RingGenArgs p) {
+  __shared__ float red[4];
+  const int b = blockIdx.x, tid = threadIdx.x, N = p.N;
+  const float a0 = p.angle[(size_t)b * p.T];
+  const float two_pi = 6.283185307179586f;
+  float ss = 0.f;
+  for (int i = tid; i < N; i += 256) {
+    float v;
+    if (p.bump_kind == 0) {
+      const float centre = a0 * (float)N / two_pi, w = (float)N / p.bump_param;
+      const float d0 = fabsf((float)i - centre), d = fminf(d0, (float)N - d0);
+      v = __expf(-(d * d) / (2.f * w * w));
+    } else {
+      v = __expf(p.bump_param * (cosf(two_pi * (float)i / (float)N - a0) - 1.f));   // scaled by exp(-kappa): cancels
+    }
+    p.r_init[(size_t)b * N + i] = v;
+    ss = fmaf(v, v, ss);
+  }
+  ss = row16_sum_dpp(ss);
+  {
+    const int i = __builtin_bit_cast(int, ss);
+    ss = (__builtin_bit_cast(float, __builtin_amdgcn_readlane(i, 0)) + __builtin_bit_cast(float, __builtin_amdgcn_readlane(i, 16))) +
+         (__builtin_bit_cast(float, __builtin_amdgcn_readlane(i, 32)) + __builtin_bit_cast(float, __builtin_amdgcn_readlane(i, 48)));
+  }
+  if ((tid & 63) == 0) red[tid >> 6] = ss;
+  __syncthreads();
+  const float inv = 1.f / sqrtf((red[0] + red[1]) + (red[2] + red[3]));
+  for (int i = tid; i < N; i += 256) p.r_init[(size_t)b * N + i] *= inv;
+}
+
+hipError_t ring_launch_generate(const RingGenArgs& a, hipStream_t st) {
+  hipLaunchKernelGGL(ring_generate_trials_kernel, dim3((a.B + 255) / 256), dim3(256), 0, st, a);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess || !a.r_init) return e;
+  hipLaunchKernelGGL(ring_generate_bump_kernel, dim3(a.B), dim3(256), 0, st, a);
+  return hipGetLastError();
+}
+
+// ------------------------------------------------------------------------------------------------
+// clip_grad_norm_ + Adam
+// ------------------------------------------------------------------------------------------------
+namespace {
+constexpr int OPT_BLOCK = 256;
+constexpr int OPT_CHUNK = 4096;   // elements per workgroup
+}  // namespace
+
+// partial[blk] = sum of squares of the workgroup's chunk of the concatenated gradients (fixed order inside)
+__global__ __launch_bounds__(OPT_BLOCK) void ring_gradnorm_partial_kernel(RingOptArgs p, float* partial) {
+  __shared__ float red[OPT_BLOCK / 64];
+  // which tensor does this workgroup's chunk belong to: chunks are dealt tensor after tensor
+  int blk = blockIdx.x, ti = 0;
+  while (ti < p.n && blk >= p.chunks[ti]) blk -= p.chunks[ti++];
+  if (ti >= p.n) return;
+  const float* g = p.grad[ti];
+  const size_t lo = (size_t)blk * OPT_CHUNK, hi = lo + OPT_CHUNK < p.numel[ti] ? lo + OPT_CHUNK : p.numel[ti];
+  float s = 0.f;
+  for (size_t i = lo + threadIdx.x; i < hi; i += OPT_BLOCK) s = fmaf(g[i], g[i], s);
+  s = row16_sum_dpp(s);
+  const int si = __builtin_bit_cast(int, s);
+  s = (__builtin_bit_cast(float, __builtin_amdgcn_readlane(si, 0)) + __builtin_bit_cast(float, __builtin_amdgcn_readlane(si, 16))) +
+      (__builtin_bit_cast(float, __builtin_amdgcn_readlane(si, 32)) + __builtin_bit_cast(float, __builtin_amdgcn_readlane(si, 48)));
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = s;
+  __syncthreads();
+  if (threadIdx.x == 0) partial[blockIdx.x] = (red[0] + red[1]) + (red[2] + red[3]);
+}
+
+// norm_out[0] = sqrt(sum of the partials, in order): one workgroup, fixed tree
+__global__ __launch_bounds__(OPT_BLOCK) void ring_gradnorm_final_kernel(const float* partial, int nblk, float* norm_out) {
+  __shared__ float red[OPT_BLOCK];
+  float s = 0.f;
+  for (int i = threadIdx.x; i < nblk; i += OPT_BLOCK) s += partial[i];
+  red[threadIdx.x] = s;
+  __syncthreads();
+  for (int w = OPT_BLOCK / 2; w > 0; w >>= 1) {
+    if ((int)threadIdx.x < w) red[threadIdx.x] += red[threadIdx.x + w];
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) norm_out[0] = sqrtf(red[0]);
+}
+
+// g <- g * min(1, max_norm / (norm + 1e-6)) (written back, as clip_grad_norm_ does); then torch.optim.Adam's update:
+// m = b1 m + (1-b1) g;  v = b2 v + (1-b2) g^2;  p -= lr / (1 - b1^t) * m / (sqrt(v) / sqrt(1 - b2^t) + eps)
+__global__ __launch_bounds__(OPT_BLOCK) void ring_clip_adam_kernel(RingOptArgs p, const float* norm) {
+  int blk = blockIdx.x, ti = 0;
+  while (ti < p.n && blk >= p.chunks[ti]) blk -= p.chunks[ti++];
+  if (ti >= p.n) return;
+  float clip = 1.f;
+  if (p.max_norm > 0.f) clip = fminf(p.max_norm / (norm[0] + 1e-6f), 1.f);
+  float* g = p.grad[ti];
+  float* w = p.param[ti];
+  float* m = p.exp_avg[ti];
+  float* v = p.exp_avg_sq[ti];
+  const size_t lo = (size_t)blk * OPT_CHUNK, hi = lo + OPT_CHUNK < p.numel[ti] ? lo + OPT_CHUNK : p.numel[ti];
+  for (size_t i = lo + threadIdx.x; i < hi; i += OPT_BLOCK) {
+    const float gi = g[i] * clip;
+    const float mi = p.beta1 * m[i] + (1.f - p.beta1) * gi;
+    const float vi = p.beta2 * v[i] + (1.f - p.beta2) * gi * gi;
+    g[i] = gi;
+    m[i] = mi;
+    v[i] = vi;
+    w[i] -= p.step_size * (mi / (sqrtf(vi) * p.inv_sqrt_bc2 + p.eps));
+  }
+}
+
+int ring_opt_chunks(size_t numel) { return (int)((numel + OPT_CHUNK - 1) / OPT_CHUNK); }
+
+// workspace: (total chunks + 1) floats; the last one receives the gradient norm (before clipping)
+hipError_t ring_launch_clip_adam(const RingOptArgs& a, float* workspace, hipStream_t st) {
+  int total = 0;
+  for (int i = 0; i < a.n; ++i) total += a.chunks[i];
+  if (total <= 0) return hipErrorInvalidValue;
+  float* norm = workspace + total;
+  hipLaunchKernelGGL(ring_gradnorm_partial_kernel, dim3(total), dim3(OPT_BLOCK), 0, st, a, workspace);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return e;
+  hipLaunchKernelGGL(ring_gradnorm_final_kernel, dim3(1), dim3(OPT_BLOCK), 0, st, workspace, total, norm);
+  e = hipGetLastError();
+  if (e != hipSuccess) return e;
+  hipLaunchKernelGGL(ring_clip_adam_kernel, dim3(total), dim3(OPT_BLOCK), 0, st, a, norm);
+  return hipGetLastError();
+}

@@ -94,6 +94,38 @@ hipError_t ring_launch_gain_fwd(const float* x, const float* params, float* out,
 hipError_t ring_launch_gain_bwd(const float* x, const float* params, const float* grad_A, float* grad_params, float* grad_x,
                                 int k, int h, long samples, void* workspace, hipStream_t st);
 
+// Synthetic input generator and optimizer tail (ring_aux.hip).
+struct RingGenArgs {
+  unsigned long long seed;
+  float* av;             // [B,T]
+  float* angle;          // [B,T]
+  float* action;         // [B,T,k]
+  float* r_init;         // [B,N] or null
+  float ratios[8];       // zero ratios to pick from
+  int n_ratios;
+  float start_ratio, max_av, bump_param;
+  int spread;            // 0: (L, R) in channels 0, 1, zeros elsewhere; 1: relu(av * linspace(-1, 1, k))
+  int bump_kind;         // 0: Gaussian of width N / bump_param on the circular distance; 1: von Mises, kappa = bump_param
+  int N, k, T, B;
+};
+hipError_t ring_launch_generate(const RingGenArgs& a, hipStream_t st);
+
+constexpr int RING_OPT_MAX_TENSORS = 16;
+struct RingOptArgs {
+  float* param[RING_OPT_MAX_TENSORS];
+  float* grad[RING_OPT_MAX_TENSORS];
+  float* exp_avg[RING_OPT_MAX_TENSORS];
+  float* exp_avg_sq[RING_OPT_MAX_TENSORS];
+  size_t numel[RING_OPT_MAX_TENSORS];
+  int chunks[RING_OPT_MAX_TENSORS];
+  int n;
+  float beta1, beta2, eps, max_norm;
+  float step_size;       // lr / (1 - beta1^t)
+  float inv_sqrt_bc2;    // 1 / sqrt(1 - beta2^t)
+};
+int ring_opt_chunks(size_t numel);
+hipError_t ring_launch_clip_adam(const RingOptArgs& a, float* workspace, hipStream_t st);
+
 // Optional event bracketing of launches (benchmark support).
 void ring_profile_set(bool on);
 bool ring_profile_on();

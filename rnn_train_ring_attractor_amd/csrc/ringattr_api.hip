@@ -5,6 +5,7 @@
 #include <stdarg.h>
 #include <stdio.h>
 #include <string.h>
+#include <math.h>
 
 #include <mutex>
 
@@ -482,6 +483,86 @@ int ringattr_gain_bwd(const void* base_signal, const void* params, const void* g
                                       (float*)grad_params, (float*)grad_base_signal, a_dim, hidden,
                                       (long)seq_len * batch_size, workspace, static_cast<hipStream_t>(stream));
   if (e != hipSuccess) return hip_fail(e, "gain network backward launch");
+  return RINGATTR_OK;
+}
+
+int ringattr_generate_inputs(unsigned long long seed, int N, int a_dim, int seq_len, int batch_size,
+                             float zero_padding_start_ratio, const float* zero_ratios, int n_zero_ratios, float max_av,
+                             int spread_action, int bump_kind, float bump_param, void* av, void* angle,
+                             void* action_signal, void* r_init, void* stream) {
+  if (N <= 0 || a_dim <= 0 || seq_len <= 0 || batch_size <= 0)
+    return fail(RINGATTR_ERR_INVALID, "N, a_dim, seq_len, batch_size must be positive (got %d, %d, %d, %d)", N, a_dim,
+                seq_len, batch_size);
+  if (!zero_ratios || n_zero_ratios < 1 || n_zero_ratios > 8)
+    return fail(RINGATTR_ERR_INVALID, "ringattr_generate_inputs: between 1 and 8 zero ratios (host array) are needed");
+  if (!(zero_padding_start_ratio >= 0.f && zero_padding_start_ratio <= 1.f))
+    return fail(RINGATTR_ERR_INVALID, "ringattr_generate_inputs: zero_padding_start_ratio must lie in [0, 1]");
+  if ((bump_kind != 0 && bump_kind != 1) || !(bump_param > 0.f))
+    return fail(RINGATTR_ERR_INVALID, "ringattr_generate_inputs: bump_kind is 0 (Gaussian) or 1 (von Mises), bump_param > 0");
+  if (!av || !angle || !action_signal) return fail(RINGATTR_ERR_INVALID, "ringattr_generate_inputs: null tensor pointer");
+  RingGenArgs a;
+  a.seed = seed;
+  a.av = (float*)av;
+  a.angle = (float*)angle;
+  a.action = (float*)action_signal;
+  a.r_init = (float*)r_init;
+  for (int i = 0; i < 8; ++i) a.ratios[i] = i < n_zero_ratios ? zero_ratios[i] : 0.f;
+  a.n_ratios = n_zero_ratios;
+  a.start_ratio = zero_padding_start_ratio;
+  a.max_av = max_av;
+  a.bump_param = bump_param;
+  a.spread = spread_action ? 1 : 0;
+  a.bump_kind = bump_kind;
+  a.N = N;
+  a.k = a_dim;
+  a.T = seq_len;
+  a.B = batch_size;
+  hipError_t e = ring_launch_generate(a, static_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return hip_fail(e, "input generator launch");
+  return RINGATTR_OK;
+}
+
+size_t ringattr_clip_adam_workspace_bytes(int n_tensors, const size_t* numel) {
+  if (n_tensors < 1 || n_tensors > RING_OPT_MAX_TENSORS || !numel) {
+    fail(RINGATTR_ERR_INVALID, "between 1 and %d tensors are supported (got %d)", RING_OPT_MAX_TENSORS, n_tensors);
+    return 0;
+  }
+  size_t chunks = 0;
+  for (int i = 0; i < n_tensors; ++i) chunks += (size_t)ring_opt_chunks(numel[i]);
+  return align_up((chunks + 1) * sizeof(float));
+}
+
+int ringattr_clip_adam(int n_tensors, void* const* params, void* const* grads, void* const* exp_avg,
+                       void* const* exp_avg_sq, const size_t* numel, float lr, float beta1, float beta2, float eps,
+                       float max_norm, int step, void* workspace, size_t workspace_bytes, void* stream) {
+  const size_t need = ringattr_clip_adam_workspace_bytes(n_tensors, numel);
+  if (need == 0) return RINGATTR_ERR_INVALID;
+  if (!params || !grads || !exp_avg || !exp_avg_sq) return fail(RINGATTR_ERR_INVALID, "ringattr_clip_adam: null pointer list");
+  if (step < 1) return fail(RINGATTR_ERR_INVALID, "ringattr_clip_adam: step counts from 1 (got %d)", step);
+  if (!workspace || workspace_bytes < need)
+    return fail(RINGATTR_ERR_WORKSPACE, "ringattr_clip_adam: workspace of %zu bytes needed, %zu given", need,
+                workspace ? workspace_bytes : (size_t)0);
+  RingOptArgs a;
+  memset(&a, 0, sizeof(a));
+  for (int i = 0; i < n_tensors; ++i) {
+    if (!params[i] || !grads[i] || !exp_avg[i] || !exp_avg_sq[i] || numel[i] == 0)
+      return fail(RINGATTR_ERR_INVALID, "ringattr_clip_adam: tensor %d has a null pointer or no elements", i);
+    a.param[i] = (float*)params[i];
+    a.grad[i] = (float*)grads[i];
+    a.exp_avg[i] = (float*)exp_avg[i];
+    a.exp_avg_sq[i] = (float*)exp_avg_sq[i];
+    a.numel[i] = numel[i];
+    a.chunks[i] = ring_opt_chunks(numel[i]);
+  }
+  a.n = n_tensors;
+  a.beta1 = beta1;
+  a.beta2 = beta2;
+  a.eps = eps;
+  a.max_norm = max_norm;
+  a.step_size = (float)((double)lr / (1.0 - pow((double)beta1, (double)step)));
+  a.inv_sqrt_bc2 = (float)(1.0 / sqrt(1.0 - pow((double)beta2, (double)step)));
+  hipError_t e = ring_launch_clip_adam(a, (float*)workspace, static_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return hip_fail(e, "clip + Adam launch");
   return RINGATTR_OK;
 }
 

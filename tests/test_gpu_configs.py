@@ -478,6 +478,13 @@ def test_training_driver_reduces_loss(gpu_device):
     assert all(np.isfinite(hist_fused))
     assert abs(hist_fused[0] - hist[0]) <= 1e-3 * abs(hist[0])
     assert np.mean(hist_fused[-5:]) < np.mean(hist_fused[:5])
+    # and with the fused clip + Adam step in place of clip_grad_norm_ + torch.optim.Adam: the same curve
+    _, hist_opt = drv.run_training(action_dim=2, num_neurons=128, training_steps=40, batch_size=64, seq_len=60,
+                                   lr=3e-3, activation="gelu", log_every=0, seed=1, fused_optimizer=True)
+    assert all(np.isfinite(hist_opt))
+    assert abs(hist_opt[0] - hist[0]) <= 1e-6 * abs(hist[0])
+    assert np.max(np.abs(np.array(hist_opt[:10]) - np.array(hist[:10]))) <= 1e-2 * abs(hist[0])
+    assert np.mean(hist_opt[-5:]) < np.mean(hist_opt[:5])
 
 
 def test_reference_signature_entry_points(gpu_device):
