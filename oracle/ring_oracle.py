@@ -318,6 +318,17 @@ def max_rel_err(x: np.ndarray, ref: np.ndarray) -> float:
     return float(np.max(np.abs(x - ref)) / (np.max(np.abs(ref)) + 1e-300))
 
 
+def elementwise_rel_err(x: np.ndarray, ref: np.ndarray, floor_frac: float = 0.1) -> float:
+    """max over the entries with |ref| >= floor_frac * max|ref| of |x - ref| / |ref|: an element-wise relative error
+    on the entries that carry the signal (below the floor the ratio measures rounding noise against near-zeros)."""
+    x = np.asarray(x, np.float64)
+    ref = np.asarray(ref, np.float64)
+    big = np.abs(ref) >= floor_frac * np.max(np.abs(ref))
+    if not big.any():
+        return 0.0
+    return float(np.max(np.abs(x - ref)[big] / np.abs(ref)[big]))
+
+
 def loss_pair_rank2(bump_tbn, target_angle, bump_weight=0.2, target_amplitude=None):
     """The training loss pair and its gradient through the rank-two form of the read-out.
 

@@ -23,7 +23,7 @@ def test_config1_inference_full_size(gpu_device):
     from rnn_train_ring_attractor_amd import ring_rnn_cuda_func
     print("[case] config1 N=256 B=1024 T=120 relu", flush=True)
     B, T, k, N = 1024, 120, 2, 256
-    p = make_problem(11, B, T, k, N, zero_ratios=(0.5,), weights="perfect")
+    p = make_problem(11, B, T, k, N, zero_ratios=(0.5,), weights="perfect", bump="vm")
     with torch.no_grad():
         hist = ring_rnn_cuda_func(_t(p["A"], gpu_device), _t(p["Wa"], gpu_device), -0.1, 0.1, _t(p["Wo"], gpu_device),
                                   _t(p["r0"], gpu_device), 0.15, "gelu")
@@ -45,7 +45,7 @@ def test_config3_geometry_long_sequence(gpu_device):
     from rnn_train_ring_attractor_amd import ring_rnn_cuda_func
     print("[case] config3 N=512 B=32 T=512 tanh", flush=True)
     B, T, k, N = 32, 512, 2, 512
-    p = make_problem(12, B, T, k, N, zero_ratios=(0.2,))
+    p = make_problem(12, B, T, k, N, zero_ratios=(0.2,), bump="vm")
     Wa = _t(p["Wa"], gpu_device).requires_grad_(True)
     Wo = _t(p["Wo"], gpu_device).requires_grad_(True)
     hist = ring_rnn_cuda_func(_t(p["A"], gpu_device), Wa, -0.1, 0.1, Wo, _t(p["r0"], gpu_device), 0.15, "tanh")
@@ -69,7 +69,7 @@ def test_headline_size_properties(gpu_device):
     print("[case] headline N=256 B=4096 T=120 gelu", flush=True)
     B, T, k, N = 4096, 120, 2, 256
     J0, J1 = -1.0 / N, 1.0
-    p = make_problem(42, B, T, k, N)
+    p = make_problem(42, B, T, k, N, bump="vm")
     A, r0, G = _t(p["A"], gpu_device), _t(p["r0"], gpu_device), _t(p["G"], gpu_device)
 
     def run(rows):

@@ -22,6 +22,8 @@ pytestmark = pytest.mark.gpu
 TRAJ_TOL = 1e-2
 GRAD_COS = 0.999
 GRAD_TOL = 2e-2
+ELEMENTWISE_TRAJ_TOL = 5e-2   # |x - ref| / |ref| on the entries that are at least 10 % of the largest
+ELEMENTWISE_GRAD_TOL = 1e-1
 MODEL_TOL = 5e-3        # HIP vs the rounding-aware CPU model (same operand rounding, fp64 accumulation)
 ACTS = {"relu": 0, "gelu": 1, "tanh": 2, "silu": 3}
 
@@ -101,6 +103,9 @@ def test_forward_trajectory_and_decoded_angle(case, gpu_device):
     assert np.isfinite(got).all()
     err = O.max_rel_err(got, ref)
     assert err <= TRAJ_TOL, f"trajectory error {err}"
+    ew = O.elementwise_rel_err(got, ref)
+    print(f"[measured] fwd {name}: max-norm err {err:.2e}, element-wise (entries >= 10% of max) {ew:.2e}", flush=True)
+    assert ew <= ELEMENTWISE_TRAJ_TOL
     model = OB.forward_backward(p["A"], p["Wa"], J0, J1, p["Wo"], p["r0"], 0.15, act,
                                 folded=_folded(N, k, p["A"]))["bump_history"]
     assert O.max_rel_err(got, model) <= MODEL_TOL
@@ -155,6 +160,9 @@ def test_backward_weight_gradients(case, gpu_device):
     assert O.max_rel_err(gWo, model["grad_Wo"]) <= model_tol
     if smooth:
         assert O.max_rel_err(gWo, ref["grad_Wo"]) <= GRAD_TOL
+        ew = O.elementwise_rel_err(gWo, ref["grad_Wo"])
+        print(f"[measured] bwd {name}: grad_Wo element-wise (entries >= 10% of max) {ew:.2e}", flush=True)
+        assert ew <= ELEMENTWISE_GRAD_TOL
     used = [c for c in range(k) if np.abs(p["A"][..., c]).max() > 0]
     for c in range(k):
         if c in used:
