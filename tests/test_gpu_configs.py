@@ -137,6 +137,15 @@ def test_long_sequence_shape_at_full_size(gpu_device):
     g = O.backward_dense(c(G[:, sl]), c(A[sl]), c(Wa0), J0, J1, c(Wo0), ref, c(r0[sl]), 0.15, "tanh")
     assert O.cosine(c(part[2]), g["grad_Wo"]) >= GRAD_COS and O.max_rel_err(c(part[2]), g["grad_Wo"]) <= GRAD_TOL
     assert O.cosine(c(part[1]), g["grad_Wa"]) >= GRAD_COS and O.max_rel_err(c(part[1]), g["grad_Wa"]) <= GRAD_TOL
+    # the backward without the forward's saved record (the reference's call pattern: nothing but bump_history is
+    # kept, the derivative record and the operand copy are recomputed from it) at the full size
+    from rnn_train_ring_attractor_amd import bwd_cuda
+    gWa, gWo = torch.empty_like(Wa0), torch.empty_like(Wo0)
+    bwd_cuda.bwd(grad_output=G, A=A, Wa=Wa0, J0=J0, J1=J1, Wo=Wo0, bump_history=full[0], r_init=r0, grad_Wa=gWa,
+                 grad_Wo=gWo, alpha=0.15, activation_type=2, accumulate=False)
+    torch.cuda.synchronize()
+    assert O.max_rel_err(c(gWa), c(full[1])) <= 1e-3 and O.max_rel_err(c(gWo), c(full[2])) <= 1e-3
+    del gWa, gWo
     doubled = run(slice(0, B), 2.0)
     assert O.max_rel_err(c(doubled[2]), 2.0 * c(full[2])) <= 1e-5 and O.max_rel_err(c(doubled[1]), 2.0 * c(full[1])) <= 1e-5
     lo, hi = run(slice(0, B // 2)), run(slice(B // 2, B))
