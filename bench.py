@@ -37,6 +37,8 @@ WORKLOADS = {
     "train_n120_b64_t120_tanh": dict(N=120, B=64, T=120, k=2, act="tanh", J0=-1.0 / 120, J1=1.0, mode="train"),
     "infer_n256_b1024_t120_relu": dict(N=256, B=1024, T=120, k=2, act="relu", J0=-1.0 / 256, J1=1.0, mode="infer"),
     "train_n512_b8192_t512_tanh": dict(N=512, B=8192, T=512, k=2, act="tanh", J0=-1.0 / 512, J1=1.0, mode="train"),
+    # a wide ring (the reference's kernels take rings up to 2048 neurons), trained at a large batch
+    "train_n1024_b2048_t120_tanh": dict(N=1024, B=2048, T=120, k=2, act="tanh", J0=-1.0 / 1024, J1=1.0, mode="train"),
     # the general ring with gain networks: two 1 -> 16 -> 1 MLPs turn the angular velocity into the (L, R) gates and
     # train through dL/d action_signal (model step: MLPs + time loop forward and backward, MLP gradients included)
     "gain_n256_b4096_t240_relu": dict(N=256, B=4096, T=240, k=2, act="relu", J0=-1.0 / 256, J1=1.0, mode="gain"),

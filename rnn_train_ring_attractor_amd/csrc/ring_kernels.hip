@@ -982,9 +982,33 @@ static bool weights_fit_lds(int NCv, int k, size_t other_dynamic) {
   return wb + other_dynamic + 20 * 1024 <= 128 * 1024;   // 20 KiB: static LDS of these kernels, rounded up
 }
 
+// Which time loop runs a problem that keeps a saved record (forward and backward must agree: the record's layout
+// differs between the persistent and the step-per-launch families).  Wide rings have only the step-per-launch
+// kernels; RINGATTR_BLOCK=1 / 0 forces / forbids them where the persistent streaming kernels also apply.
+bool ring_uses_step_kernels(int N, int k, int NCv, int nbt) {
+  if (NCv > 8) return true;
+  if (NCv < 4 || ring_uses_resident(N, k)) return false;
+  const char* v = getenv("RINGATTR_BLOCK");
+  if (v && (v[0] == '0' || v[0] == '1')) return v[0] == '1';
+  (void)nbt;
+  return false;
+}
+
+// Which step-per-launch family: the block kernels (K-outer, three matrices' products at a time) are ahead on few
+// batch tiles, the one-tile-per-workgroup kernels of ring_bign.hip (up to 1.6 times) on many; measured crossover
+// about nbt * NC = 512 (N = 1024: 512 rows, N = 2048: 256 rows).  RINGATTR_WIDE=1 / 0 forces one or the other
+// (cross-checks); the two share the record layout, so forward and backward may choose independently.
+static bool step_prefers_wide(int NCv, int nbt) {
+  if (NCv % 4 != 0) return false;
+  const char* v = getenv("RINGATTR_WIDE");
+  if (v && (v[0] == '0' || v[0] == '1')) return v[0] == '1';
+  return (long)nbt * NCv > 512;
+}
+
 hipError_t ring_launch_fwd(const RingFwdArgs& a, int NCv, hipStream_t st) {
   ProfScope prof(1, st);
-  if (NCv > 8) return ring_launch_wide_fwd(a, NCv, false, 4, st);
+  if (ring_uses_step_kernels(a.N, a.k, NCv, a.nbt))
+    return step_prefers_wide(NCv, a.nbt) ? ring_launch_wide_fwd(a, NCv, false, 4, st) : ring_launch_block_fwd(a, NCv, false, st);
   // A forward that keeps nothing for a backward, on few batch tiles, with weights too large to stay on chip: the
   // persistent kernels would pull every weight byte through a handful of compute units once per step.  One launch per
   // step with the output columns split over workgroups spreads that over the device (a launch costs a few
@@ -1015,7 +1039,8 @@ hipError_t ring_launch_fwd(const RingFwdArgs& a, int NCv, hipStream_t st) {
 // numbers the forward would have saved, and no pass over the weights per (batch tile, step).
 hipError_t ring_launch_rebuild(const RingFwdArgs& a, int NCv, hipStream_t st) {
   ProfScope prof(2, st);
-  if (NCv > 8) return ring_launch_wide_fwd(a, NCv, true, 4, st);
+  if (ring_uses_step_kernels(a.N, a.k, NCv, a.nbt))
+    return step_prefers_wide(NCv, a.nbt) ? ring_launch_wide_fwd(a, NCv, true, 4, st) : ring_launch_block_fwd(a, NCv, true, st);
   if (ring_uses_resident(a.N, a.k)) {
     RingFwdArgs f = a;
     f.hist = nullptr;
@@ -1037,9 +1062,10 @@ static hipError_t launch_bptt_stream(const RingBpttArgs& a, dim3 grid, size_t dy
 hipError_t ring_launch_bptt(const RingBpttArgs& a, int NCv, hipStream_t st) {
   ProfScope prof(3, st);
   hipError_t e = hipErrorInvalidValue;
-  if (NCv > 8) {
+  if (ring_uses_step_kernels(a.N, a.k, NCv, a.nbt)) {
     if (a.grad_A || a.loss_coef || !a.wide_carry) return hipErrorInvalidValue;   // the C ABI rejects these before
-    return ring_launch_wide_bptt(a, NCv, a.wide_carry, st);
+    return step_prefers_wide(NCv, a.nbt) ? ring_launch_wide_bptt(a, NCv, a.wide_carry, st)
+                                  : ring_launch_block_bptt(a, NCv, a.wide_carry, st);
   }
   // (the parentheses keep the commas of the template argument lists away from the dispatch macros)
   if (a.grad_A && !ring_uses_resident(a.N, a.k)) {   // the streaming kernel's dL/dA variant

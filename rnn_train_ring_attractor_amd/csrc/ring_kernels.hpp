@@ -73,6 +73,13 @@ size_t ring_wide_carry_bytes(int NC, int nbt);
 hipError_t ring_launch_wide_fwd(const RingFwdArgs& a, int NC, bool rebuild, int tiles_per_wave, hipStream_t st);
 hipError_t ring_launch_wide_bptt(const RingBpttArgs& a, int NC, float* carry, hipStream_t st);
 
+// Step-per-launch kernels with several batch tiles per workgroup (ring_block.hip); same saved-record layout and
+// carry buffer as the wide-ring kernels.
+hipError_t ring_launch_block_fwd(const RingFwdArgs& a, int NC, bool rebuild, hipStream_t st);
+hipError_t ring_launch_block_bptt(const RingBpttArgs& a, int NC, float* carry, hipStream_t st);
+// which kernel family runs a problem with a saved record: 0 persistent, 1 step-per-launch (wide or block)
+bool ring_uses_step_kernels(int N, int k, int NC, int nbt);
+
 // LDS-tiled weight-gradient contraction for NC in {4, 8, 16, 24, 32} (ring_dw.hip).
 bool ring_dw_tiled_applicable(int NC);
 int ring_dw_tiled_nz(int NC, int k, long nchunk);

@@ -77,7 +77,7 @@ int make_geo(int N, int k, int T, int B, Geo& g) {
   if (nz < 1) nz = 1;
   g.nz = ring_dw_tiled_applicable(nc) ? ring_dw_tiled_nz(nc, k, nchunk) : (int)nz;
   g.partial_bytes = align_up((size_t)g.nz * (1 + k) * g.NPAD * g.NPAD * 4);
-  g.carry_bytes = nc > 8 ? align_up(ring_wide_carry_bytes(nc, g.nbt)) : 0;
+  g.carry_bytes = nc >= 4 ? align_up(ring_wide_carry_bytes(nc, g.nbt)) : 0;   // (small; sized whichever family runs)
   return RINGATTR_OK;
 }
 
@@ -97,7 +97,7 @@ int hip_fail(hipError_t e, const char* what) {
 // wrote under the buffer's address; a backward that finds no matching note (another process state, a copied
 // buffer, RINGATTR_STREAMING changed in between) packs its own copy instead of trusting the one in the buffer.
 constexpr int kSavedNotes = 256;
-struct SavedNote { const void* ptr; int family; };   // family: 1 streaming, 2 weight-resident
+struct SavedNote { const void* ptr; int family; };   // family: 1 streaming, 2 weight-resident, 3 step-per-launch
 std::mutex g_saved_mu;
 SavedNote g_saved_notes[kSavedNotes] = {};
 int g_saved_next = 0;
@@ -191,7 +191,7 @@ int ringattr_fwd(const void* A, const void* Wa, float J0, float J1, const void* 
   hipError_t e = ring_launch_pack2((const float*)Wo, (const float*)Wa, N, a_dim, g.NC, workspace, 0, resident, s0, h0,
                                    wpack_t, 1, 0, s0, h0, st);
   if (e != hipSuccess) return hip_fail(e, "pack weights");
-  if (saved) saved_note_put(saved, resident ? 2 : 1);
+  if (saved) saved_note_put(saved, ring_uses_step_kernels(N, a_dim, g.NC, g.nbt) ? 3 : (resident ? 2 : 1));
 
   RingFwdArgs a;
   a.A = (const float*)A;
@@ -279,8 +279,10 @@ static int bwd_impl(const char* who, const void* grad_output, const void* loss_w
     return fail(RINGATTR_ERR_INVALID, "%s: null tensor pointer", who);
   if (grad_A && (size_t)2 * a_dim * 64 * sizeof(float) > 24 * 1024)
     return fail(RINGATTR_ERR_INVALID, "%s: grad_A is supported for a_dim <= 48 (got %d)", who, a_dim);
-  if (g.NC > 8 && (grad_A || loss_workspace))
-    return fail(RINGATTR_ERR_INVALID, "%s: grad_A and the fused loss backward are supported for N <= 512 (got %d)", who, N);
+  const bool step_family = ring_uses_step_kernels(N, a_dim, g.NC, g.nbt);
+  if (step_family && (grad_A || loss_workspace))
+    return fail(RINGATTR_ERR_INVALID, "%s: grad_A and the fused loss backward are not available on the step-per-launch "
+                "kernels (N = %d > 512, or RINGATTR_BLOCK=1)", who, N);
   if (!aligned16(grad_output) || !aligned16(A) || !aligned16(Wa) || !aligned16(Wo) || !aligned16(bump_history) ||
       !aligned16(r_init) || !aligned16(grad_Wa) || !aligned16(grad_Wo) || !aligned16(saved) ||
       !aligned16(grad_r_init) || !aligned16(grad_A) || !aligned16(workspace))
@@ -342,7 +344,12 @@ static int bwd_impl(const char* who, const void* grad_output, const void* loss_w
   const bool resident = ring_uses_resident(N, a_dim);
   const bool bptt_resident = resident;
   hipError_t e = hipSuccess;
-  if (saved && saved_note_get(saved) == (bptt_resident ? 2 : 1)) {
+  const int family = step_family ? 3 : (bptt_resident ? 2 : 1);
+  const int noted = saved ? saved_note_get(saved) : 0;
+  if (noted != 0 && (noted == 3) != (family == 3))
+    return fail(RINGATTR_ERR_INVALID, "%s: the saved buffer was filled by the other kernel family (its derivative record "
+                "has a different layout); run forward and backward under the same RINGATTR_BLOCK setting", who);
+  if (saved && noted == family) {
     // the forward left the transposed copy, in the form this BPTT kernel expects, behind the saved activations
     wb = (char*)const_cast<void*>(saved) + g.side_bytes + g.pair_bytes;
   } else {

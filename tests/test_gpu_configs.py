@@ -212,6 +212,50 @@ def test_paired_batch_tiles_equal_single_tiles(B, T, k, N, act, saved, gpu_devic
     assert O.cosine(outs["2"][3], ref["grad_r_init"]) >= 0.999
 
 
+@pytest.mark.parametrize("B,T,k,N,act,force,saved", [
+    (40, 6, 2, 1024, "tanh", {"RINGATTR_WIDE": ("0", "1")}, True),     # wide ring: block kernels against one-tile kernels
+    (24, 5, 3, 700, "gelu", {"RINGATTR_WIDE": ("0", "1")}, False),     # ragged, backward rebuilds the record
+    (72, 7, 2, 512, "silu", {"RINGATTR_BLOCK": ("0", "1")}, True),     # persistent streaming against block (two tiles per workgroup)
+    (40, 6, 5, 300, "relu", {"RINGATTR_BLOCK": ("0", "1")}, False),
+])
+def test_step_per_launch_families_agree(B, T, k, N, act, force, saved, gpu_device, monkeypatch):
+    """The step-per-launch kernels (block, one-tile) and the persistent streaming kernels evaluate the same recurrence
+    on the same bf16 operands; they differ in accumulation order only.  Each forced pair must agree to rounding, and
+    the second run is also held to the oracle."""
+    from rnn_train_ring_attractor_amd import rnn_cuda
+    print(f"[case] step families B={B} T={T} k={k} N={N} {act} {force} saved={saved}", flush=True)
+    p = make_problem(31 + N + k, B, T, k, N)
+    acts = {"relu": 0, "gelu": 1, "tanh": 2, "silu": 3}
+    J0, J1 = (-1.0 / N, 1.0) if act == "relu" else (-0.1, 0.3)
+    (var, modes), = force.items()
+    outs = {}
+    for mode in modes:
+        monkeypatch.setenv(var, mode)
+        A, Wa, Wo, r0, G = (_t(p[x], gpu_device) for x in ("A", "Wa", "Wo", "r0", "G"))
+        hist = torch.empty(T, B, N, device=gpu_device)
+        sv = torch.empty(rnn_cuda.saved_nbytes(N, k, T, B), dtype=torch.uint8, device=gpu_device) if saved else None
+        rnn_cuda.fwd_cuda.fwd(A=A, Wa=Wa, J0=J0, J1=J1, Wo=Wo, r_init=r0, bump_history=hist, alpha=0.15,
+                              activation_type=acts[act], saved=sv)
+        gWa, gWo = torch.zeros_like(Wa), torch.zeros_like(Wo)
+        gr0 = torch.empty_like(r0)
+        rnn_cuda.bwd_cuda.bwd(grad_output=G, A=A, Wa=Wa, J0=J0, J1=J1, Wo=Wo, bump_history=hist, r_init=r0,
+                              grad_Wa=gWa, grad_Wo=gWo, alpha=0.15, activation_type=acts[act],
+                              saved=sv, grad_r_init=gr0)
+        torch.cuda.synchronize()
+        outs[mode] = [x.cpu().numpy() for x in (hist, gWa, gWo, gr0)]
+    a, b = outs[modes[0]], outs[modes[1]]
+    assert O.max_rel_err(a[0], b[0]) <= 1e-4
+    for x, y in zip(a[1:], b[1:]):
+        # a last-bit difference in fp32 can flip the bf16 rounding of an operand copy (or a relu kink)
+        assert O.max_rel_err(x, y) <= (2e-2 if act == "relu" else 3e-3)
+    ref_hist, _ = O.forward_dense(p["A"], p["Wa"], J0, J1, p["Wo"], p["r0"], 0.15, act)
+    assert O.max_rel_err(b[0], ref_hist) <= TRAJ_TOL
+    ref = O.backward_dense(p["G"], p["A"], p["Wa"], J0, J1, p["Wo"], ref_hist, p["r0"], 0.15, act)
+    floor = 0.995 if act == "relu" else 0.999       # bf16 operands move samples across the relu kink
+    assert O.cosine(b[2], ref["grad_Wo"]) >= floor and O.cosine(b[1], ref["grad_Wa"]) >= floor
+    assert O.cosine(b[3], ref["grad_r_init"]) >= floor
+
+
 @pytest.mark.parametrize("driven", [(3, 9), (5,), ()], ids=["two", "one", "none"])
 def test_silent_action_channels_are_compacted(driven, gpu_device, monkeypatch):
     """With a_dim > 2 and the caller's statement that at most two named channels are driven, the Python operator runs
