@@ -141,6 +141,11 @@ RINGATTR_API int ringattr_bwd_loss(const void* loss_workspace, const void* upstr
                       const void* saved, void* grad_A, void* grad_r_init,
                       void* workspace, size_t workspace_bytes, void* stream);
 
+/* 1 when ringattr_bwd_loss can serve this shape (the persistent kernel families: N <= 512 unless RINGATTR_BLOCK=1
+ * moves the shape to the step-per-launch kernels), 0 when the caller has to run ringattr_loss_bwd and hand its
+ * [T,B,N] result to ringattr_bwd instead (the host-side operator does).  No counterpart in the reference. */
+RINGATTR_API int ringattr_bwd_loss_available(int N, int a_dim, int seq_len, int batch_size);
+
 /* Gain networks of the action signal, forward and backward.  Replaces the per-channel nn.Sequential(Linear(1,h), GELU,
  * Linear(h,1), Softplus) evaluation and its autograd in the reference models (train/train_ring_attractor.py:70-79,
  * 136-146; train/train_general_ring_attractor.py:38-46, 99-109): per sample, step and channel c

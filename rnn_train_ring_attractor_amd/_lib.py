@@ -39,6 +39,7 @@ PROTOTYPES = {
                                   c_void_p, c_size_t, c_void_p]),
     "ringattr_loss_bwd": (c_int, [c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_int, c_int, c_int,
                                   c_void_p, c_size_t, c_void_p]),
+    "ringattr_bwd_loss_available": (c_int, [c_int] * 4),
     "ringattr_bwd_loss": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_float, c_void_p, c_void_p, c_void_p,
                                   c_void_p, c_void_p, c_float, c_int, c_int, c_int, c_int, c_int, c_int,
                                   c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),

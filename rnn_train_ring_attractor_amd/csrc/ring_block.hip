@@ -315,6 +315,79 @@ __global__ __launch_bounds__(256) void ring_block_bptt_kernel(RingBpttArgs p, in
   }
 }
 
+// dL/dA for the step-per-launch families, after the BPTT steps have left g (bf16, paired tile order) for every step:
+//   grad_A[b, t, c] = sum_i g[t, b, i] * (Wa[c] @ r_prev[t, b])_i
+// No recurrence: one workgroup per (batch tile, step) stages the tile's r_prev rows as the forward does, walks all
+// column blocks with the forward fragments of three channels at a time, multiplies each product by the lane's g
+// (the paired layout is exactly the MFMA result layout) and reduces over neurons -- lanes by DPP, waves through LDS
+// in wave order, so the result does not depend on scheduling.  Wf: forward-orientation packed weights.
+template <int TPW>
+__global__ __launch_bounds__(256) void ring_block_grad_A_kernel(RingBpttArgs p, const bf16x8* __restrict__ Wf, int NC) {
+  extern __shared__ __attribute__((aligned(16))) char block_lds[];
+  bf16x8* xb = reinterpret_cast<bf16x8*>(block_lds);
+  __shared__ float rs[16];
+  __shared__ float part[3][4][16];
+  const int tid = threadIdx.x, wv = tid >> 6, lane = tid & 63, q = lane >> 4, n = lane & 15;
+  const int bt = blockIdx.x, t = blockIdx.y;
+  const int N = p.N, B = p.B, T = p.T, k = p.k, NPAD = 64 * NC, slots = 2 * NC * 4 * XG, KCH = 2 * NC;
+  const float* prev = (t == 0) ? p.r_init : p.hist + (size_t)(t - 1) * B * N;
+  stage_tiles<1>(xb, slots, rs, NPAD, tid, [&](int row, int j) { return load4_masked(prev, N, B, 16 * bt + row, j); });
+  lds_barrier();
+
+  for (int m0 = 1; m0 <= k; m0 += 3) {
+    float ga[3][4];
+#pragma unroll
+    for (int a = 0; a < 3; ++a)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) ga[a][e] = 0.f;
+    for (int cb = 0; cb < NC / TPW; ++cb) {
+      const int tg0 = 4 * TPW * cb + TPW * wv;
+      const bf16x8* wm[3];
+#pragma unroll
+      for (int a = 0; a < 3; ++a)   // a slot past the last channel reads channel k again (valid memory), result unused
+        wm[a] = Wf + ((size_t)(m0 + a <= k ? m0 + a : k) * 4 * NC + tg0) * KCH * 64 + lane;
+      f32x4 pr[3][TPW];
+#pragma unroll
+      for (int a = 0; a < 3; ++a)
+#pragma unroll
+        for (int cl = 0; cl < TPW; ++cl) pr[a][cl] = f32x4{0.f, 0.f, 0.f, 0.f};
+      for (int kc0 = 0; kc0 < KCH; kc0 += 4) {          // NC is even, so KCH is a multiple of four
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const int kc = kc0 + u;
+          const bf16x8 af = xb[(kc * 4 + q) * XG + n];
+#pragma unroll
+          for (int a = 0; a < 3; ++a)
+#pragma unroll
+            for (int cl = 0; cl < TPW; ++cl) pr[a][cl] = mfma16(af, wm[a][((size_t)cl * KCH + kc) * 64], pr[a][cl]);
+        }
+      }
+#pragma unroll
+      for (int cl = 0; cl < TPW; ++cl) {
+        const bf16x4 gv = *reinterpret_cast<const bf16x4*>(p.gfrag + pair_off_rt(NC, t, p.nbt, bt, tg0 + cl, lane));
+#pragma unroll
+        for (int a = 0; a < 3; ++a)
+#pragma unroll
+          for (int e = 0; e < 4; ++e) ga[a][e] = fmaf(pr[a][cl][e], (float)gv[e], ga[a][e]);
+      }
+    }
+#pragma unroll
+    for (int a = 0; a < 3; ++a)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const float sum = row16_sum_dpp(ga[a][e]);
+        if (n == 0) part[a][wv][4 * q + e] = sum;
+      }
+    lds_barrier();
+    if (tid < 48) {
+      const int a = tid >> 4, row = tid & 15, c = m0 - 1 + a, b = 16 * bt + row;
+      if (c < k && b < B)
+        p.grad_A[((size_t)b * T + t) * k + c] = ((part[a][0][row] + part[a][1][row]) + part[a][2][row]) + part[a][3][row];
+    }
+    lds_barrier();
+  }
+}
+
 // ------------------------------------------------------------------------------------------------
 // Launchers
 // ------------------------------------------------------------------------------------------------
@@ -411,4 +484,15 @@ hipError_t ring_launch_block_bptt(const RingBpttArgs& a, int NC, float* carry, h
     case 2: return block_bptt_rt<2>(a, NC, carry, st);
     default: return block_bptt_rt<1>(a, NC, carry, st);
   }
+}
+
+// a.grad_A, a.gfrag (complete), a.hist, a.r_init; Wf: forward-orientation packed weights (matrix 0 is not read)
+hipError_t ring_launch_block_grad_A(const RingBpttArgs& a, const void* Wf, int NC, hipStream_t st) {
+  if (NC % 2 != 0 || !a.grad_A || !a.gfrag || !a.hist || !a.r_init || !Wf) return hipErrorInvalidValue;
+  if (a.T > 65535) return hipErrorInvalidValue;   // grid.y
+  const size_t dyn = (size_t)2 * NC * 4 * XG * sizeof(bf16x8);
+  hipError_t e = block_attr(ring_block_grad_A_kernel<2>, dyn);
+  if (e != hipSuccess) return e;
+  hipLaunchKernelGGL((ring_block_grad_A_kernel<2>), dim3(a.nbt, a.T), dim3(256), dyn, st, a, (const bf16x8*)Wf, NC);
+  return hipGetLastError();
 }

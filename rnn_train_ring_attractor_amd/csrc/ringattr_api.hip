@@ -266,6 +266,12 @@ int ringattr_bwd_loss(const void* loss_workspace, const void* upstream, const vo
                   workspace, workspace_bytes, stream);
 }
 
+int ringattr_bwd_loss_available(int N, int a_dim, int seq_len, int batch_size) {
+  Geo g;
+  if (N > 1024 || make_geo(N, a_dim, seq_len, batch_size, g) != RINGATTR_OK) return 0;
+  return ring_uses_step_kernels(N, a_dim, g.NC, g.nbt) ? 0 : 1;
+}
+
 static int bwd_impl(const char* who, const void* grad_output, const void* loss_workspace, const void* upstream, const void* A,
                     const void* Wa, float J0, float J1, const void* Wo, const void* bump_history, const void* r_init,
                     void* grad_Wa, void* grad_Wo, float alpha, int N, int a_dim, int seq_len, int batch_size,
@@ -280,9 +286,11 @@ static int bwd_impl(const char* who, const void* grad_output, const void* loss_w
   if (grad_A && (size_t)2 * a_dim * 64 * sizeof(float) > 24 * 1024)
     return fail(RINGATTR_ERR_INVALID, "%s: grad_A is supported for a_dim <= 48 (got %d)", who, a_dim);
   const bool step_family = ring_uses_step_kernels(N, a_dim, g.NC, g.nbt);
-  if (step_family && (grad_A || loss_workspace))
-    return fail(RINGATTR_ERR_INVALID, "%s: grad_A and the fused loss backward are not available on the step-per-launch "
-                "kernels (N = %d > 512, or RINGATTR_BLOCK=1)", who, N);
+  if (step_family && loss_workspace)
+    return fail(RINGATTR_ERR_INVALID, "%s: the fused loss backward is not available on the step-per-launch kernels "
+                "(N = %d > 512, or RINGATTR_BLOCK=1); run ringattr_loss_bwd and pass its result to ringattr_bwd", who, N);
+  if (step_family && grad_A && seq_len > 65535)
+    return fail(RINGATTR_ERR_INVALID, "%s: grad_A on the step-per-launch kernels supports seq_len <= 65535", who);
   if (!aligned16(grad_output) || !aligned16(A) || !aligned16(Wa) || !aligned16(Wo) || !aligned16(bump_history) ||
       !aligned16(r_init) || !aligned16(grad_Wa) || !aligned16(grad_Wo) || !aligned16(saved) ||
       !aligned16(grad_r_init) || !aligned16(grad_A) || !aligned16(workspace))
@@ -366,7 +374,7 @@ static int bwd_impl(const char* who, const void* grad_output, const void* loss_w
   b.gfrag = gfrag;
   b.rfrag = rfrag;
   b.grad_r_init = (float*)grad_r_init;
-  b.grad_A = (float*)grad_A;
+  b.grad_A = step_family ? nullptr : (float*)grad_A;   // the step-per-launch families take dL/dA in a pass of its own
   b.hist = (const float*)bump_history;
   b.r_init = (const float*)r_init;
   b.wide_carry = carry;
@@ -383,6 +391,14 @@ static int bwd_impl(const char* who, const void* grad_output, const void* loss_w
   b.nbt = g.nbt;
   e = ring_launch_bptt(b, g.NC, st);
   if (e != hipSuccess) return hip_fail(e, "BPTT launch");
+  if (step_family && grad_A) {
+    // forward-orientation fragments, packed into the split-K partial area (not yet in use, and never smaller)
+    e = ring_launch_pack((const float*)Wo, (const float*)Wa, partial, N, a_dim, g.NC, 0, 0, 1.f, 0.f, st);
+    if (e != hipSuccess) return hip_fail(e, "pack weights");
+    b.grad_A = (float*)grad_A;
+    e = ring_launch_block_grad_A(b, partial, g.NC, st);
+    if (e != hipSuccess) return hip_fail(e, "grad_A launch");
+  }
 
   RingDwArgs d;
   d.A = (const float*)A;

@@ -123,18 +123,32 @@ class RingRnnLossFunc(Function):
             _lib.check(lib.ringattr_loss_fwd(hist.data_ptr(), angle.data_ptr(), amp.data_ptr() if amp is not None else None,
                                              float(bump_weight), out.data_ptr(), N, T, B, lws.data_ptr(), nbytes,
                                              torch.cuda.current_stream(dev).cuda_stream))
-        ctx.save_for_backward(A, Wa_c, Wo_c, hist, r0, saved, lws)
-        ctx.J0, ctx.J1, ctx.alpha, ctx.act = J0, J1, alpha, act
+        ctx.save_for_backward(A, Wa_c, Wo_c, hist, r0, saved, lws, angle, amp)
+        ctx.J0, ctx.J1, ctx.alpha, ctx.act, ctx.bump_weight = J0, J1, alpha, act, float(bump_weight)
         ctx.mark_non_differentiable(out, hist)
         return out[0].clone(), out, hist
 
     @staticmethod
     def backward(ctx, grad_total, _grad_parts, _grad_hist):
-        A, Wa, Wo, hist, r0, saved, lws = ctx.saved_tensors
+        A, Wa, Wo, hist, r0, saved, lws, angle, amp = ctx.saved_tensors
         grad_Wa, grad_Wo = torch.empty_like(Wa), torch.empty_like(Wo)    # written, not accumulated into
         grad_A = torch.empty_like(A) if ctx.needs_input_grad[0] else None
         grad_r0 = torch.empty_like(r0) if ctx.needs_input_grad[5] else None
         up = grad_total.to(torch.float32).reshape(1).contiguous()
+        T, B, N = hist.shape
+        lib = _lib.load()
+        if not lib.ringattr_bwd_loss_available(N, A.shape[2], T, B):
+            # the step-per-launch kernels (wide rings) read grad_output: the loss head writes it, the backward reads it
+            grad_hist = torch.empty_like(hist)
+            dev = hist.device
+            with torch.cuda.device(dev):
+                _lib.check(lib.ringattr_loss_bwd(hist.data_ptr(), angle.data_ptr(), amp.data_ptr() if amp is not None else None,
+                                                 ctx.bump_weight, up.data_ptr(), grad_hist.data_ptr(), N, T, B,
+                                                 lws.data_ptr(), lws.numel(), torch.cuda.current_stream(dev).cuda_stream))
+            bwd_cuda.bwd(grad_output=grad_hist, A=A, Wa=Wa, J0=ctx.J0, J1=ctx.J1, Wo=Wo, bump_history=hist, r_init=r0,
+                         grad_Wa=grad_Wa, grad_Wo=grad_Wo, alpha=ctx.alpha, activation_type=ctx.act, saved=saved,
+                         grad_A=grad_A, grad_r_init=grad_r0, accumulate=False)
+            return (grad_A, grad_Wa, None, None, grad_Wo, grad_r0, None, None, None, None, None) + (None,) * ctx.extra_inputs
         bwd_cuda.bwd(grad_output=None, A=A, Wa=Wa, J0=ctx.J0, J1=ctx.J1, Wo=Wo, bump_history=hist, r_init=r0,
                      grad_Wa=grad_Wa, grad_Wo=grad_Wo, alpha=ctx.alpha, activation_type=ctx.act, saved=saved,
                      grad_A=grad_A, grad_r_init=grad_r0, loss_workspace=lws, loss_upstream=up, accumulate=False)

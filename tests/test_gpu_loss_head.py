@@ -75,7 +75,8 @@ def test_loss_head_agrees_with_the_torch_chain_on_operator_output(gpu_device):
     (37, 9, 2, 200, "tanh", True, "1", "random"),     # the streaming kernels, four column tiles
     (20, 6, 3, 96, "silu", True, "0", "random"),      # the streaming kernels, two column tiles, three action channels
     (40, 5, 2, 512, "tanh", True, "0", "random"),     # widest tiling
-], ids=["n256_full", "n256_random", "n200_masked", "n200_streaming", "n96_k3", "n512"])
+    (24, 5, 2, 1024, "tanh", True, "0", "random"),    # wide ring: the operator chains loss backward and time-loop backward
+], ids=["n256_full", "n256_random", "n200_masked", "n200_streaming", "n96_k3", "n512", "n1024_step"])
 def test_time_loop_and_loss_as_one_operator(B, T, k, N, act, own, streaming, weights, gpu_device, monkeypatch):
     """ring_rnn_loss_func (one backward call, the loss gradient formed inside the BPTT kernel) against
     ring_rnn_cuda_func + ring_loss_pair (the gradient written to HBM and read back), and against the fp64 oracle:
@@ -123,8 +124,9 @@ def test_time_loop_and_loss_as_one_operator(B, T, k, N, act, own, streaming, wei
         assert O.max_rel_err(got, ref[key]) <= 2e-2, key
 
 
-@pytest.mark.parametrize("B,T,k,N,act", [(24, 8, 2, 120, "tanh"), (20, 6, 2, 256, "gelu"), (18, 5, 3, 300, "silu")],
-                         ids=["n120", "n256", "n300_k3"])
+@pytest.mark.parametrize("B,T,k,N,act", [(24, 8, 2, 120, "tanh"), (20, 6, 2, 256, "gelu"), (18, 5, 3, 300, "silu"),
+                                         (16, 4, 2, 640, "tanh")],
+                         ids=["n120", "n256", "n300_k3", "n640_step"])
 def test_one_operator_also_returns_the_action_signal_gradient(B, T, k, N, act, gpu_device):
     """dL/d action_signal and dL/d r_init through ring_rnn_loss_func (loss gradient formed inside the BPTT kernel
     that also produces dL/dA) against ring_rnn_cuda_func + ring_loss_pair."""

@@ -205,8 +205,10 @@ def test_backward_without_saved_buffer_rebuilds_it(case, gpu_device):
 @pytest.mark.parametrize("B,T,k,N,act,action", [(40, 24, 2, 120, "tanh", "lr"), (48, 20, 2, 256, "gelu", "lr"),
                                                 (21, 9, 3, 200, "silu", "dense"), (32, 12, 16, 64, "tanh", "spread"),
                                                 (32, 7, 2, 256, "tanh", "dense"), (37, 10, 2, 200, "silu", "dense"),
-                                                (64, 66, 2, 256, "relu", "lr")],
-                         ids=["n120", "n256", "ragged_k3", "k16", "n256_odd_T", "n200_ragged_resident", "n256_relu_T66"])
+                                                (64, 66, 2, 256, "relu", "lr"), (24, 6, 3, 700, "silu", "dense"),
+                                                (20, 5, 2, 1024, "tanh", "lr"), (18, 4, 4, 1300, "gelu", "spread")],
+                         ids=["n120", "n256", "ragged_k3", "k16", "n256_odd_T", "n200_ragged_resident", "n256_relu_T66",
+                              "n700_k3_step", "n1024_step", "n1300_k4_step"])
 def test_gradients_of_action_signal_and_initial_state(B, T, k, N, act, action, gpu_device):
     """dL/d action_signal and dL/d r_init, which the reference operator does not return (cpp/ring_rnn_cuda.py:144);
     pinned by the fp64 oracle, whose grad_A / grad_r_init are themselves checked by finite differences."""
