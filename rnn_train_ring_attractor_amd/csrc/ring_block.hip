@@ -22,6 +22,24 @@
 
 namespace {
 
+// Which (row group, column block) a workgroup takes.  Workgroups go to the eight XCDs round-robin by linear index,
+// and every XCD has its own L2.  With the plain (x = row group, y = column block) order each XCD sees every column
+// block, i.e. pulls the whole packed weight set out of HBM for itself -- eight fetches of every weight byte per
+// step, which is what bounds small batches of wide rings.  When the column blocks divide by eight, XCD x instead
+// owns column blocks x * cpx .. (x+1) * cpx - 1 for all row groups: each weight byte leaves HBM once per step and is
+// shared through that XCD's L2 by the row groups running side by side.  (Any placement gives correct results; the
+// mapping only decides what the caches see.)  xcd_map = 0 keeps the plain order.
+__device__ __forceinline__ void block_coords(int xcd_map, int& rg, int& cb) {
+  const int nrg = gridDim.x, ncb = gridDim.y;
+  rg = blockIdx.x;
+  cb = blockIdx.y;
+  if (xcd_map && (ncb & 7) == 0) {
+    const int L = blockIdx.x + nrg * blockIdx.y, xcd = L & 7, w = L >> 3, cpx = ncb >> 3;
+    rg = w % nrg;
+    cb = xcd * cpx + w / nrg;
+  }
+}
+
 // Stage RT batch tiles' operand rows (bf16, tile i at xb + i * slots) and their fp32 row sums (rs[16*i + row]).
 template <int RT, typename F>
 __device__ __forceinline__ void stage_tiles(bf16x8* xb, int slots, float* rs, int NPAD, int tid, F&& value4) {
@@ -79,7 +97,7 @@ __device__ __forceinline__ void block_products(const bf16x8* xb, int slots, cons
                                                f32x4 (&acc)[RT][TPW]) {
   const int KCH = 2 * NC, q = lane >> 4, n = lane & 15;
   const unsigned long long active = staged ? active_channels_rt<RT>(gl, k, lane) : ~0ull;
-  constexpr int PD = 2;                                    // K chunks of weight fragments in flight
+  constexpr int PD = 8 / TPW;                              // K chunks of weight fragments in flight (24 KiB per wave)
   for (int m0 = 0; m0 <= k; m0 += 3) {
     bool use[3];
     const bf16x8* wm[3];
@@ -165,12 +183,14 @@ __device__ __forceinline__ void block_products(const bf16x8* xb, int slots, cons
 // One forward step for RT batch tiles x 64*TPW neurons per workgroup (REBUILD: the saved record of every step at
 // once from an existing history, grid.z = T).
 template <int ACT, bool REBUILD, int RT, int TPW>
-__global__ __launch_bounds__(256) void ring_block_fwd_kernel(RingFwdArgs p, int NC, int t_arg) {
+__global__ __launch_bounds__(256) void ring_block_fwd_kernel(RingFwdArgs p, int NC, int t_arg, int xcd_map) {
   extern __shared__ __attribute__((aligned(16))) char block_lds[];
   bf16x8* xb = reinterpret_cast<bf16x8*>(block_lds);
   __shared__ float rs[16 * RT];
   const int tid = threadIdx.x, wv = tid >> 6, lane = tid & 63, q = lane >> 4, n = lane & 15;
-  const int bt0 = blockIdx.x * RT, cb = blockIdx.y, t = REBUILD ? (int)blockIdx.z : t_arg;
+  int rgi, cb;
+  block_coords(xcd_map, rgi, cb);
+  const int bt0 = rgi * RT, t = REBUILD ? (int)blockIdx.z : t_arg;
   const int N = p.N, B = p.B, T = p.T, NPAD = 64 * NC, slots = 2 * NC * 4 * XG;
   const bool staged = p.k <= BN_GATE_KMAX;
   float* gl = reinterpret_cast<float*>(xb + (size_t)RT * slots);
@@ -236,12 +256,14 @@ __global__ __launch_bounds__(256) void ring_block_fwd_kernel(RingFwdArgs p, int 
 // One BPTT step t for RT batch tiles x 64*TPW neurons per workgroup (see ring_wide_bptt_kernel for the recurrence).
 template <int RT, int TPW>
 __global__ __launch_bounds__(256) void ring_block_bptt_kernel(RingBpttArgs p, int NC, int t, const float* carry_in,
-                                                              float* carry_out) {
+                                                              float* carry_out, int xcd_map) {
   extern __shared__ __attribute__((aligned(16))) char block_lds[];
   bf16x8* xb = reinterpret_cast<bf16x8*>(block_lds);
   __shared__ float rs[16 * RT];
   const int tid = threadIdx.x, wv = tid >> 6, lane = tid & 63, q = lane >> 4, n = lane & 15;
-  const int bt0 = blockIdx.x * RT, cb = blockIdx.y;
+  int rgi, cb;
+  block_coords(xcd_map, rgi, cb);
+  const int bt0 = rgi * RT;
   const int N = p.N, B = p.B, T = p.T, NPAD = 64 * NC, slots = 2 * NC * 4 * XG;
   const bool staged = p.k <= BN_GATE_KMAX;
   float* gl = reinterpret_cast<float*>(xb + (size_t)RT * slots);
@@ -396,18 +418,45 @@ static size_t block_lds_bytes(int NC, int RT, int k) {
   return (size_t)RT * 2 * NC * 4 * XG * sizeof(bf16x8) + (k <= BN_GATE_KMAX ? (size_t)RT * 16 * k * sizeof(float) : 0);
 }
 
-// Row tiles per workgroup: two while LDS holds their operand rows and the grid still covers the device about
-// once, else one; tiles per wave: two (a workgroup then owns 128 neurons).
+// Tiles per wave (a workgroup owns 64 * tpw neurons) and row tiles per workgroup, from measurements on 16 to 256
+// batch tiles at N = 1024 and 2048:
+//  * many matrices (more than two groups of three, e.g. 16 action channels): the weight stream dominates.  Two row
+//    tiles per workgroup (every fetched fragment feeds two MFMAs) and one tile per wave while all workgroups are
+//    resident at once (twice the streams in flight), two tiles per wave beyond that;
+//  * few matrices: staging the operand rows is what a workgroup waits for, so one row tile and two tiles per wave
+//    (fewest workgroups re-staging the same rows) until the grid covers the device also with two row tiles.
+// RINGATTR_BLOCK_SHAPE=<rt><tpw> (e.g. 21) forces a shape (cross-checks).
+bool ring_block_many_matrices(int k) { return 1 + k > 6; }
+
 void ring_block_geometry(int NC, int nbt, int k, int* rt_out, int* tpw_out) {
   int dev = 0, cus = 0;
   if (hipGetDevice(&dev) != hipSuccess ||
       hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) cus = 256;
-  const int tpw = 2;
-  const int ncb = NC / tpw;
-  int rt = 2;
-  while (rt > 1 && (block_lds_bytes(NC, rt, k) + 2 * 1024 > 160 * 1024 || (long)((nbt + rt - 1) / rt) * ncb < cus)) rt >>= 1;
+  const size_t lds_cap = 160 * 1024 - 2 * 1024;
+  int rt, tpw;
+  if (ring_block_many_matrices(k)) {
+    rt = (nbt >= 2 && block_lds_bytes(NC, 2, k) <= lds_cap) ? 2 : 1;
+    const long per_cu = (long)(lds_cap / block_lds_bytes(NC, rt, k));
+    tpw = (long)((nbt + rt - 1) / rt) * NC <= (long)cus * (per_cu > 0 ? per_cu : 1) ? 1 : 2;
+  } else {
+    tpw = 2;
+    rt = (block_lds_bytes(NC, 2, k) <= lds_cap && (long)((nbt + 1) / 2) * (NC / 2) >= cus) ? 2 : 1;
+  }
+  if (const char* v = getenv("RINGATTR_BLOCK_SHAPE")) {
+    if ((v[0] == '1' || v[0] == '2') && (v[1] == '1' || v[1] == '2') && v[2] == 0) {
+      const int frt = v[0] - '0';
+      if (block_lds_bytes(NC, frt, k) <= lds_cap) rt = frt;
+      tpw = v[1] - '0';
+    }
+  }
   *rt_out = rt;
   *tpw_out = tpw;
+}
+
+// RINGATTR_XCD_MAP=0: plain workgroup order (see block_coords)
+static int block_xcd_map() {
+  const char* v = getenv("RINGATTR_XCD_MAP");
+  return (v && v[0] == '0') ? 0 : 1;
 }
 
 template <typename K>
@@ -415,21 +464,21 @@ static hipError_t block_attr(K kern, size_t dyn) {
   return hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)dyn);
 }
 
-template <int ACT, int RT>
-static hipError_t block_fwd_rt(const RingFwdArgs& a, int NC, bool rebuild, hipStream_t st) {
-  constexpr int TPW = 2;
+template <int ACT, int RT, int TPW>
+static hipError_t block_fwd_shape(const RingFwdArgs& a, int NC, bool rebuild, hipStream_t st) {
   const size_t dyn = block_lds_bytes(NC, RT, a.k);
   const dim3 grid((a.nbt + RT - 1) / RT, NC / TPW, rebuild ? a.T : 1);
+  const int xm = block_xcd_map();
   if (rebuild) {
     hipError_t e = block_attr(ring_block_fwd_kernel<ACT, true, RT, TPW>, dyn);
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL((ring_block_fwd_kernel<ACT, true, RT, TPW>), grid, dim3(256), dyn, st, a, NC, 0);
+    hipLaunchKernelGGL((ring_block_fwd_kernel<ACT, true, RT, TPW>), grid, dim3(256), dyn, st, a, NC, 0, xm);
     return hipGetLastError();
   }
   hipError_t e = block_attr(ring_block_fwd_kernel<ACT, false, RT, TPW>, dyn);
   if (e != hipSuccess) return e;
   for (int t = 0; t < a.T; ++t) {
-    hipLaunchKernelGGL((ring_block_fwd_kernel<ACT, false, RT, TPW>), grid, dim3(256), dyn, st, a, NC, t);
+    hipLaunchKernelGGL((ring_block_fwd_kernel<ACT, false, RT, TPW>), grid, dim3(256), dyn, st, a, NC, t, xm);
     e = hipGetLastError();
     if (e != hipSuccess) return e;
   }
@@ -437,11 +486,9 @@ static hipError_t block_fwd_rt(const RingFwdArgs& a, int NC, bool rebuild, hipSt
 }
 
 template <int ACT>
-static hipError_t block_fwd_act(const RingFwdArgs& a, int NC, bool rebuild, int rt, hipStream_t st) {
-  switch (rt) {
-    case 2: return block_fwd_rt<ACT, 2>(a, NC, rebuild, st);
-    default: return block_fwd_rt<ACT, 1>(a, NC, rebuild, st);
-  }
+static hipError_t block_fwd_act(const RingFwdArgs& a, int NC, bool rebuild, int rt, int tpw, hipStream_t st) {
+  if (rt == 2) return tpw == 2 ? block_fwd_shape<ACT, 2, 2>(a, NC, rebuild, st) : block_fwd_shape<ACT, 2, 1>(a, NC, rebuild, st);
+  return tpw == 2 ? block_fwd_shape<ACT, 1, 2>(a, NC, rebuild, st) : block_fwd_shape<ACT, 1, 1>(a, NC, rebuild, st);
 }
 
 hipError_t ring_launch_block_fwd(const RingFwdArgs& a, int NC, bool rebuild, hipStream_t st) {
@@ -449,26 +496,26 @@ hipError_t ring_launch_block_fwd(const RingFwdArgs& a, int NC, bool rebuild, hip
   int rt, tpw;
   ring_block_geometry(NC, a.nbt, a.k, &rt, &tpw);
   switch (a.act) {
-    case ACT_RELU: return block_fwd_act<ACT_RELU>(a, NC, rebuild, rt, st);
-    case ACT_GELU: return block_fwd_act<ACT_GELU>(a, NC, rebuild, rt, st);
-    case ACT_TANH: return block_fwd_act<ACT_TANH>(a, NC, rebuild, rt, st);
-    case ACT_SILU: return block_fwd_act<ACT_SILU>(a, NC, rebuild, rt, st);
+    case ACT_RELU: return block_fwd_act<ACT_RELU>(a, NC, rebuild, rt, tpw, st);
+    case ACT_GELU: return block_fwd_act<ACT_GELU>(a, NC, rebuild, rt, tpw, st);
+    case ACT_TANH: return block_fwd_act<ACT_TANH>(a, NC, rebuild, rt, tpw, st);
+    case ACT_SILU: return block_fwd_act<ACT_SILU>(a, NC, rebuild, rt, tpw, st);
     default: return hipErrorInvalidValue;
   }
 }
 
-template <int RT>
-static hipError_t block_bptt_rt(const RingBpttArgs& a, int NC, float* carry, hipStream_t st) {
-  constexpr int TPW = 2;
+template <int RT, int TPW>
+static hipError_t block_bptt_shape(const RingBpttArgs& a, int NC, float* carry, hipStream_t st) {
   const size_t dyn = block_lds_bytes(NC, RT, a.k);
   hipError_t e = block_attr(ring_block_bptt_kernel<RT, TPW>, dyn);
   if (e != hipSuccess) return e;
   const size_t half = (size_t)16 * a.nbt * 64 * NC;
   const dim3 grid((a.nbt + RT - 1) / RT, NC / TPW);
+  const int xm = block_xcd_map();
   for (int t = a.T - 1, u = 0; t >= 0; --t, ++u) {
     const float* cin = (u == 0) ? nullptr : carry + (size_t)((u - 1) & 1) * half;
     float* cout = carry + (size_t)(u & 1) * half;
-    hipLaunchKernelGGL((ring_block_bptt_kernel<RT, TPW>), grid, dim3(256), dyn, st, a, NC, t, cin, cout);
+    hipLaunchKernelGGL((ring_block_bptt_kernel<RT, TPW>), grid, dim3(256), dyn, st, a, NC, t, cin, cout, xm);
     e = hipGetLastError();
     if (e != hipSuccess) return e;
   }
@@ -480,10 +527,8 @@ hipError_t ring_launch_block_bptt(const RingBpttArgs& a, int NC, float* carry, h
   if (NC % 2 != 0) return hipErrorInvalidValue;
   int rt, tpw;
   ring_block_geometry(NC, a.nbt, a.k, &rt, &tpw);
-  switch (rt) {
-    case 2: return block_bptt_rt<2>(a, NC, carry, st);
-    default: return block_bptt_rt<1>(a, NC, carry, st);
-  }
+  if (rt == 2) return tpw == 2 ? block_bptt_shape<2, 2>(a, NC, carry, st) : block_bptt_shape<2, 1>(a, NC, carry, st);
+  return tpw == 2 ? block_bptt_shape<1, 2>(a, NC, carry, st) : block_bptt_shape<1, 1>(a, NC, carry, st);
 }
 
 // a.grad_A, a.gfrag (complete), a.hist, a.r_init; Wf: forward-orientation packed weights (matrix 0 is not read)

@@ -994,21 +994,23 @@ bool ring_uses_step_kernels(int N, int k, int NCv, int nbt) {
   return false;
 }
 
-// Which step-per-launch family: the block kernels (K-outer, three matrices' products at a time) are ahead on few
-// batch tiles, the one-tile-per-workgroup kernels of ring_bign.hip (up to 1.6 times) on many; measured crossover
-// about nbt * NC = 512 (N = 1024: 512 rows, N = 2048: 256 rows).  RINGATTR_WIDE=1 / 0 forces one or the other
-// (cross-checks); the two share the record layout, so forward and backward may choose independently.
-static bool step_prefers_wide(int NCv, int nbt) {
+// Which step-per-launch family.  With few matrices the block kernels (K-outer, three matrices' products at a time)
+// are ahead on few batch tiles and the one-tile-per-workgroup kernels of ring_bign.hip (up to 1.6 times) on many;
+// measured crossover about nbt * NC = 512 (N = 1024: 512 rows, N = 2048: 256 rows).  With many matrices (16 action
+// channels) the block kernels lead at every measured batch size (1.3 to 2 times).  RINGATTR_WIDE=1 / 0 forces one or
+// the other (cross-checks); the two share the record layout, so forward and backward may choose independently.
+static bool step_prefers_wide(int NCv, int nbt, int k) {
   if (NCv % 4 != 0) return false;
   const char* v = getenv("RINGATTR_WIDE");
   if (v && (v[0] == '0' || v[0] == '1')) return v[0] == '1';
+  if (ring_block_many_matrices(k)) return false;
   return (long)nbt * NCv > 512;
 }
 
 hipError_t ring_launch_fwd(const RingFwdArgs& a, int NCv, hipStream_t st) {
   ProfScope prof(1, st);
   if (ring_uses_step_kernels(a.N, a.k, NCv, a.nbt))
-    return step_prefers_wide(NCv, a.nbt) ? ring_launch_wide_fwd(a, NCv, false, 4, st) : ring_launch_block_fwd(a, NCv, false, st);
+    return step_prefers_wide(NCv, a.nbt, a.k) ? ring_launch_wide_fwd(a, NCv, false, 4, st) : ring_launch_block_fwd(a, NCv, false, st);
   // A forward that keeps nothing for a backward, on few batch tiles, with weights too large to stay on chip: the
   // persistent kernels would pull every weight byte through a handful of compute units once per step.  One launch per
   // step with the output columns split over workgroups spreads that over the device (a launch costs a few
@@ -1040,7 +1042,7 @@ hipError_t ring_launch_fwd(const RingFwdArgs& a, int NCv, hipStream_t st) {
 hipError_t ring_launch_rebuild(const RingFwdArgs& a, int NCv, hipStream_t st) {
   ProfScope prof(2, st);
   if (ring_uses_step_kernels(a.N, a.k, NCv, a.nbt))
-    return step_prefers_wide(NCv, a.nbt) ? ring_launch_wide_fwd(a, NCv, true, 4, st) : ring_launch_block_fwd(a, NCv, true, st);
+    return step_prefers_wide(NCv, a.nbt, a.k) ? ring_launch_wide_fwd(a, NCv, true, 4, st) : ring_launch_block_fwd(a, NCv, true, st);
   if (ring_uses_resident(a.N, a.k)) {
     RingFwdArgs f = a;
     f.hist = nullptr;
@@ -1064,7 +1066,7 @@ hipError_t ring_launch_bptt(const RingBpttArgs& a, int NCv, hipStream_t st) {
   hipError_t e = hipErrorInvalidValue;
   if (ring_uses_step_kernels(a.N, a.k, NCv, a.nbt)) {
     if (a.grad_A || a.loss_coef || !a.wide_carry) return hipErrorInvalidValue;   // the C ABI rejects these before
-    return step_prefers_wide(NCv, a.nbt) ? ring_launch_wide_bptt(a, NCv, a.wide_carry, st)
+    return step_prefers_wide(NCv, a.nbt, a.k) ? ring_launch_wide_bptt(a, NCv, a.wide_carry, st)
                                   : ring_launch_block_bptt(a, NCv, a.wide_carry, st);
   }
   // (the parentheses keep the commas of the template argument lists away from the dispatch macros)

@@ -77,6 +77,7 @@ hipError_t ring_launch_wide_bptt(const RingBpttArgs& a, int NC, float* carry, hi
 // carry buffer as the wide-ring kernels.
 hipError_t ring_launch_block_fwd(const RingFwdArgs& a, int NC, bool rebuild, hipStream_t st);
 hipError_t ring_launch_block_bptt(const RingBpttArgs& a, int NC, float* carry, hipStream_t st);
+bool ring_block_many_matrices(int k);   // the weight stream dominates a step: the block kernels lead at any batch size
 // dL/dA of the step-per-launch families: a separate pass after the BPTT steps (Wf: forward-orientation packed weights)
 hipError_t ring_launch_block_grad_A(const RingBpttArgs& a, const void* Wf, int NC, hipStream_t st);
 // which kernel family runs a problem with a saved record: 0 persistent, 1 step-per-launch (wide or block)

@@ -256,6 +256,39 @@ def test_step_per_launch_families_agree(B, T, k, N, act, force, saved, gpu_devic
     assert O.cosine(b[3], ref["grad_r_init"]) >= floor
 
 
+@pytest.mark.parametrize("B,T,k,N,act", [(72, 5, 3, 1024, "tanh"), (40, 4, 7, 640, "silu")], ids=["n1024_k3", "n640_k7"])
+def test_block_kernel_shapes_and_workgroup_orders_agree_bitwise(B, T, k, N, act, gpu_device, monkeypatch):
+    """The block kernels come in four shapes (one or two row tiles per workgroup, one or two column tiles per wave)
+    and two workgroup orders (plain, or column blocks pinned to an XCD).  Shape and order decide which workgroup
+    computes an element, not how: every variant must give the same bits, forward and backward."""
+    from rnn_train_ring_attractor_amd import rnn_cuda
+    print(f"[case] block shapes B={B} T={T} k={k} N={N} {act}", flush=True)
+    p = make_problem(91 + N, B, T, k, N)
+    acts = {"relu": 0, "gelu": 1, "tanh": 2, "silu": 3}
+    monkeypatch.setenv("RINGATTR_WIDE", "0")
+    outs = []
+    for shape, xcd in (("12", "1"), ("11", "1"), ("21", "1"), ("22", "1"), ("12", "0"), ("21", "0")):
+        monkeypatch.setenv("RINGATTR_BLOCK_SHAPE", shape)
+        monkeypatch.setenv("RINGATTR_XCD_MAP", xcd)
+        A, Wa, Wo, r0, G = (_t(p[x], gpu_device) for x in ("A", "Wa", "Wo", "r0", "G"))
+        hist = torch.empty(T, B, N, device=gpu_device)
+        sv = torch.empty(rnn_cuda.saved_nbytes(N, k, T, B), dtype=torch.uint8, device=gpu_device)
+        rnn_cuda.fwd_cuda.fwd(A=A, Wa=Wa, J0=-0.1, J1=0.3, Wo=Wo, r_init=r0, bump_history=hist, alpha=0.15,
+                              activation_type=acts[act], saved=sv)
+        gWa, gWo = torch.zeros_like(Wa), torch.zeros_like(Wo)
+        gr0, gA = torch.empty_like(r0), torch.empty_like(A)
+        rnn_cuda.bwd_cuda.bwd(grad_output=G, A=A, Wa=Wa, J0=-0.1, J1=0.3, Wo=Wo, bump_history=hist, r_init=r0,
+                              grad_Wa=gWa, grad_Wo=gWo, alpha=0.15, activation_type=acts[act],
+                              saved=sv, grad_r_init=gr0, grad_A=gA)
+        torch.cuda.synchronize()
+        outs.append([x.cpu().numpy() for x in (hist, gWa, gWo, gr0, gA)])
+    for other in outs[1:]:
+        for a, b in zip(outs[0], other):
+            assert np.array_equal(a, b)
+    ref_hist, _ = O.forward_dense(p["A"], p["Wa"], -0.1, 0.3, p["Wo"], p["r0"], 0.15, act)
+    assert O.max_rel_err(outs[0][0], ref_hist) <= TRAJ_TOL
+
+
 @pytest.mark.parametrize("driven", [(3, 9), (5,), ()], ids=["two", "one", "none"])
 def test_silent_action_channels_are_compacted(driven, gpu_device, monkeypatch):
     """With a_dim > 2 and the caller's statement that at most two named channels are driven, the Python operator runs
