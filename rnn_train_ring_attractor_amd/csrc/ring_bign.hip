@@ -82,13 +82,15 @@ __device__ __forceinline__ void wide_products(const bf16x8* xb, const bf16x8* __
 // TPW column tiles per wave: a workgroup owns 64 * TPW neurons.  Wide rings use 4; narrower rings with few batch
 // tiles use fewer so that the step still spreads over the device (forward without saved record only).
 template <int ACT, bool REBUILD, int TPW>
-__global__ __launch_bounds__(256) void ring_wide_fwd_kernel(RingFwdArgs p, int NC, int t_arg) {
+__global__ __launch_bounds__(256) void ring_wide_fwd_kernel(RingFwdArgs p, int NC, int t_arg, int xcd_map) {
   extern __shared__ __attribute__((aligned(16))) char wide_lds[];
   bf16x8* xb = reinterpret_cast<bf16x8*>(wide_lds);
   __shared__ float rs[16];
   __shared__ float gl[16 * BN_GATE_KMAX];
   const int tid = threadIdx.x, wv = tid >> 6, lane = tid & 63, q = lane >> 4, n = lane & 15;
-  const int bt = blockIdx.x, cb = blockIdx.y, t = REBUILD ? (int)blockIdx.z : t_arg;
+  int bt, cb;
+  step_block_coords(xcd_map, bt, cb);
+  const int t = REBUILD ? (int)blockIdx.z : t_arg;
   const int N = p.N, B = p.B, T = p.T, NPAD = 64 * NC;
   const bool staged = p.k <= BN_GATE_KMAX;
   const float* prev = (t == 0) ? p.r_init : p.hist + (size_t)(t - 1) * B * N;
@@ -148,13 +150,14 @@ __global__ __launch_bounds__(256) void ring_wide_fwd_kernel(RingFwdArgs p, int N
 // tile), carry_out = (1-alpha) G + J0 sum(g) + J1 (g Wo) + sum_c A_c (g Wa_c) for the workgroup's own 256 neurons.
 // carry_in == nullptr at the last time step (zero carry); at t == 0 the host points carry_out at grad_r_init or scratch.
 __global__ __launch_bounds__(256) void ring_wide_bptt_kernel(RingBpttArgs p, int NC, int t, const float* carry_in,
-                                                             float* carry_out) {
+                                                             float* carry_out, int xcd_map) {
   extern __shared__ __attribute__((aligned(16))) char wide_lds[];
   bf16x8* xb = reinterpret_cast<bf16x8*>(wide_lds);
   __shared__ float rs[16];
   __shared__ float gl[16 * BN_GATE_KMAX];
   const int tid = threadIdx.x, wv = tid >> 6, lane = tid & 63, q = lane >> 4, n = lane & 15;
-  const int bt = blockIdx.x, cb = blockIdx.y;
+  int bt, cb;
+  step_block_coords(xcd_map, bt, cb);
   const int N = p.N, B = p.B, T = p.T, NPAD = 64 * NC;
   const bool staged = p.k <= BN_GATE_KMAX;
   const size_t rows_pad = (size_t)16 * p.nbt;
@@ -235,13 +238,13 @@ static hipError_t wide_fwd_tpw(const RingFwdArgs& a, int NC, bool rebuild, hipSt
   if (rebuild) {
     hipError_t e = wide_attr(ring_wide_fwd_kernel<ACT, true, TPW>, dyn);
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL((ring_wide_fwd_kernel<ACT, true, TPW>), dim3(a.nbt, ncb, a.T), dim3(256), dyn, st, a, NC, 0);
+    hipLaunchKernelGGL((ring_wide_fwd_kernel<ACT, true, TPW>), dim3(a.nbt, ncb, a.T), dim3(256), dyn, st, a, NC, 0, step_xcd_map());
     return hipGetLastError();
   }
   hipError_t e = wide_attr(ring_wide_fwd_kernel<ACT, false, TPW>, dyn);
   if (e != hipSuccess) return e;
   for (int t = 0; t < a.T; ++t) {
-    hipLaunchKernelGGL((ring_wide_fwd_kernel<ACT, false, TPW>), dim3(a.nbt, ncb), dim3(256), dyn, st, a, NC, t);
+    hipLaunchKernelGGL((ring_wide_fwd_kernel<ACT, false, TPW>), dim3(a.nbt, ncb), dim3(256), dyn, st, a, NC, t, step_xcd_map());
     e = hipGetLastError();
     if (e != hipSuccess) return e;
   }
@@ -277,7 +280,7 @@ hipError_t ring_launch_wide_bptt(const RingBpttArgs& a, int NC, float* carry, hi
   for (int t = a.T - 1, u = 0; t >= 0; --t, ++u) {
     const float* cin = (u == 0) ? nullptr : carry + (size_t)((u - 1) & 1) * half;
     float* cout = carry + (size_t)(u & 1) * half;
-    hipLaunchKernelGGL(ring_wide_bptt_kernel, dim3(a.nbt, ncb), dim3(256), dyn, st, a, NC, t, cin, cout);
+    hipLaunchKernelGGL(ring_wide_bptt_kernel, dim3(a.nbt, ncb), dim3(256), dyn, st, a, NC, t, cin, cout, step_xcd_map());
     e = hipGetLastError();
     if (e != hipSuccess) return e;
   }

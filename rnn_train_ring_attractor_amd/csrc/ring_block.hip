@@ -22,24 +22,6 @@
 
 namespace {
 
-// Which (row group, column block) a workgroup takes.  Workgroups go to the eight XCDs round-robin by linear index,
-// and every XCD has its own L2.  With the plain (x = row group, y = column block) order each XCD sees every column
-// block, i.e. pulls the whole packed weight set out of HBM for itself -- eight fetches of every weight byte per
-// step, which is what bounds small batches of wide rings.  When the column blocks divide by eight, XCD x instead
-// owns column blocks x * cpx .. (x+1) * cpx - 1 for all row groups: each weight byte leaves HBM once per step and is
-// shared through that XCD's L2 by the row groups running side by side.  (Any placement gives correct results; the
-// mapping only decides what the caches see.)  xcd_map = 0 keeps the plain order.
-__device__ __forceinline__ void block_coords(int xcd_map, int& rg, int& cb) {
-  const int nrg = gridDim.x, ncb = gridDim.y;
-  rg = blockIdx.x;
-  cb = blockIdx.y;
-  if (xcd_map && (ncb & 7) == 0) {
-    const int L = blockIdx.x + nrg * blockIdx.y, xcd = L & 7, w = L >> 3, cpx = ncb >> 3;
-    rg = w % nrg;
-    cb = xcd * cpx + w / nrg;
-  }
-}
-
 // Stage RT batch tiles' operand rows (bf16, tile i at xb + i * slots) and their fp32 row sums (rs[16*i + row]).
 template <int RT, typename F>
 __device__ __forceinline__ void stage_tiles(bf16x8* xb, int slots, float* rs, int NPAD, int tid, F&& value4) {
@@ -189,7 +171,7 @@ __global__ __launch_bounds__(256) void ring_block_fwd_kernel(RingFwdArgs p, int 
   __shared__ float rs[16 * RT];
   const int tid = threadIdx.x, wv = tid >> 6, lane = tid & 63, q = lane >> 4, n = lane & 15;
   int rgi, cb;
-  block_coords(xcd_map, rgi, cb);
+  step_block_coords(xcd_map, rgi, cb);
   const int bt0 = rgi * RT, t = REBUILD ? (int)blockIdx.z : t_arg;
   const int N = p.N, B = p.B, T = p.T, NPAD = 64 * NC, slots = 2 * NC * 4 * XG;
   const bool staged = p.k <= BN_GATE_KMAX;
@@ -262,7 +244,7 @@ __global__ __launch_bounds__(256) void ring_block_bptt_kernel(RingBpttArgs p, in
   __shared__ float rs[16 * RT];
   const int tid = threadIdx.x, wv = tid >> 6, lane = tid & 63, q = lane >> 4, n = lane & 15;
   int rgi, cb;
-  block_coords(xcd_map, rgi, cb);
+  step_block_coords(xcd_map, rgi, cb);
   const int bt0 = rgi * RT;
   const int N = p.N, B = p.B, T = p.T, NPAD = 64 * NC, slots = 2 * NC * 4 * XG;
   const bool staged = p.k <= BN_GATE_KMAX;
@@ -453,12 +435,6 @@ void ring_block_geometry(int NC, int nbt, int k, int* rt_out, int* tpw_out) {
   *tpw_out = tpw;
 }
 
-// RINGATTR_XCD_MAP=0: plain workgroup order (see block_coords)
-static int block_xcd_map() {
-  const char* v = getenv("RINGATTR_XCD_MAP");
-  return (v && v[0] == '0') ? 0 : 1;
-}
-
 template <typename K>
 static hipError_t block_attr(K kern, size_t dyn) {
   return hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)dyn);
@@ -468,7 +444,7 @@ template <int ACT, int RT, int TPW>
 static hipError_t block_fwd_shape(const RingFwdArgs& a, int NC, bool rebuild, hipStream_t st) {
   const size_t dyn = block_lds_bytes(NC, RT, a.k);
   const dim3 grid((a.nbt + RT - 1) / RT, NC / TPW, rebuild ? a.T : 1);
-  const int xm = block_xcd_map();
+  const int xm = step_xcd_map();
   if (rebuild) {
     hipError_t e = block_attr(ring_block_fwd_kernel<ACT, true, RT, TPW>, dyn);
     if (e != hipSuccess) return e;
@@ -511,7 +487,7 @@ static hipError_t block_bptt_shape(const RingBpttArgs& a, int NC, float* carry, 
   if (e != hipSuccess) return e;
   const size_t half = (size_t)16 * a.nbt * 64 * NC;
   const dim3 grid((a.nbt + RT - 1) / RT, NC / TPW);
-  const int xm = block_xcd_map();
+  const int xm = step_xcd_map();
   for (int t = a.T - 1, u = 0; t >= 0; --t, ++u) {
     const float* cin = (u == 0) ? nullptr : carry + (size_t)((u - 1) & 1) * half;
     float* cout = carry + (size_t)(u & 1) * half;

@@ -4,9 +4,38 @@
 #include "ring_common.hpp"
 #include "ring_kernels.hpp"
 
+#include <stdlib.h>
+
 namespace {
 
 constexpr int BN_GATE_KMAX = 64;
+
+// Which (row group, column block) a workgroup takes.  Workgroups go to the eight XCDs round-robin by linear index,
+// and every XCD has its own L2.  With the plain (x = row group, y = column block) order each XCD sees every column
+// block, i.e. pulls the whole packed weight set out of HBM for itself -- eight fetches of every weight byte per
+// step, which is what bounds small batches of wide rings.  When the column blocks divide by eight, XCD x instead
+// owns column blocks x * cpx .. (x+1) * cpx - 1 for all row groups: each weight byte leaves HBM once per step and is
+// shared through that XCD's L2 by the row groups running side by side.  With fewer than eight column blocks the
+// packed weights are small enough for every XCD's L2, and letting several XCDs share a block was measured to cost a
+// little, so those grids keep the plain order.  Any placement gives correct results; the mapping only decides what
+// the caches see.  xcd_map = 0 keeps the plain order.
+__device__ __forceinline__ void step_block_coords(int xcd_map, int& rg, int& cb) {
+  const int nrg = gridDim.x, ncb = gridDim.y;
+  rg = blockIdx.x;
+  cb = blockIdx.y;
+  if (xcd_map && (ncb & 7) == 0) {
+    const int L = blockIdx.x + nrg * blockIdx.y, xcd = L & 7, w = L >> 3, cpx = ncb >> 3;
+    rg = w % nrg;
+    cb = xcd * cpx + w / nrg;
+  }
+}
+
+// RINGATTR_XCD_MAP=0: plain workgroup order (see step_block_coords)
+inline int step_xcd_map() {
+  const char* v = getenv("RINGATTR_XCD_MAP");
+  return (v && v[0] == '0') ? 0 : 1;
+}
+
 
 __device__ __forceinline__ size_t pair_off_rt(int NC, int t, int nbt, int bt, int tile, int lane) {
   return (((((size_t)(t >> 1) * nbt + bt) * (size_t)(4 * NC) + tile) * 64 + lane) * 2 + (t & 1)) * 4;

@@ -267,8 +267,10 @@ def test_block_kernel_shapes_and_workgroup_orders_agree_bitwise(B, T, k, N, act,
     acts = {"relu": 0, "gelu": 1, "tanh": 2, "silu": 3}
     monkeypatch.setenv("RINGATTR_WIDE", "0")
     outs = []
-    for shape, xcd in (("12", "1"), ("11", "1"), ("21", "1"), ("22", "1"), ("12", "0"), ("21", "0")):
-        monkeypatch.setenv("RINGATTR_BLOCK_SHAPE", shape)
+    # (shape "w": the one-tile-per-workgroup family, compared between its two workgroup orders only)
+    for shape, xcd in (("12", "1"), ("11", "1"), ("21", "1"), ("22", "1"), ("12", "0"), ("21", "0"), ("w", "1"), ("w", "0")):
+        monkeypatch.setenv("RINGATTR_WIDE", "1" if shape == "w" else "0")
+        monkeypatch.setenv("RINGATTR_BLOCK_SHAPE", "12" if shape == "w" else shape)
         monkeypatch.setenv("RINGATTR_XCD_MAP", xcd)
         A, Wa, Wo, r0, G = (_t(p[x], gpu_device) for x in ("A", "Wa", "Wo", "r0", "G"))
         hist = torch.empty(T, B, N, device=gpu_device)
@@ -282,9 +284,11 @@ def test_block_kernel_shapes_and_workgroup_orders_agree_bitwise(B, T, k, N, act,
                               saved=sv, grad_r_init=gr0, grad_A=gA)
         torch.cuda.synchronize()
         outs.append([x.cpu().numpy() for x in (hist, gWa, gWo, gr0, gA)])
-    for other in outs[1:]:
+    for other in outs[1:6]:
         for a, b in zip(outs[0], other):
             assert np.array_equal(a, b)
+    for a, b in zip(outs[6], outs[7]):
+        assert np.array_equal(a, b)
     ref_hist, _ = O.forward_dense(p["A"], p["Wa"], -0.1, 0.3, p["Wo"], p["r0"], 0.15, act)
     assert O.max_rel_err(outs[0][0], ref_hist) <= TRAJ_TOL
 
