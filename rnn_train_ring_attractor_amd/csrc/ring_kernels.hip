@@ -1008,6 +1008,8 @@ static bool step_prefers_wide(int NCv, int nbt, int k) {
 }
 
 hipError_t ring_launch_fwd(const RingFwdArgs& a, int NCv, hipStream_t st) {
+  // the kernels write the derivative record and the operand copy together: both or neither
+  if ((a.dfrag != nullptr) != (a.rfrag != nullptr)) return hipErrorInvalidValue;
   ProfScope prof(1, st);
   if (ring_uses_step_kernels(a.N, a.k, NCv, a.nbt))
     return step_prefers_wide(NCv, a.nbt, a.k) ? ring_launch_wide_fwd(a, NCv, false, 4, st) : ring_launch_block_fwd(a, NCv, false, st);
@@ -1040,6 +1042,7 @@ hipError_t ring_launch_fwd(const RingFwdArgs& a, int NCv, hipStream_t st) {
 // from r_init with its history stores switched off (a.hist is not read): the same kernel, the same
 // numbers the forward would have saved, and no pass over the weights per (batch tile, step).
 hipError_t ring_launch_rebuild(const RingFwdArgs& a, int NCv, hipStream_t st) {
+  if (!a.dfrag || !a.rfrag) return hipErrorInvalidValue;
   ProfScope prof(2, st);
   if (ring_uses_step_kernels(a.N, a.k, NCv, a.nbt))
     return step_prefers_wide(NCv, a.nbt, a.k) ? ring_launch_wide_fwd(a, NCv, true, 4, st) : ring_launch_block_fwd(a, NCv, true, st);
