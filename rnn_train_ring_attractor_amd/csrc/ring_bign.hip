@@ -29,8 +29,29 @@ __device__ __forceinline__ void wide_products(const bf16x8* xb, const bf16x8* __
                                               int NC, int tg0, int lane, f32x4 (&acc)[TPW]) {
   const int KCH = 2 * NC, q = lane >> 4, n = lane & 15;
   const unsigned long long active = staged ? active_channels(gl, k, lane) : ~0ull;
-  for (int mm = 0; mm <= k; ++mm) {
-    if (mm > 0 && staged && !((active >> (mm - 1)) & 1ull)) continue;
+  // next matrix worth multiplying after mm (matrix 1 + c is gated by channel c), or -1
+  auto next_matrix = [&](int mm) {
+    if (!staged) return mm < k ? mm + 1 : -1;
+    const unsigned long long rest = mm >= 64 ? 0ull : (active >> mm);
+    const int nx = rest ? mm + 1 + (int)__builtin_ctzll(rest) : -1;
+    return nx <= k ? nx : -1;
+  };
+  // tile tg0 + cl, chunk kc of matrix mm: fragment ((mm * 4NC + tile) * KCH + kc) * 64 + lane
+  auto matrix_ptr = [&](int mm) { return Wp + ((size_t)mm * 4 * NC + tg0) * KCH * 64 + lane; };
+  // The weights of a step are one stream: the prefetch runs one group of BN_KG chunks ahead and straight across
+  // matrix boundaries, so the pipeline fills once per step, not once per matrix.  (KCH / BN_KG is even, so every
+  // matrix starts in register buffer 0.)
+  bf16x8 wf[2][BN_KG][TPW];
+  {
+    const bf16x8* w0 = matrix_ptr(0);
+#pragma unroll
+    for (int u = 0; u < BN_KG; ++u)
+#pragma unroll
+      for (int cl = 0; cl < TPW; ++cl) wf[0][u][cl] = w0[((size_t)cl * KCH + u) * 64];
+  }
+  const int ngroups = KCH / BN_KG;         // KCH = 2 NC is a multiple of 8
+  for (int mm = 0; mm >= 0;) {
+    const int nxt = next_matrix(mm);
     float coef[4];
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
@@ -41,23 +62,17 @@ __device__ __forceinline__ void wide_products(const bf16x8* xb, const bf16x8* __
     f32x4 p[TPW];
 #pragma unroll
     for (int cl = 0; cl < TPW; ++cl) p[cl] = f32x4{0.f, 0.f, 0.f, 0.f};
-    // tile tg0 + cl, chunk kc: fragment ((mm * 4NC + tile) * KCH + kc) * 64 + lane
-    const bf16x8* wm = Wp + ((size_t)mm * 4 * NC + tg0) * KCH * 64 + lane;
-    bf16x8 wf[2][BN_KG][TPW];
-#pragma unroll
-    for (int u = 0; u < BN_KG; ++u)
-#pragma unroll
-      for (int cl = 0; cl < TPW; ++cl) wf[0][u][cl] = wm[((size_t)cl * KCH + u) * 64];
-    const int ngroups = KCH / BN_KG;       // KCH = 2 NC is a multiple of 8
+    const bf16x8* wm = matrix_ptr(mm);
+    const bf16x8* wn = matrix_ptr(nxt >= 0 ? nxt : mm);   // past the last matrix: a re-read, unused
     for (int g2 = 0; g2 < ngroups; g2 += 2) {
 #pragma unroll
       for (int half = 0; half < 2; ++half) {
         const int g = g2 + half;
-        const int gn = g + 1 < ngroups ? g + 1 : g;     // past the end: a re-read, unused
+        const bf16x8* src = g + 1 < ngroups ? wm + (size_t)(g + 1) * BN_KG * 64 : wn;
 #pragma unroll
         for (int u = 0; u < BN_KG; ++u)
 #pragma unroll
-          for (int cl = 0; cl < TPW; ++cl) wf[half ^ 1][u][cl] = wm[((size_t)cl * KCH + gn * BN_KG + u) * 64];
+          for (int cl = 0; cl < TPW; ++cl) wf[half ^ 1][u][cl] = src[((size_t)cl * KCH + u) * 64];
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int u = 0; u < BN_KG; ++u) {
@@ -72,6 +87,7 @@ __device__ __forceinline__ void wide_products(const bf16x8* xb, const bf16x8* __
     for (int cl = 0; cl < TPW; ++cl)
 #pragma unroll
       for (int e = 0; e < 4; ++e) acc[cl][e] = fmaf(coef[e], p[cl][e], acc[cl][e]);
+    mm = nxt;
   }
 }
 
