@@ -201,6 +201,66 @@ class GeneralizedRingAttractorNoGain(nn.Module):
         return (proj / proj.max(dim=2, keepdim=True)[0]).clone(), bump.clone()
 
 
+class GeneralizedRingAttractor(nn.Module):
+    """The general ring with one learned input gain per action channel (reference:
+    train/train_general_ring_attractor.py:22-153): A[b,t,c] = action[b,t,c] * gain_c(|action[b,t,c]|), each gain a
+    1 -> h -> 1 MLP (GELU hidden, softplus output), then the leaky recurrence over `action_dim` action matrices
+    through the HIP operator, which also returns dL/d action_signal for the gain networks.  Same constructor,
+    parameter names (`gain_nets`, `Wo`, `Wa`) and return values as the reference."""
+
+    def __init__(self, num_neurons, action_dim=2, tau=10.0, dt=1.0, activation="tanh", initialization="random",
+                 hidden_gain_neurons=16):
+        super().__init__()
+        self.num_neurons, self.action_dim, self.tau, self.dt = num_neurons, action_dim, tau, dt
+        self.activation_name, self.initialization = activation, initialization
+        self.gain_nets = nn.ModuleList([
+            nn.Sequential(nn.Linear(1, hidden_gain_neurons), nn.GELU(), nn.Linear(hidden_gain_neurons, 1), nn.Softplus())
+            for _ in range(action_dim)])
+        idx = torch.arange(num_neurons, dtype=torch.float32)
+        diff = 2 * math.pi * (idx[:, None] - idx[None, :]) / num_neurons
+        self.register_buffer("W_delta7", torch.cos(diff))
+        self.J0, self.J1 = -0.1, 0.1
+        scale = 1.0 / math.sqrt(num_neurons)
+        self.Wo = nn.Parameter(torch.randn(num_neurons, num_neurons) * scale)
+        if initialization == "random":
+            self.Wa = nn.Parameter(torch.randn(action_dim, num_neurons, num_neurons) * scale)
+        elif initialization == "perfect":
+            phases = [math.pi / 4, -math.pi / 4] if action_dim == 2 else [c * 2 * math.pi / action_dim for c in range(action_dim)]
+            self.Wa = nn.Parameter(torch.stack([torch.cos(diff + ph) for ph in phases]))
+        else:
+            raise ValueError(f"Unknown initialization: {initialization}")
+
+    def gated_action_signal(self, action_signal):
+        """[B,T,k] action signal -> action * gain(|action|) per channel.  On the GPU all gain networks run as one HIP
+        operator (forward and backward); on the CPU (tests of the module itself) as the torch modules they are."""
+        if action_signal.is_cuda:
+            from .gain import pack_gain_nets, ring_gain_func
+            return ring_gain_func(action_signal, pack_gain_nets(list(self.gain_nets)))
+        gains = [net(action_signal[:, :, c:c + 1].abs()) for c, net in enumerate(self.gain_nets)]
+        return action_signal * torch.cat(gains, dim=2)
+
+    def forward_history(self, action_signal, r_init=None):
+        """bump_history [T,B,N] as the operator returns it (gain networks, then the time loop; no read-out)."""
+        from .ring_rnn_cuda import ring_rnn_cuda_func
+        batch_size, _, action_dim = action_signal.shape
+        assert action_dim == self.action_dim, f"Expected action_dim {self.action_dim}, got {action_dim}"
+        if r_init is None:
+            angle = torch.full((batch_size,), math.pi, device=self.Wo.device)
+            r_init = create_initial_bump(angle, self.num_neurons, device=self.Wo.device)
+        return ring_rnn_cuda_func(action_signal=self.gated_action_signal(action_signal), Wa=self.Wa, J0=self.J0,
+                                  J1=self.J1, Wo=self.Wo, r_init=r_init, alpha=0.15, activation=self.activation_name)
+
+    def forward(self, action_signal, r_init=None):
+        bump = self.forward_history(action_signal, r_init).permute(1, 0, 2)
+        proj = bump @ self.W_delta7
+        return (proj / proj.max(dim=2, keepdim=True)[0]).clone(), bump.clone()
+
+
+def plot_general_ring_matrices(ring_rnn, title_prefix=""):
+    """Plotting is outside the accelerated path; kept as a no-op so driver scripts need no edits."""
+    return None
+
+
 class LeakyRingAttractor(nn.Module):
     """The two-channel model with learned input gains (reference: train/train_ring_attractor.py:55-187):
     L = gain_l(relu(-av)) * relu(-av), R = gain_r(relu(av)) * relu(av), each gain a 1 -> h -> 1 MLP (GELU hidden,

@@ -435,6 +435,47 @@ def test_gain_network_model_trains_through_the_operator(gpu_device):
         assert O.max_rel_err(got, ref) <= 2e-2, n
 
 
+@pytest.mark.parametrize("N,k,B,T", [(256, 4, 48, 24), (640, 6, 24, 10)], ids=["n256_k4", "n640_k6_step"])
+def test_general_ring_with_per_channel_gains(N, k, B, T, gpu_device):
+    """host.GeneralizedRingAttractor (train/train_general_ring_attractor.py:22-153 of the reference): one gain
+    network per action channel in front of the operator.  Loss and every parameter gradient against CPU autograd
+    of the torch port with the same parameters (the port evaluates the gain networks as torch modules)."""
+    from oracle import torch_port as TP
+    from rnn_train_ring_attractor_amd import host
+    print(f"[case] general ring with gains N={N} k={k} B={B} T={T}", flush=True)
+    torch.manual_seed(11)
+    model = host.GeneralizedRingAttractor(N, action_dim=k, activation="tanh", initialization="random")
+    av, angle = host.generate_av_integration_data_ultra_fast(B, T)
+    # (an even channel count: relu(av * linspace(-1, 1, k)) then has no identically zero channel)
+    action = host.av_to_action_signal_ND(av, action_dim=k, zero_padding=False)
+    r0 = host.create_initial_bump(angle[:, 0], N)
+
+    def loss_of(r_hist, bump):
+        return host.cosine_similarity_loss(r_hist, angle.to(r_hist.device)) + 0.2 * host.bump_amplitude_loss(bump)
+
+    A_cpu = model.gated_action_signal(action)
+    bump_cpu = TP.ring_forward(A_cpu, model.Wa, model.J0, model.J1, model.Wo, r0, 0.15, "tanh").permute(1, 0, 2)
+    proj = bump_cpu @ model.W_delta7
+    loss_cpu = loss_of(proj / proj.max(dim=2, keepdim=True)[0], bump_cpu)
+    loss_cpu.backward()
+    want = {n: p.grad.clone() for n, p in model.named_parameters()}
+    model.zero_grad()
+
+    model.to(gpu_device)
+    r_hist, bump = model(action.to(gpu_device), r0.to(gpu_device))
+    assert r_hist.shape == (B, T, N) and bump.shape == (B, T, N)
+    loss = loss_of(r_hist, bump)
+    loss.backward()
+    torch.cuda.synchronize()
+    assert abs(float(loss) - float(loss_cpu)) <= 1e-2 * abs(float(loss_cpu))
+    assert len(want) == 2 + 4 * k
+    for n, p in model.named_parameters():
+        got, ref = p.grad.cpu().numpy(), want[n].numpy()
+        assert np.isfinite(got).all(), n
+        assert O.cosine(got, ref) >= 0.999, n
+        assert O.max_rel_err(got, ref) <= 2e-2, n
+
+
 def _gain_model(N, act, dev, seed=5):
     from rnn_train_ring_attractor_amd import host
     torch.manual_seed(seed)

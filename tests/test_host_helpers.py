@@ -61,3 +61,23 @@ def test_dataset_structure_and_batch_cursor():
         ds.generate_batch(51)
     with pytest.raises(IndexError):
         ds[50]
+
+
+def test_general_ring_gain_networks_follow_the_reference_formula():
+    """GeneralizedRingAttractor.gated_action_signal on the CPU: action * gain_c(|action|) per channel
+    (train/train_general_ring_attractor.py:99-109 of the reference), and the module path the reference uses."""
+    import torch
+    from train.train_general_ring_attractor import GeneralizedRingAttractor
+    torch.manual_seed(3)
+    m = GeneralizedRingAttractor(32, action_dim=3, hidden_gain_neurons=8)
+    assert [n for n, _ in m.named_parameters()][:2] == ["Wo", "Wa"] and len(m.gain_nets) == 3
+    a = torch.randn(5, 7, 3)
+    got = m.gated_action_signal(a)
+    for c in range(3):
+        net = m.gain_nets[c]
+        x = a[:, :, c].abs().reshape(-1, 1)
+        h = torch.nn.functional.gelu(x @ net[0].weight.t() + net[0].bias)
+        gain = torch.nn.functional.softplus(h @ net[2].weight.t() + net[2].bias).reshape(5, 7)
+        assert torch.allclose(got[:, :, c], a[:, :, c] * gain, atol=1e-6)
+    with torch.no_grad():
+        assert GeneralizedRingAttractor(16, action_dim=2, initialization="perfect").Wa.shape == (2, 16, 16)
