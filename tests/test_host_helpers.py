@@ -81,3 +81,20 @@ def test_general_ring_gain_networks_follow_the_reference_formula():
         assert torch.allclose(got[:, :, c], a[:, :, c] * gain, atol=1e-6)
     with torch.no_grad():
         assert GeneralizedRingAttractor(16, action_dim=2, initialization="perfect").Wa.shape == (2, 16, 16)
+
+
+def test_comparison_helper_reports_mismatches(capsys):
+    """utils.benchmark.check_tensor_match (reference utils/benchmark.py:21-56): allclose verdict plus a report."""
+    import torch
+    from utils.benchmark import check_tensor_match, set_seed
+    set_seed(7)
+    a = torch.randn(4, 5)
+    assert check_tensor_match(a.clone(), a, "same") is True
+    b = a.clone()
+    b[1, 2] += 0.5
+    b[3, 4] -= 0.25
+    assert check_tensor_match(b, a, "two off", rtol=1e-5, atol=1e-8) is False
+    out = capsys.readouterr().out
+    assert "same match!" in out and "Total mismatched elements: 2 out of 20 (10.0%)" in out and "[1,2]" in out and "[3,4]" in out
+    set_seed(7)
+    assert torch.equal(torch.randn(4, 5), a)
