@@ -618,6 +618,21 @@ def test_training_driver_reduces_loss(gpu_device):
     assert np.mean(hist_opt[-5:]) < np.mean(hist_opt[:5])
 
 
+def test_training_and_evaluation_entry_point(gpu_device):
+    """run_training_and_evaluation, the reference script's entry point (train_general_ring_no_gain.py:261-376 there):
+    training followed by the single-trial evaluation with both decoders, on the padded 16-channel action signal."""
+    import train_general_ring_no_gain as drv
+    print("[case] training + evaluation entry point N=128 k=16", flush=True)
+    model, hist, res = drv.run_training_and_evaluation(action_dim=16, training_steps=30, num_neurons=128, batch_size=32,
+                                                       seq_len=40, lr=3e-3, log_every=0, seed=2)
+    assert len(hist) == 30 and all(np.isfinite(hist))
+    assert res["cos_activity"].shape == (1, 40, 128) and res["bump_activity"].shape == (1, 40, 128)
+    assert res["decoded_pv"].shape == (1, 40) and res["decoded_argmax"].shape == (1, 40)
+    assert 0.0 <= res["mean_abs_error_pv"] <= np.pi and 0.0 <= res["mean_abs_error_argmax"] <= np.pi
+    # the aligned target starts where the model's default bump sits
+    assert abs(float(res["aligned_target"][0, 0]) - np.pi) <= 1e-5
+
+
 def test_reference_signature_entry_points(gpu_device):
     """fwd_cuda / bwd_cuda with the reference's exact C argument lists (null stream, own scratch)."""
     import ctypes
