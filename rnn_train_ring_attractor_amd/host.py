@@ -107,19 +107,24 @@ def generate_av_integration_data_ultra_fast(num_trials, seq_len, zero_padding_st
     return av, angle
 
 
+def generate_av_integration_data_chunked(num_trials, seq_len, zero_padding_start_ratio=0.1, zero_ratios_in_rest=None,
+                                         max_av=0.1 * math.pi, device="cpu", chunk_size=10000):
+    """The same trials generated `chunk_size` at a time and concatenated (bounded temporaries for large sets;
+    reference: utils/generate_av_integration_data.py:61-108)."""
+    parts = [generate_av_integration_data_ultra_fast(min(chunk_size, num_trials - start), seq_len, zero_padding_start_ratio,
+                                                     zero_ratios_in_rest, max_av, device)
+             for start in range(0, num_trials, chunk_size)]
+    return torch.cat([a for a, _ in parts]), torch.cat([g for _, g in parts])
+
+
 class AVIntegrationDataset(torch.utils.data.Dataset):
     """Pre-generated AV trials with a shuffled batch cursor (generate_batch wraps and reshuffles)."""
 
     def __init__(self, num_samples, seq_len, zero_padding_start_ratio=0.1, zero_ratios_in_rest=None,
                  max_av=0.1 * math.pi, device="cpu", fast_mode=True, chunk_size=10000):
         self.num_samples, self.seq_len, self.device = num_samples, seq_len, torch.device(device)
-        av, ang = [], []
-        for start in range(0, num_samples, chunk_size):
-            a, g = generate_av_integration_data_ultra_fast(min(chunk_size, num_samples - start), seq_len,
-                                                           zero_padding_start_ratio, zero_ratios_in_rest, max_av, device)
-            av.append(a)
-            ang.append(g)
-        self.av_data, self.angle_data = torch.cat(av), torch.cat(ang)
+        self.av_data, self.angle_data = generate_av_integration_data_chunked(
+            num_samples, seq_len, zero_padding_start_ratio, zero_ratios_in_rest, max_av, device, chunk_size)
         self.current_index = 0
         self.shuffled_indices = torch.randperm(num_samples, device=device)
 

@@ -98,3 +98,18 @@ def test_comparison_helper_reports_mismatches(capsys):
     assert "same match!" in out and "Total mismatched elements: 2 out of 20 (10.0%)" in out and "[1,2]" in out and "[3,4]" in out
     set_seed(7)
     assert torch.equal(torch.randn(4, 5), a)
+
+
+def test_chunked_generator_concatenates_trials():
+    """utils.generate_av_integration_data.generate_av_integration_data_chunked: chunking changes nothing but the
+    temporaries -- shapes, the leading zero block and angle = cumulative sum of av hold across chunk borders."""
+    import torch
+    from utils.generate_av_integration_data import generate_av_integration_data_chunked
+    torch.manual_seed(0)
+    av, ang = generate_av_integration_data_chunked(25, 40, zero_padding_start_ratio=0.1, zero_ratios_in_rest=[0.5],
+                                                   chunk_size=10)
+    assert av.shape == (25, 40) and ang.shape == (25, 40)
+    assert torch.all(av[:, :4] == 0)
+    assert float(av.abs().max()) <= 0.1 * 3.141593
+    step = torch.remainder(ang[:, 1:] - ang[:, :-1] - av[:, :-1] + 3.141592653589793, 2 * 3.141592653589793) - 3.141592653589793
+    assert float(step.abs().max()) <= 1e-4
