@@ -46,10 +46,12 @@ WORKLOADS = {
     "train_n256_b128_t100_k16pad_gelu": dict(N=256, B=128, T=100, k=16, act="gelu", J0=-0.1, J1=0.1, mode="train",
                                              driven=(0, 1)),
 }
-# the shapes of the reference's published latency table (assets/REPORT.md:5-10): forward, B=256, T=20, 16 dense channels
-for _n in (128, 256, 384, 512, 1024, 2048):
-    WORKLOADS[f"report_fwd_n{_n}_b256_t20_k16"] = dict(N=_n, B=256, T=20, k=16, act="silu", J0=-0.1, J1=0.1, mode="infer",
-                                                      action="dense")
+# the shapes of the reference's published latency table (assets/REPORT.md:5-10): forward, B=256, T=20, 16 dense channels,
+# plus its rows with more channels (:11-12) and the widths it could only run on its fp32 kernel (:13-16, k % 16 != 0)
+for _n, _k in [(n, 16) for n in (128, 256, 384, 512, 1024, 2048)] + [(2048, 32), (2048, 64)] + \
+        [(1024, k) for k in (2, 3, 6, 12)]:
+    WORKLOADS[f"report_fwd_n{_n}_b256_t20_k{_k}"] = dict(N=_n, B=256, T=20, k=_k, act="silu", J0=-0.1, J1=0.1,
+                                                        mode="infer", action="dense")
 
 
 def make_inputs(cfg, device):

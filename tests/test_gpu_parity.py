@@ -68,6 +68,9 @@ CASES = [
     ("n2048_k3_tanh",  20,   4,  3, 2048, "tanh", -0.01, 0.1, "dense"),
     ("n700_k16_pad",   32,   5, 16, 700, "silu", -0.05, 0.2, "lr"),       # ragged width, zero-padded channels
     ("n1500_relu",     17,   3,  2, 1500, "relu", -1 / 1500, 1.0, "dense"),
+    # the reference's published many-channel rows (assets/REPORT.md:11-12: 32 and 64 channels)
+    ("n2048_k32_dense", 16,  2, 32, 2048, "silu", -0.01, 0.1, "dense"),
+    ("n1024_k64_dense", 16,  3, 64, 1024, "tanh", -0.01, 0.1, "dense"),
 ]
 
 
