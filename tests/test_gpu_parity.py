@@ -209,9 +209,12 @@ def test_backward_without_saved_buffer_rebuilds_it(case, gpu_device):
                                                 (21, 9, 3, 200, "silu", "dense"), (32, 12, 16, 64, "tanh", "spread"),
                                                 (32, 7, 2, 256, "tanh", "dense"), (37, 10, 2, 200, "silu", "dense"),
                                                 (64, 66, 2, 256, "relu", "lr"), (24, 6, 3, 700, "silu", "dense"),
-                                                (20, 5, 2, 1024, "tanh", "lr"), (18, 4, 4, 1300, "gelu", "spread")],
+                                                (20, 5, 2, 1024, "tanh", "lr"), (18, 4, 4, 1300, "gelu", "spread"),
+                                                (1, 3, 2, 256, "gelu", "dense"), (1, 2, 2, 2048, "tanh", "dense"),
+                                                (1, 1, 2, 40, "tanh", "dense")],
                          ids=["n120", "n256", "ragged_k3", "k16", "n256_odd_T", "n200_ragged_resident", "n256_relu_T66",
-                              "n700_k3_step", "n1024_step", "n1300_k4_step"])
+                              "n700_k3_step", "n1024_step", "n1300_k4_step",
+                              "one_sample_resident", "one_sample_n2048_step", "one_sample_one_step"])
 def test_gradients_of_action_signal_and_initial_state(B, T, k, N, act, action, gpu_device):
     """dL/d action_signal and dL/d r_init, which the reference operator does not return (cpp/ring_rnn_cuda.py:144);
     pinned by the fp64 oracle, whose grad_A / grad_r_init are themselves checked by finite differences."""
