@@ -183,11 +183,19 @@ RINGATTR_API int ringattr_generate_inputs(unsigned long long seed, int N, int a_
  * The gradient norm is summed in a fixed order (repeatable).  params / grads / exp_avg / exp_avg_sq are HOST arrays of
  * n_tensors device pointers, numel a host array; grads are scaled in place by min(1, max_norm / (norm + 1e-6))
  * (max_norm <= 0: no clipping), then m, v and the parameters are updated in place; `step` counts from 1.
- * The workspace's last float receives the gradient norm before clipping. */
+ * The gradient norm before clipping is left in the workspace as float number sum_i ceil(numel[i] / 4096) (behind the
+ * per-chunk partial sums). */
 RINGATTR_API size_t ringattr_clip_adam_workspace_bytes(int n_tensors, const size_t* numel);
 RINGATTR_API int ringattr_clip_adam(int n_tensors, void* const* params, void* const* grads, void* const* exp_avg,
                       void* const* exp_avg_sq, const size_t* numel, float lr, float beta1, float beta2, float eps,
                       float max_norm, int step, void* workspace, size_t workspace_bytes, void* stream);
+/* The same step with Adam's step number kept on the device: step_counter is a device int32 (zero before the first
+ * step) that the call advances by one and derives the bias corrections from, so a training step recorded into a HIP
+ * graph keeps counting on every replay (torch.optim.Adam(capturable=True) keeps its step on the device likewise;
+ * the reference's eager loop, root train_general_ring_no_gain.py:333-336, has no counterpart). */
+RINGATTR_API int ringattr_clip_adam_counted(int n_tensors, void* const* params, void* const* grads, void* const* exp_avg,
+                      void* const* exp_avg_sq, const size_t* numel, float lr, float beta1, float beta2, float eps,
+                      float max_norm, void* step_counter, void* workspace, size_t workspace_bytes, void* stream);
 
 /* Per-kernel timing for benchmarks; no counterpart in the reference.  While enabled, every kernel
  * launch is bracketed by two HIP events recorded on the launch stream.  ringattr_profile_read waits

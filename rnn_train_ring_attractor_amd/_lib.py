@@ -54,6 +54,10 @@ PROTOTYPES = {
     "ringattr_clip_adam": (c_int, [c_int, ctypes.POINTER(c_void_p), ctypes.POINTER(c_void_p), ctypes.POINTER(c_void_p),
                                    ctypes.POINTER(c_void_p), ctypes.POINTER(c_size_t), c_float, c_float, c_float,
                                    c_float, c_float, c_int, c_void_p, c_size_t, c_void_p]),
+    "ringattr_clip_adam_counted": (c_int, [c_int, ctypes.POINTER(c_void_p), ctypes.POINTER(c_void_p),
+                                           ctypes.POINTER(c_void_p), ctypes.POINTER(c_void_p), ctypes.POINTER(c_size_t),
+                                           c_float, c_float, c_float, c_float, c_float, c_void_p, c_void_p, c_size_t,
+                                           c_void_p]),
     "ringattr_profile_enable": (c_int, [c_int]),
     "ringattr_profile_read": (c_int, [ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_longlong)]),
     "fwd_cuda": (None, [c_void_p, c_void_p, c_float, c_float, c_void_p, c_void_p, c_void_p, c_float,

@@ -150,8 +150,11 @@ __global__ __launch_bounds__(OPT_BLOCK) void ring_gradnorm_partial_kernel(RingOp
   if (threadIdx.x == 0) partial[blockIdx.x] = (red[0] + red[1]) + (red[2] + red[3]);
 }
 
-// norm_out[0] = sqrt(sum of the partials, in order): one workgroup, fixed tree
-__global__ __launch_bounds__(OPT_BLOCK) void ring_gradnorm_final_kernel(const float* partial, int nblk, float* norm_out) {
+// norm_out[0] = sqrt(sum of the partials, in order): one workgroup, fixed tree.  With a device step counter the same
+// thread advances it and leaves Adam's two bias-correction factors of the new step in norm_out[1], norm_out[2].
+__global__ __launch_bounds__(OPT_BLOCK) void ring_gradnorm_final_kernel(const float* partial, int nblk, float* norm_out,
+                                                                        int* step_counter, float lr, float beta1,
+                                                                        float beta2) {
   __shared__ float red[OPT_BLOCK];
   float s = 0.f;
   for (int i = threadIdx.x; i < nblk; i += OPT_BLOCK) s += partial[i];
@@ -161,7 +164,15 @@ __global__ __launch_bounds__(OPT_BLOCK) void ring_gradnorm_final_kernel(const fl
     if ((int)threadIdx.x < w) red[threadIdx.x] += red[threadIdx.x + w];
     __syncthreads();
   }
-  if (threadIdx.x == 0) norm_out[0] = sqrtf(red[0]);
+  if (threadIdx.x == 0) {
+    norm_out[0] = sqrtf(red[0]);
+    if (step_counter) {
+      const int t = step_counter[0] + 1;
+      step_counter[0] = t;
+      norm_out[1] = (float)((double)lr / (1.0 - pow((double)beta1, (double)t)));
+      norm_out[2] = (float)(1.0 / sqrt(1.0 - pow((double)beta2, (double)t)));
+    }
+  }
 }
 
 // g <- g * min(1, max_norm / (norm + 1e-6)) (written back, as clip_grad_norm_ does); then torch.optim.Adam's update:
@@ -177,6 +188,8 @@ __global__ __launch_bounds__(OPT_BLOCK) void ring_clip_adam_kernel(RingOptArgs p
   float* m = p.exp_avg[ti];
   float* v = p.exp_avg_sq[ti];
   const size_t lo = (size_t)blk * OPT_CHUNK, hi = lo + OPT_CHUNK < p.numel[ti] ? lo + OPT_CHUNK : p.numel[ti];
+  const float step_size = p.step_counter ? norm[1] : p.step_size;
+  const float inv_sqrt_bc2 = p.step_counter ? norm[2] : p.inv_sqrt_bc2;
   for (size_t i = lo + threadIdx.x; i < hi; i += OPT_BLOCK) {
     const float gi = g[i] * clip;
     const float mi = p.beta1 * m[i] + (1.f - p.beta1) * gi;
@@ -184,13 +197,14 @@ __global__ __launch_bounds__(OPT_BLOCK) void ring_clip_adam_kernel(RingOptArgs p
     g[i] = gi;
     m[i] = mi;
     v[i] = vi;
-    w[i] -= p.step_size * (mi / (sqrtf(vi) * p.inv_sqrt_bc2 + p.eps));
+    w[i] -= step_size * (mi / (sqrtf(vi) * inv_sqrt_bc2 + p.eps));
   }
 }
 
 int ring_opt_chunks(size_t numel) { return (int)((numel + OPT_CHUNK - 1) / OPT_CHUNK); }
 
-// workspace: (total chunks + 1) floats; the last one receives the gradient norm (before clipping)
+// workspace: (total chunks + 3) floats; behind the partial sums: the gradient norm (before clipping) and, with a device
+// step counter, the step's two bias-correction factors
 hipError_t ring_launch_clip_adam(const RingOptArgs& a, float* workspace, hipStream_t st) {
   int total = 0;
   for (int i = 0; i < a.n; ++i) total += a.chunks[i];
@@ -199,7 +213,8 @@ hipError_t ring_launch_clip_adam(const RingOptArgs& a, float* workspace, hipStre
   hipLaunchKernelGGL(ring_gradnorm_partial_kernel, dim3(total), dim3(OPT_BLOCK), 0, st, a, workspace);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return e;
-  hipLaunchKernelGGL(ring_gradnorm_final_kernel, dim3(1), dim3(OPT_BLOCK), 0, st, workspace, total, norm);
+  hipLaunchKernelGGL(ring_gradnorm_final_kernel, dim3(1), dim3(OPT_BLOCK), 0, st, workspace, total, norm, a.step_counter,
+                     a.lr, a.beta1, a.beta2);
   e = hipGetLastError();
   if (e != hipSuccess) return e;
   hipLaunchKernelGGL(ring_clip_adam_kernel, dim3(total), dim3(OPT_BLOCK), 0, st, a, norm);

@@ -132,6 +132,8 @@ struct RingOptArgs {
   float beta1, beta2, eps, max_norm;
   float step_size;       // lr / (1 - beta1^t)
   float inv_sqrt_bc2;    // 1 / sqrt(1 - beta2^t)
+  int* step_counter;     // non-null: t lives on the device; the call advances it and derives the two factors itself
+  float lr;              // (used with step_counter)
 };
 int ring_opt_chunks(size_t numel);
 hipError_t ring_launch_clip_adam(const RingOptArgs& a, float* workspace, hipStream_t st);

@@ -552,16 +552,40 @@ size_t ringattr_clip_adam_workspace_bytes(int n_tensors, const size_t* numel) {
   }
   size_t chunks = 0;
   for (int i = 0; i < n_tensors; ++i) chunks += (size_t)ring_opt_chunks(numel[i]);
-  return align_up((chunks + 1) * sizeof(float));
+  return align_up((chunks + 3) * sizeof(float));
 }
+
+// step_counter != null: the step number lives on the device (ringattr_clip_adam_counted); otherwise `step` is it.
+static int clip_adam_impl(int n_tensors, void* const* params, void* const* grads, void* const* exp_avg,
+                          void* const* exp_avg_sq, const size_t* numel, float lr, float beta1, float beta2, float eps,
+                          float max_norm, int step, void* step_counter, void* workspace, size_t workspace_bytes,
+                          void* stream);
 
 int ringattr_clip_adam(int n_tensors, void* const* params, void* const* grads, void* const* exp_avg,
                        void* const* exp_avg_sq, const size_t* numel, float lr, float beta1, float beta2, float eps,
                        float max_norm, int step, void* workspace, size_t workspace_bytes, void* stream) {
+  if (step < 1) return fail(RINGATTR_ERR_INVALID, "ringattr_clip_adam: step counts from 1 (got %d)", step);
+  return clip_adam_impl(n_tensors, params, grads, exp_avg, exp_avg_sq, numel, lr, beta1, beta2, eps, max_norm, step,
+                        nullptr, workspace, workspace_bytes, stream);
+}
+
+int ringattr_clip_adam_counted(int n_tensors, void* const* params, void* const* grads, void* const* exp_avg,
+                               void* const* exp_avg_sq, const size_t* numel, float lr, float beta1, float beta2,
+                               float eps, float max_norm, void* step_counter, void* workspace, size_t workspace_bytes,
+                               void* stream) {
+  if (!step_counter || (reinterpret_cast<uintptr_t>(step_counter) & 3))
+    return fail(RINGATTR_ERR_INVALID, "ringattr_clip_adam_counted: the step counter must be a 4-byte aligned device pointer");
+  return clip_adam_impl(n_tensors, params, grads, exp_avg, exp_avg_sq, numel, lr, beta1, beta2, eps, max_norm, 1,
+                        step_counter, workspace, workspace_bytes, stream);
+}
+
+static int clip_adam_impl(int n_tensors, void* const* params, void* const* grads, void* const* exp_avg,
+                          void* const* exp_avg_sq, const size_t* numel, float lr, float beta1, float beta2, float eps,
+                          float max_norm, int step, void* step_counter, void* workspace, size_t workspace_bytes,
+                          void* stream) {
   const size_t need = ringattr_clip_adam_workspace_bytes(n_tensors, numel);
   if (need == 0) return RINGATTR_ERR_INVALID;
   if (!params || !grads || !exp_avg || !exp_avg_sq) return fail(RINGATTR_ERR_INVALID, "ringattr_clip_adam: null pointer list");
-  if (step < 1) return fail(RINGATTR_ERR_INVALID, "ringattr_clip_adam: step counts from 1 (got %d)", step);
   if (!workspace || workspace_bytes < need)
     return fail(RINGATTR_ERR_WORKSPACE, "ringattr_clip_adam: workspace of %zu bytes needed, %zu given", need,
                 workspace ? workspace_bytes : (size_t)0);
@@ -584,6 +608,8 @@ int ringattr_clip_adam(int n_tensors, void* const* params, void* const* grads, v
   a.max_norm = max_norm;
   a.step_size = (float)((double)lr / (1.0 - pow((double)beta1, (double)step)));
   a.inv_sqrt_bc2 = (float)(1.0 / sqrt(1.0 - pow((double)beta2, (double)step)));
+  a.step_counter = (int*)step_counter;
+  a.lr = lr;
   hipError_t e = ring_launch_clip_adam(a, (float*)workspace, static_cast<hipStream_t>(stream));
   if (e != hipSuccess) return hip_fail(e, "clip + Adam launch");
   return RINGATTR_OK;

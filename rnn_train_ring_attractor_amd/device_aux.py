@@ -49,9 +49,12 @@ class FusedClipAdam:
 
     Same update as torch.optim.Adam (no weight decay, no amsgrad) after torch.nn.utils.clip_grad_norm_; state
     (exp_avg, exp_avg_sq, step) is kept per tensor as torch does.  `last_grad_norm` is a device scalar (the norm
-    before clipping) that is only valid after the step has run on the stream; reading it synchronises."""
+    before clipping) that is only valid after the step has run on the stream; reading it synchronises.
+    capturable=True keeps Adam's step number in a device counter that every step advances itself, so a training step
+    recorded into a HIP graph goes on counting when the graph is replayed (the host-side `step_count` still counts
+    the calls made from Python, not the replays)."""
 
-    def __init__(self, params, lr=1e-3, betas=(0.9, 0.999), eps=1e-8, max_norm=1.0):
+    def __init__(self, params, lr=1e-3, betas=(0.9, 0.999), eps=1e-8, max_norm=1.0, capturable=False):
         self.params = [p for p in params if p.requires_grad]
         if not 1 <= len(self.params) <= 16:
             raise ValueError(f"FusedClipAdam handles 1..16 parameter tensors, got {len(self.params)}")
@@ -62,6 +65,7 @@ class FusedClipAdam:
         self.exp_avg = [torch.zeros_like(p) for p in self.params]
         self.exp_avg_sq = [torch.zeros_like(p) for p in self.params]
         self.step_count = 0
+        self.step_counter = torch.zeros(1, dtype=torch.int32, device=self.params[0].device) if capturable else None
         n = len(self.params)
         self._numel = (ctypes.c_size_t * n)(*[p.numel() for p in self.params])
         lib = _lib.load()
@@ -93,7 +97,11 @@ class FusedClipAdam:
         ptrs = lambda ts: (ctypes.c_void_p * n)(*[t.data_ptr() for t in ts])
         dev = self.params[0].device
         with torch.cuda.device(dev), torch.no_grad():
-            _lib.check(_lib.load().ringattr_clip_adam(
-                n, ptrs(self.params), ptrs(grads), ptrs(self.exp_avg), ptrs(self.exp_avg_sq), self._numel, self.lr,
-                self.betas[0], self.betas[1], self.eps, self.max_norm, self.step_count, self._ws.data_ptr(),
-                self._ws_bytes, torch.cuda.current_stream(dev).cuda_stream))
+            lib, stream = _lib.load(), torch.cuda.current_stream(dev).cuda_stream
+            common = (n, ptrs(self.params), ptrs(grads), ptrs(self.exp_avg), ptrs(self.exp_avg_sq), self._numel, self.lr,
+                      self.betas[0], self.betas[1], self.eps, self.max_norm)
+            if self.step_counter is not None:
+                _lib.check(lib.ringattr_clip_adam_counted(*common, self.step_counter.data_ptr(), self._ws.data_ptr(),
+                                                          self._ws_bytes, stream))
+            else:
+                _lib.check(lib.ringattr_clip_adam(*common, self.step_count, self._ws.data_ptr(), self._ws_bytes, stream))

@@ -1,0 +1,111 @@
+"""The operator under HIP graph capture: forward + backward recorded once, replayed on new inputs.
+
+Nothing on the operator path allocates through HIP, synchronises or reads the device back, so a caller may record a
+training step into a graph.  Every replay is checked against an eager run on the same inputs (the kernels sum in a
+fixed order, so the comparison is bitwise), with eager work and synchronisations between the replays."""
+import numpy as np
+import pytest
+import torch
+
+from tests.ring_cases import make_problem
+
+pytestmark = pytest.mark.gpu
+
+CASES = [
+    # name,        B,  T, k,   N, act
+    ("resident",  48, 10, 2, 256, "gelu"),
+    ("streaming", 40, 12, 2, 120, "tanh"),
+    ("step",      24,  5, 3, 640, "silu"),
+]
+
+
+@pytest.mark.parametrize("case", CASES, ids=[c[0] for c in CASES])
+def test_forward_backward_replays_from_a_graph(case, gpu_device):
+    from rnn_train_ring_attractor_amd import ring_rnn_cuda_func
+    name, B, T, k, N, act = case
+    print(f"[case] graph {name} B={B} T={T} k={k} N={N} {act}", flush=True)
+    J0, J1 = -0.05, 0.4
+    problems = [make_problem(900 + i, B, T, k, N, action="dense") for i in range(3)]
+
+    def dev(x):
+        return torch.tensor(x, device=gpu_device)
+
+    p0 = problems[0]
+    A, r0, G = dev(p0["A"]), dev(p0["r0"]), dev(p0["G"])
+    Wa, Wo = dev(p0["Wa"]).requires_grad_(True), dev(p0["Wo"]).requires_grad_(True)
+
+    def step(A, Wa, Wo, r0, G):
+        hist = ring_rnn_cuda_func(A, Wa, J0, J1, Wo, r0, 0.15, act)
+        hist.backward(G)
+        return hist
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(2):                       # the allocator and lazily initialised state settle outside the capture
+            Wa.grad = Wo.grad = None
+            step(A, Wa, Wo, r0, G)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    Wa.grad = Wo.grad = None
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        hist = step(A, Wa, Wo, r0, G)
+
+    for rep, p in enumerate(problems[::-1] + problems[:1]):
+        with torch.no_grad():
+            for dst, key in ((A, "A"), (r0, "r0"), (G, "G"), (Wa, "Wa"), (Wo, "Wo")):
+                dst.copy_(dev(p[key]))
+        graph.replay()
+        torch.cuda.synchronize()
+        got = (hist.detach().clone(), Wa.grad.clone(), Wo.grad.clone())
+        # the same inputs through the eager path (its own tensors), with a synchronisation before the next replay
+        eWa, eWo = dev(p["Wa"]).requires_grad_(True), dev(p["Wo"]).requires_grad_(True)
+        ehist = step(dev(p["A"]), eWa, eWo, dev(p["r0"]), dev(p["G"]))
+        torch.cuda.synchronize()
+        assert np.isfinite(got[0].cpu().numpy()).all()
+        assert torch.equal(got[0], ehist.detach()), f"replay {rep}: history differs from the eager run"
+        assert torch.equal(got[1], eWa.grad), f"replay {rep}: grad_Wa differs from the eager run"
+        assert torch.equal(got[2], eWo.grad), f"replay {rep}: grad_Wo differs from the eager run"
+        assert float(got[1].abs().max()) > 0
+
+
+def test_device_counted_optimizer_matches_the_host_counted_one(gpu_device):
+    """FusedClipAdam(capturable=True) keeps Adam's step number on the device; five steps agree with the variant that
+    receives the number from the host, and the counter has advanced once per step."""
+    from rnn_train_ring_attractor_amd import FusedClipAdam
+    print("[case] counted clip + Adam", flush=True)
+    torch.manual_seed(5)
+    shapes = [(256, 256), (2, 256, 256), (16,), (5000,)]
+    init = [torch.randn(s, device=gpu_device) for s in shapes]
+    host = [x.clone().requires_grad_(True) for x in init]
+    counted = [x.clone().requires_grad_(True) for x in init]
+    opt_h = FusedClipAdam(host, lr=3e-3, betas=(0.9, 0.99), max_norm=1.0)
+    opt_c = FusedClipAdam(counted, lr=3e-3, betas=(0.9, 0.99), max_norm=1.0, capturable=True)
+    for step in range(5):
+        grads = [torch.randn(s, device=gpu_device) * (3.0 if step % 2 == 0 else 0.01) for s in shapes]
+        for p, q, g in zip(host, counted, grads):
+            p.grad, q.grad = g.clone(), g.clone()
+        opt_h.step()
+        opt_c.step()
+        torch.cuda.synchronize()
+        for p, q in zip(host, counted):
+            torch.testing.assert_close(q.detach(), p.detach(), rtol=1e-6, atol=1e-8)
+    assert int(opt_c.step_counter) == 5
+
+
+def test_training_driver_replays_its_step_from_a_graph(gpu_device):
+    """The driver's graph mode (three eager steps, then one recorded step replayed) follows the eager run with the
+    same seed step for step: zero-padded action channels (the compaction and its device-side check are inside the
+    recording), fused loss head, backward, device-counted clip + Adam."""
+    import train_general_ring_no_gain as drv
+    print("[case] training driver under a HIP graph N=256 B=32 T=30 k=16", flush=True)
+    kw = dict(action_dim=16, num_neurons=256, training_steps=14, batch_size=32, seq_len=30, lr=3e-3, activation="gelu",
+              log_every=0, seed=2, fused_loss=True, fused_optimizer=True)
+    _, eager = drv.run_training(**kw)
+    _, replayed = drv.run_training(hip_graph=True, **kw)
+    assert len(replayed) == 14 and all(np.isfinite(replayed))
+    np.testing.assert_allclose(replayed, eager, rtol=1e-5, atol=1e-7)
+    assert np.mean(replayed[-4:]) < np.mean(replayed[:4])
+    with pytest.raises(ValueError):
+        drv.run_training(hip_graph=True, **dict(kw, fused_loss=False))

@@ -14,20 +14,27 @@ from rnn_train_ring_attractor_amd.host import (  # noqa: F401
 
 
 def run_training(action_dim=2, num_neurons=256, training_steps=1000, batch_size=128, seq_len=100, lr=1e-3,
-                 activation="gelu", log_every=10, seed=0, fused_loss=False, fused_optimizer=False):
+                 activation="gelu", log_every=10, seed=0, fused_loss=False, fused_optimizer=False, hip_graph=False):
+    """hip_graph=True records one training step (action signal, initial bump, time loop, loss head, backward, clipping
+    and Adam) into a HIP graph after three eager steps and replays it for the rest of the run: one graph launch per
+    step instead of some thirty kernel launches and the Python between them.  It needs both fused options (their
+    kernels neither allocate through HIP nor read the device back, and the fused optimizer counts its steps on the
+    device); the loss values stay on the device and are read only where they are printed and at the end."""
     torch.manual_seed(seed)
     device = torch.device("cuda")
+    if hip_graph and not (fused_loss and fused_optimizer):
+        raise ValueError("hip_graph=True records the fused loss head and the fused optimizer step: "
+                         "pass fused_loss=True and fused_optimizer=True")
     data = AVIntegrationDataset(num_samples=min(training_steps * batch_size, 200_000), seq_len=seq_len,
                                 zero_padding_start_ratio=0.1, zero_ratios_in_rest=[0.2, 0.5, 0.8], device="cuda")
     model = GeneralizedRingAttractorNoGain(num_neurons, action_dim=action_dim, activation=activation).to(device)
     if fused_optimizer:       # clip_grad_norm_ + Adam.step() as three kernel launches
         from rnn_train_ring_attractor_amd import FusedClipAdam
-        opt = FusedClipAdam(model.parameters(), lr=lr, max_norm=1.0)
+        opt = FusedClipAdam(model.parameters(), lr=lr, max_norm=1.0, capturable=hip_graph)
     else:
         opt = torch.optim.Adam(model.parameters(), lr=lr)
-    history = []
-    for step in range(training_steps):
-        av, target = data.generate_batch(batch_size)
+
+    def train_step(av, target):
         action = av_to_action_signal_ND(av, action_dim)
         r_init = create_initial_bump(target[:, 0], num_neurons, device=device)
         if fused_loss:
@@ -41,10 +48,51 @@ def run_training(action_dim=2, num_neurons=256, training_steps=1000, batch_size=
         if not fused_optimizer:
             torch.nn.utils.clip_grad_norm_(model.parameters(), 1.0)
         opt.step()
-        history.append(float(total))
+        return total.detach(), loss.detach()
+
+    def report(step, total, loss):
         if log_every and step % log_every == 0:
-            print(f"Step {step}/{training_steps}, Total Loss: {history[-1]:.4f}, Main loss: {float(loss):.4f}")
-    return model, history
+            print(f"Step {step}/{training_steps}, Total Loss: {float(total):.4f}, Main loss: {float(loss):.4f}")
+
+    if not hip_graph:
+        history = []
+        for step in range(training_steps):
+            total, loss = train_step(*data.generate_batch(batch_size))
+            history.append(float(total))
+            report(step, total, loss)
+        return model, history
+
+    # Graph mode: the batch lands in two static tensors, everything behind them is recorded once.
+    static_av = torch.empty(batch_size, seq_len, device=device)
+    static_target = torch.empty(batch_size, seq_len, device=device)
+    totals = torch.zeros(training_steps, device=device)
+
+    def load_batch():
+        av, target = data.generate_batch(batch_size)
+        static_av.copy_(av)
+        static_target.copy_(target)
+
+    eager_steps = min(3, training_steps)          # real training steps; they also settle the allocator
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for step in range(eager_steps):
+            load_batch()
+            total, loss = train_step(static_av, static_target)
+            totals[step] = total
+            report(step, total, loss)
+    torch.cuda.current_stream().wait_stream(side)
+    if eager_steps < training_steps:
+        opt.zero_grad()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            g_total, g_loss = train_step(static_av, static_target)
+        for step in range(eager_steps, training_steps):
+            load_batch()
+            graph.replay()
+            totals[step] = g_total
+            report(step, g_total, g_loss)
+    return model, totals.tolist()
 
 
 def evaluate(model, action_dim, seq_len=100, seed=1):
@@ -87,6 +135,8 @@ if __name__ == "__main__":
     ap.add_argument("--steps", type=int, default=1000)
     ap.add_argument("--fused_loss", action="store_true", help="loss pair and its gradient by the fused HIP loss head")
     ap.add_argument("--fused_optimizer", action="store_true", help="gradient clipping + Adam as one fused HIP step")
+    ap.add_argument("--hip_graph", action="store_true",
+                    help="record the training step into a HIP graph and replay it (implies both fused options)")
     a = ap.parse_args()
-    run_training_and_evaluation(action_dim=a.action_dim, training_steps=a.steps, fused_loss=a.fused_loss,
-                                fused_optimizer=a.fused_optimizer)
+    run_training_and_evaluation(action_dim=a.action_dim, training_steps=a.steps, fused_loss=a.fused_loss or a.hip_graph,
+                                fused_optimizer=a.fused_optimizer or a.hip_graph, hip_graph=a.hip_graph)
