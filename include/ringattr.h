@@ -117,7 +117,7 @@ RINGATTR_API int ringattr_bwd(const void* grad_output, const void* A, const void
  *   loss_out          3 floats on the device: total, cos-sim loss, amplitude loss
  *   upstream          one float on the device (d objective / d total) or NULL for 1
  *   grad_history      [T,B,N], overwritten with d total / d bump_history * upstream
- * ringattr_loss_bwd needs the workspace ringattr_loss_fwd filled for the same inputs.  N <= 1024. */
+ * ringattr_loss_bwd needs the workspace ringattr_loss_fwd filled for the same inputs.  N <= 2048. */
 RINGATTR_API size_t ringattr_loss_workspace_bytes(int N, int seq_len, int batch_size);
 RINGATTR_API int ringattr_loss_fwd(const void* bump_history, const void* target_angle, const void* target_amplitude,
                       float bump_weight, void* loss_out, int N, int seq_len, int batch_size,

@@ -21,7 +21,7 @@
 namespace {
 
 constexpr int L_ROWS_PER_BLOCK = 4;      // one wave per row at a time, four waves per workgroup
-constexpr int L_MAXCH = 4;               // 256-element chunks per row held as per-lane constants (N <= 1024)
+constexpr int L_MAXCH = 8;               // 256-element chunks per row held as per-lane constants (N <= 2048)
 
 struct LossConsts {
   float a1, a2, b1, b2;
@@ -299,6 +299,8 @@ size_t ring_loss_workspace_bytes(int T, int B) {
     else if (nch == 1) { constexpr int NCH = 1; constexpr bool VEC = false; CALL; } \
     else if (nch == 2 && vec) { constexpr int NCH = 2; constexpr bool VEC = true; CALL; } \
     else if (nch == 2) { constexpr int NCH = 2; constexpr bool VEC = false; CALL; } \
+    else if (nch <= 4 && vec) { constexpr int NCH = 4; constexpr bool VEC = true; CALL; } \
+    else if (nch <= 4) { constexpr int NCH = 4; constexpr bool VEC = false; CALL; } \
     else if (vec) { constexpr int NCH = L_MAXCH; constexpr bool VEC = true; CALL; } \
     else { constexpr int NCH = L_MAXCH; constexpr bool VEC = false; CALL; }         \
   }

@@ -260,7 +260,7 @@ int ringattr_bwd_loss(const void* loss_workspace, const void* upstream, const vo
                       void* stream) {
   if (!loss_workspace) return fail(RINGATTR_ERR_INVALID, "ringattr_bwd_loss: null loss workspace");
   if (!aligned16(loss_workspace)) return fail(RINGATTR_ERR_INVALID, "ringattr_bwd_loss: every pointer must be 16-byte aligned");
-  if (N > 1024) return fail(RINGATTR_ERR_INVALID, "the loss head supports N <= 1024 (got %d)", N);
+  if (N > 2048) return fail(RINGATTR_ERR_INVALID, "the loss head supports N <= 2048 (got %d)", N);
   return bwd_impl("ringattr_bwd_loss", nullptr, loss_workspace, upstream, A, Wa, J0, J1, Wo, bump_history, r_init, grad_Wa,
                   grad_Wo, alpha, N, a_dim, seq_len, batch_size, activation_type, accumulate, saved, grad_A, grad_r_init,
                   workspace, workspace_bytes, stream);
@@ -268,7 +268,7 @@ int ringattr_bwd_loss(const void* loss_workspace, const void* upstream, const vo
 
 int ringattr_bwd_loss_available(int N, int a_dim, int seq_len, int batch_size) {
   Geo g;
-  if (N > 1024 || make_geo(N, a_dim, seq_len, batch_size, g) != RINGATTR_OK) return 0;
+  if (make_geo(N, a_dim, seq_len, batch_size, g) != RINGATTR_OK) return 0;
   return ring_uses_step_kernels(N, a_dim, g.NC, g.nbt) ? 0 : 1;
 }
 
@@ -425,8 +425,8 @@ size_t ringattr_loss_workspace_bytes(int N, int seq_len, int batch_size) {
     fail(RINGATTR_ERR_INVALID, "N, seq_len, batch_size must be positive (got %d, %d, %d)", N, seq_len, batch_size);
     return 0;
   }
-  if (N > 1024) {
-    fail(RINGATTR_ERR_INVALID, "the loss head supports N <= 1024 (got %d)", N);
+  if (N > 2048) {
+    fail(RINGATTR_ERR_INVALID, "the loss head supports N <= 2048 (got %d)", N);
     return 0;
   }
   return align_up(ring_loss_workspace_bytes(seq_len, batch_size));

@@ -17,7 +17,8 @@ def _bumps(rng, T, B, N):
 
 
 @pytest.mark.parametrize("T,B,N,own", [(20, 37, 256, True), (7, 5, 130, True), (9, 16, 512, False), (3, 4, 24, True),
-                                        (5, 3, 700, False)], ids=["n256", "n130_scalar", "n512_given_target", "n24", "n700"])
+                                        (5, 3, 700, False), (4, 6, 2048, True), (3, 5, 1130, False)],
+                         ids=["n256", "n130_scalar", "n512_given_target", "n24", "n700", "n2048", "n1130_scalar"])
 def test_loss_and_gradient_match_the_oracle(T, B, N, own, gpu_device):
     from rnn_train_ring_attractor_amd import ring_loss_pair
     print(f"[case] loss head T={T} B={B} N={N}", flush=True)
@@ -76,7 +77,10 @@ def test_loss_head_agrees_with_the_torch_chain_on_operator_output(gpu_device):
     (20, 6, 3, 96, "silu", True, "0", "random"),      # the streaming kernels, two column tiles, three action channels
     (40, 5, 2, 512, "tanh", True, "0", "random"),     # widest tiling
     (24, 5, 2, 1024, "tanh", True, "0", "random"),    # wide ring: the operator chains loss backward and time-loop backward
-], ids=["n256_full", "n256_random", "n200_masked", "n200_streaming", "n96_k3", "n512", "n1024_step"])
+    (18, 4, 2, 2048, "tanh", True, "0", "random"),    # the widest ring (eight 256-neuron chunks per row in the loss head)
+    (18, 4, 2, 1301, "silu", False, "0", "random"),   # six chunks, ragged width (scalar row loads)
+], ids=["n256_full", "n256_random", "n200_masked", "n200_streaming", "n96_k3", "n512", "n1024_step", "n2048_step",
+        "n1301_step"])
 def test_time_loop_and_loss_as_one_operator(B, T, k, N, act, own, streaming, weights, gpu_device, monkeypatch):
     """ring_rnn_loss_func (one backward call, the loss gradient formed inside the BPTT kernel) against
     ring_rnn_cuda_func + ring_loss_pair (the gradient written to HBM and read back), and against the fp64 oracle:
