@@ -8,7 +8,7 @@
 // front of the time loop instead of inside it: 8 bytes per sample-step of traffic, and the time-loop kernels stay as
 // they are.  Backward: from dL/dA (which the BPTT kernels produce) to the 3h + 1 parameter gradients per channel,
 // summed over B*T samples in a fixed order (per-thread partial sums, fixed tree inside a workgroup, per-workgroup
-// partials summed in workgroup order by a second launch), and optionally dL/dx.
+// partials summed in a fixed order by a second launch), and optionally dL/dx.
 //
 // Parameters are packed per channel as [w1[0..h) | b1[0..h) | w2[0..h) | b2]; gradients use the same packing.
 #include "ring_common.hpp"
@@ -142,19 +142,28 @@ __global__ __launch_bounds__(GAIN_THREADS) void ring_gain_bwd_kernel(const float
     partial[((size_t)blockIdx.x * k + c) * PS + o] = ((red[0][o] + red[1][o]) + red[2][o]) + red[3][o];
 }
 
-// grad_params[c][3h+1] = sum over workgroups (in workgroup order) of partial[blk][c][3H+1], un-padded
+// grad_params[c][3h+1] = sum over workgroups of partial[blk][c][3H+1], un-padded.  One wave per output: lane l adds
+// the partials of workgroups l, l + 64, ... in that order (independent loads, all in flight together), then the 64
+// lane sums are combined by a fixed butterfly, so the result does not depend on scheduling.
 template <int H>
 __global__ __launch_bounds__(GAIN_THREADS) void ring_gain_reduce_kernel(const float* __restrict__ partial,
                                                                         float* __restrict__ grad_params, int k, int h,
                                                                         int nblk) {
   constexpr int PS = 3 * H + 1;
-  const int i = blockIdx.x * GAIN_THREADS + threadIdx.x;
-  if (i >= k * (3 * h + 1)) return;
+  const int lane = threadIdx.x & 63;
+  const int i = blockIdx.x * (GAIN_THREADS / 64) + (threadIdx.x >> 6);
+  if (i >= k * (3 * h + 1)) return;                        // whole waves leave together
   const int c = i / (3 * h + 1), o = i % (3 * h + 1);
   const int po = o == 3 * h ? 3 * H : (o / h) * H + (o % h);
   float s = 0.f;
-  for (int b = 0; b < nblk; ++b) s += partial[((size_t)b * k + c) * PS + po];
-  grad_params[i] = s;
+  for (int b = lane; b < nblk; b += 64) s += partial[((size_t)b * k + c) * PS + po];
+  s = row16_sum_dpp(s);
+  const int si = __builtin_bit_cast(int, s);
+  const float total = (__builtin_bit_cast(float, __builtin_amdgcn_readlane(si, 0)) +
+                       __builtin_bit_cast(float, __builtin_amdgcn_readlane(si, 16))) +
+                      (__builtin_bit_cast(float, __builtin_amdgcn_readlane(si, 32)) +
+                       __builtin_bit_cast(float, __builtin_amdgcn_readlane(si, 48)));
+  if (lane == 0) grad_params[i] = total;
 }
 
 static int gain_pad(int h) { return h <= 8 ? 8 : (h <= 16 ? 16 : (h <= 32 ? 32 : 0)); }
@@ -202,7 +211,7 @@ hipError_t ring_launch_gain_bwd(const float* x, const float* params, const float
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return e;
   const int n = k * (3 * h + 1);
-  const unsigned rb = (unsigned)((n + GAIN_THREADS - 1) / GAIN_THREADS);
+  const unsigned rb = (unsigned)((n + GAIN_THREADS / 64 - 1) / (GAIN_THREADS / 64));   // one wave per output
   switch (H) {
     case 8: hipLaunchKernelGGL(ring_gain_reduce_kernel<8>, dim3(rb), dim3(GAIN_THREADS), 0, st, partial, grad_params, k, h, nblk); break;
     case 16: hipLaunchKernelGGL(ring_gain_reduce_kernel<16>, dim3(rb), dim3(GAIN_THREADS), 0, st, partial, grad_params, k, h, nblk); break;
