@@ -126,6 +126,18 @@ RINGATTR_API int ringattr_loss_bwd(const void* bump_history, const void* target_
                       float bump_weight, const void* upstream, void* grad_history, int N, int seq_len,
                       int batch_size, const void* workspace, size_t workspace_bytes, void* stream);
 
+/* ringattr_fwd followed by ringattr_loss_fwd in one call (same arguments, the time loop's first): the forward of
+ *   total = loss_pair(bump_history),  bump_history = forward(...)
+ * Where the weight-resident forward kernel serves the shape (128 < N <= 256, a_dim = 2) it forms the loss head's three
+ * sums per history row itself, right after the activation, and the loss needs no pass of its own over the history
+ * (-4N bytes read per sample-step); other shapes run the two stages back to back.  Either way loss_workspace ends up
+ * as ringattr_loss_fwd leaves it (for ringattr_loss_bwd / ringattr_bwd_loss).  No counterpart in the reference. */
+RINGATTR_API int ringattr_fwd_loss(const void* A, const void* Wa, float J0, float J1, const void* Wo, const void* r_init,
+                      void* bump_history, float alpha, int N, int a_dim, int seq_len, int batch_size,
+                      int activation_type, void* saved, void* workspace, size_t workspace_bytes,
+                      const void* target_angle, const void* target_amplitude, float bump_weight, void* loss_out,
+                      void* loss_workspace, size_t loss_workspace_bytes, void* stream);
+
 /* ringattr_bwd with the loss head's gradient in place of grad_output: the backward of
  *   total = loss_pair(bump_history),  bump_history = forward(...)
  * in one call.  No counterpart in the reference (its training script lets autograd chain the torch loss ops into

@@ -29,6 +29,9 @@ PROTOTYPES = {
     "ringattr_bwd_workspace_bytes": (c_size_t, [c_int] * 5),
     "ringattr_fwd": (c_int, [c_void_p, c_void_p, c_float, c_float, c_void_p, c_void_p, c_void_p, c_float,
                              c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_size_t, c_void_p]),
+    "ringattr_fwd_loss": (c_int, [c_void_p, c_void_p, c_float, c_float, c_void_p, c_void_p, c_void_p, c_float,
+                                  c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_size_t,
+                                  c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_size_t, c_void_p]),
     "ringattr_fwd_noalloc": (c_int, [c_void_p, c_void_p, c_float, c_float, c_void_p, c_void_p, c_void_p, c_float,
                                      c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p]),
     "ringattr_bwd": (c_int, [c_void_p, c_void_p, c_void_p, c_float, c_float, c_void_p, c_void_p, c_void_p,

@@ -14,6 +14,9 @@ struct RingFwdArgs {
   __bf16* rfrag;         // bf16 r_prev in tile order, or null
   float J0, J1, alpha;
   int N, k, T, B, nbt, act;
+  // Loss head's per-row sums (sum_i r_i cos(phi_i), sum_i r_i sin(phi_i), sum_i |r_i|, -) of every history row
+  // [T*B], written by the weight-resident forward kernel itself when non-null (other kernels ignore it).
+  ring_f32x4* loss_stats = nullptr;
 };
 
 struct RingBpttArgs {
@@ -91,7 +94,10 @@ hipError_t ring_launch_dw_tiled(const RingDwArgs& a, int NC, hipStream_t st);
 // Fused decode + loss head over the state history (ring_loss.hip).
 size_t ring_loss_workspace_bytes(int T, int B);
 hipError_t ring_launch_loss_fwd(const float* hist, const float* angle, const float* target_amp, float bump_weight,
-                                float* loss_out, int N, int T, int B, void* workspace, hipStream_t st);
+                                float* loss_out, int N, int T, int B, void* workspace, bool have_row_sums,
+                                hipStream_t st);
+// where the forward kernel leaves the per-row sums for ring_launch_loss_fwd(..., have_row_sums = true)
+ring_f32x4* ring_loss_row_sums(void* workspace);
 hipError_t ring_launch_loss_bwd(const float* hist, const float* angle, const float* target_amp, float bump_weight,
                                 const float* upstream, float* grad_hist, int N, int T, int B, const void* workspace,
                                 hipStream_t st);

@@ -322,14 +322,19 @@ static LossWs carve(void* workspace, int T, int B) {
   return w;
 }
 
+// have_row_sums: the workspace's row-sum array (ring_loss_row_sums) is already filled (by the forward kernel); the
+// pass over the history is skipped and `hist` is not read.
 hipError_t ring_launch_loss_fwd(const float* hist, const float* angle, const float* target_amp, float bump_weight,
-                                float* loss_out, int N, int T, int B, void* workspace, hipStream_t st) {
+                                float* loss_out, int N, int T, int B, void* workspace, bool have_row_sums,
+                                hipStream_t st) {
   if (N > 256 * L_MAXCH) return hipErrorInvalidValue;
   const LossWs w = carve(workspace, T, B);
   const LossConsts k = loss_consts(N);
   const long rows = (long)T * B;
   const int grid = loss_grid(rows);
-  LOSS_DISPATCH(hipLaunchKernelGGL((ring_loss_stats_kernel<NCH, VEC>), dim3(grid), dim3(256), 0, st, hist, w.stats, N, T, B));
+  if (!have_row_sums) {
+    LOSS_DISPATCH(hipLaunchKernelGGL((ring_loss_stats_kernel<NCH, VEC>), dim3(grid), dim3(256), 0, st, hist, w.stats, N, T, B));
+  }
   hipLaunchKernelGGL(ring_loss_rows_kernel, dim3((B + 31) / 32), dim3(256), 0, st, w.stats, target_amp, w.tgt, w.dsum, w.sq,
                      T, B);
   const int dgrid = (int)((rows + 255) / 256 < 2048 ? (rows + 255) / 256 : 2048);
@@ -338,6 +343,10 @@ hipError_t ring_launch_loss_fwd(const float* hist, const float* angle, const flo
   hipLaunchKernelGGL(ring_loss_final_kernel, dim3(1), dim3(256), 0, st, w.partial, dgrid, w.sq, B, 1.f / (float)rows,
                      bump_weight, loss_out);
   return hipGetLastError();
+}
+
+ring_f32x4* ring_loss_row_sums(void* workspace) {
+  return reinterpret_cast<ring_f32x4*>(workspace);         // carve(): the per-row array leads the workspace
 }
 
 const ring_f32x4* ring_loss_row_coefficients(const void* workspace) {

@@ -97,7 +97,8 @@ __device__ __forceinline__ void load_resident(const bf16x8* Wp, bf16x8* wl, bf16
 namespace {
 
 constexpr int R8_HALF_SLOTS = 4 * 4 * XG;   // 16-byte slots of one operand half (4 K chunks)
-constexpr size_t R8_LDS_BYTES = (size_t)(R_WLDS_SLOTS + 3 * R8_HALF_SLOTS) * 16 + 2 * R_GCH * 16 * 8;
+constexpr size_t R8_STAT_FLOATS = 2 * 8 * 3 * 16;   // loss-head row sums per wave: [step parity][wave][C, S, |r|][row]
+constexpr size_t R8_LDS_BYTES = (size_t)(R_WLDS_SLOTS + 3 * R8_HALF_SLOTS) * 16 + 2 * R_GCH * 16 * 8 + R8_STAT_FLOATS * 4;
 
 __device__ __forceinline__ void load_resident8(const bf16x8* Wp, bf16x8* wl, bf16x8 (&wreg)[2][2][R_KCH], int w, int h,
                                                int lane) {
@@ -126,13 +127,18 @@ __device__ __forceinline__ void write_half(bf16x8* half, const float (&v)[4][2],
 
 }  // namespace
 
-template <int ACT, bool SAVE, bool FULL>
+// STATS: also leave the loss head's three sums of every history row (sum_i r_i cos(phi_i), sum_i r_i sin(phi_i),
+// sum_i |r_i|, phi_i = 2 pi i / N) in p.loss_stats[t * B + b], so that the loss needs no pass of its own over the
+// history.  Each wave reduces its 32 neurons' share over the row group's 16 lanes right after the activation, the
+// eight shares meet in LDS (buffer by step parity) and wave 0 adds them in wave order behind the next barrier.
+template <int ACT, bool SAVE, bool FULL, bool STATS>
 __global__ __launch_bounds__(512) void ring_fwd_res256_kernel(RingFwdArgs p) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
   bf16x8* wlds = reinterpret_cast<bf16x8*>(smem);
   bf16x8* xE = wlds + R_WLDS_SLOTS;               // two buffers, step parity
   bf16x8* xL = xE + 2 * R8_HALF_SLOTS;
   f32x2* gbuf = reinterpret_cast<f32x2*>(xL + R8_HALF_SLOTS);
+  float* statp = reinterpret_cast<float*>(gbuf + 2 * R_GCH * 16);
 
   const int tid = threadIdx.x, w8 = tid >> 6, h = w8 >> 2, w = w8 & 3, lane = tid & 63, q = lane >> 4, n = lane & 15;
   const int bt = blockIdx.x;
@@ -165,6 +171,42 @@ __global__ __launch_bounds__(512) void ring_fwd_res256_kernel(RingFwdArgs p) {
     for (int cc = 0; cc < 2; ++cc) {
       bf16x4 pk = {(__bf16)r[0][cc], (__bf16)r[1][cc], (__bf16)r[2][cc], (__bf16)r[3][cc]};
       *reinterpret_cast<bf16x4*>(p.rfrag + pair_offset<R_NC>(t, p.nbt, bt, w * R_NC + ct0 + cc, lc)) = pk;
+    }
+  };
+  float scs[2] = {0.f, 0.f}, ssn[2] = {0.f, 0.f};
+  if constexpr (STATS) {
+#pragma unroll
+    for (int cc = 0; cc < 2; ++cc) sincosf(6.283185307179586f * (float)(i0 + cc) / (float)N, &ssn[cc], &scs[cc]);
+  }
+  // r[][] holds this wave's part of history row `row_t` (masked entries are zero): its share of the three sums
+  auto stat_share = [&](int row_t) {
+    float* dst = statp + (size_t)(((row_t & 1) * 8 + w8) * 3) * 16 + 4 * q;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      float c = fmaf(r[e][1], scs[1], r[e][0] * scs[0]);
+      float sn = fmaf(r[e][1], ssn[1], r[e][0] * ssn[0]);
+      float ab = fabsf(r[e][0]) + fabsf(r[e][1]);
+      c = row16_sum_dpp(c);
+      sn = row16_sum_dpp(sn);
+      ab = row16_sum_dpp(ab);
+      if (n == 0) {
+        dst[e] = c;
+        dst[16 + e] = sn;
+        dst[32 + e] = ab;
+      }
+    }
+  };
+  // the eight shares of row `row_t` are complete behind a barrier: wave 0 adds them in wave order and stores the row sums
+  auto stat_flush = [&](int row_t) {
+    if (w8 == 0) {
+      const int kind = lane >> 4, row = lane & 15, b = 16 * bt + row;
+      float v = 0.f;
+      if (kind < 3) {
+        const float* src = statp + (size_t)((row_t & 1) * 8 * 3 + kind) * 16 + row;
+#pragma unroll
+        for (int wv = 0; wv < 8; ++wv) v += src[wv * 3 * 16];
+      }
+      if (b < B) reinterpret_cast<float*>(p.loss_stats + (size_t)row_t * B + b)[kind] = v;
     }
   };
   write_half(h ? xL : xE, r, w, q, n);
@@ -300,10 +342,14 @@ __global__ __launch_bounds__(512) void ring_fwd_res256_kernel(RingFwdArgs p) {
       if (l == 0 && (ci + 1) * R_GCH < T) gates_fetch(p.A, T, B, bt, ci + 1, +1, tid, gs);
       contract_half(0, xE + (t & 1) * R8_HALF_SLOTS, t - 1, emit);
       lds_barrier();   // B_t
+      if constexpr (STATS) {
+        if (t > 0) stat_flush(t - 1);            // both roles' shares of row t-1 are in
+      }
       contract_half(1, xL, t - 1, emit);
       float x[4][2];
       preactivation(t, x);
       activate(x);
+      if constexpr (STATS) stat_share(t);
       if (t + 1 < T) write_half(xE + ((t + 1) & 1) * R8_HALF_SLOTS, r, w, q, n);
       // the next chunk's gates are first read after barrier B of its first step
       if (l == R_GCH - 1 && t + 1 < T) gates_publish(gbuf + ((ci + 1) & 1) * R_GCH * 16, tid, B, bt, gs);
@@ -321,6 +367,7 @@ __global__ __launch_bounds__(512) void ring_fwd_res256_kernel(RingFwdArgs p) {
     lds_barrier();   // A_1
     for (int t = 1; t < T; ++t) {
       activate(x);   // step t-1 -> r^L_t
+      if constexpr (STATS) stat_share(t - 1);
       write_half(xL, r, w, q, n);
       lds_barrier();   // B_t
       contract_half(0, xE + (t & 1) * R8_HALF_SLOTS, t - 1, with_stores);
@@ -329,6 +376,11 @@ __global__ __launch_bounds__(512) void ring_fwd_res256_kernel(RingFwdArgs p) {
       lds_barrier();   // A_{t+1}
     }
     activate(x);
+    if constexpr (STATS) stat_share(T - 1);
+  }
+  if constexpr (STATS) {
+    lds_barrier();                                 // the late role's share of the last row
+    stat_flush(T - 1);
   }
   // stores of the last step (its state is not an operand of any further step)
 #pragma unroll
@@ -730,9 +782,9 @@ __global__ __launch_bounds__(256) void ring_bptt_res256_kernel(RingBpttArgs p) {
 // ------------------------------------------------------------------------------------------------
 bool ring_res256_applicable(int N, int k) { return k == 2 && N > 128 && N <= 256; }
 
-template <int ACT, bool SAVE, bool FULL>
+template <int ACT, bool SAVE, bool FULL, bool STATS>
 static hipError_t launch_fwd_variant(const RingFwdArgs& a, hipStream_t st) {
-  auto kern = ring_fwd_res256_kernel<ACT, SAVE, FULL>;
+  auto kern = ring_fwd_res256_kernel<ACT, SAVE, FULL, STATS>;
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                                      (int)R8_LDS_BYTES);
   if (e != hipSuccess) return e;
@@ -743,8 +795,12 @@ static hipError_t launch_fwd_variant(const RingFwdArgs& a, hipStream_t st) {
 template <int ACT>
 static hipError_t launch_fwd_act(const RingFwdArgs& a, hipStream_t st) {
   const bool full = (a.N == 256) && (a.B % 16 == 0);
-  if (a.dfrag) return full ? launch_fwd_variant<ACT, true, true>(a, st) : launch_fwd_variant<ACT, true, false>(a, st);
-  return full ? launch_fwd_variant<ACT, false, true>(a, st) : launch_fwd_variant<ACT, false, false>(a, st);
+  if (a.loss_stats) {
+    if (a.dfrag) return full ? launch_fwd_variant<ACT, true, true, true>(a, st) : launch_fwd_variant<ACT, true, false, true>(a, st);
+    return full ? launch_fwd_variant<ACT, false, true, true>(a, st) : launch_fwd_variant<ACT, false, false, true>(a, st);
+  }
+  if (a.dfrag) return full ? launch_fwd_variant<ACT, true, true, false>(a, st) : launch_fwd_variant<ACT, true, false, false>(a, st);
+  return full ? launch_fwd_variant<ACT, false, true, false>(a, st) : launch_fwd_variant<ACT, false, false, false>(a, st);
 }
 
 hipError_t ring_launch_fwd_res256(const RingFwdArgs& a, hipStream_t st) {

@@ -167,9 +167,47 @@ size_t ringattr_bwd_workspace_bytes(int N, int a_dim, int seq_len, int batch_siz
   return s;
 }
 
+// loss_stats != null: the forward kernel that can do so also leaves the loss head's per-row sums there; *stats_done
+// says whether it did.
+static int fwd_impl(const void* A, const void* Wa, float J0, float J1, const void* Wo, const void* r_init,
+                    void* bump_history, float alpha, int N, int a_dim, int seq_len, int batch_size, int activation_type,
+                    void* saved, void* workspace, size_t workspace_bytes, ring_f32x4* loss_stats, bool* stats_done,
+                    void* stream);
+
 int ringattr_fwd(const void* A, const void* Wa, float J0, float J1, const void* Wo, const void* r_init,
                  void* bump_history, float alpha, int N, int a_dim, int seq_len, int batch_size,
                  int activation_type, void* saved, void* workspace, size_t workspace_bytes, void* stream) {
+  return fwd_impl(A, Wa, J0, J1, Wo, r_init, bump_history, alpha, N, a_dim, seq_len, batch_size, activation_type, saved,
+                  workspace, workspace_bytes, nullptr, nullptr, stream);
+}
+
+int ringattr_fwd_loss(const void* A, const void* Wa, float J0, float J1, const void* Wo, const void* r_init,
+                      void* bump_history, float alpha, int N, int a_dim, int seq_len, int batch_size, int activation_type,
+                      void* saved, void* workspace, size_t workspace_bytes, const void* target_angle,
+                      const void* target_amplitude, float bump_weight, void* loss_out, void* loss_workspace,
+                      size_t loss_workspace_bytes, void* stream) {
+  const size_t need = ringattr_loss_workspace_bytes(N, seq_len, batch_size);
+  if (need == 0) return RINGATTR_ERR_INVALID;
+  if (!target_angle || !loss_out) return fail(RINGATTR_ERR_INVALID, "ringattr_fwd_loss: null tensor pointer");
+  if (!aligned16(loss_workspace)) return fail(RINGATTR_ERR_INVALID, "ringattr_fwd_loss: every pointer must be 16-byte aligned");
+  if (!loss_workspace || loss_workspace_bytes < need)
+    return fail(RINGATTR_ERR_WORKSPACE, "ringattr_fwd_loss: loss workspace of %zu bytes needed, %zu given", need,
+                loss_workspace ? loss_workspace_bytes : (size_t)0);
+  bool stats_done = false;
+  const int rc = fwd_impl(A, Wa, J0, J1, Wo, r_init, bump_history, alpha, N, a_dim, seq_len, batch_size, activation_type,
+                          saved, workspace, workspace_bytes, ring_loss_row_sums(loss_workspace), &stats_done, stream);
+  if (rc) return rc;
+  hipError_t e = ring_launch_loss_fwd((const float*)bump_history, (const float*)target_angle, (const float*)target_amplitude,
+                                      bump_weight, (float*)loss_out, N, seq_len, batch_size, loss_workspace, stats_done,
+                                      static_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return hip_fail(e, "loss head forward launch");
+  return RINGATTR_OK;
+}
+
+static int fwd_impl(const void* A, const void* Wa, float J0, float J1, const void* Wo, const void* r_init,
+                    void* bump_history, float alpha, int N, int a_dim, int seq_len, int batch_size, int activation_type,
+                    void* saved, void* workspace, size_t workspace_bytes, ring_f32x4* loss_stats, bool* stats_done,
+                    void* stream) {
   Geo g;
   int rc = make_geo(N, a_dim, seq_len, batch_size, g);
   if (rc) return rc;
@@ -209,6 +247,9 @@ int ringattr_fwd(const void* A, const void* Wa, float J0, float J1, const void* 
   a.B = batch_size;
   a.nbt = g.nbt;
   a.act = activation_type;
+  // only the weight-resident forward kernel forms the loss head's row sums
+  a.loss_stats = (resident && !ring_uses_step_kernels(N, a_dim, g.NC, g.nbt)) ? loss_stats : nullptr;
+  if (stats_done) *stats_done = a.loss_stats != nullptr;
   e = ring_launch_fwd(a, g.NC, st);
   if (e != hipSuccess) return hip_fail(e, "forward launch");
   return RINGATTR_OK;
@@ -444,7 +485,7 @@ int ringattr_loss_fwd(const void* bump_history, const void* target_angle, const 
     return fail(RINGATTR_ERR_WORKSPACE, "ringattr_loss_fwd: workspace of %zu bytes needed, %zu given", need,
                 workspace ? workspace_bytes : (size_t)0);
   hipError_t e = ring_launch_loss_fwd((const float*)bump_history, (const float*)target_angle, (const float*)target_amplitude,
-                                      bump_weight, (float*)loss_out, N, seq_len, batch_size, workspace,
+                                      bump_weight, (float*)loss_out, N, seq_len, batch_size, workspace, false,
                                       static_cast<hipStream_t>(stream));
   if (e != hipSuccess) return hip_fail(e, "loss head forward launch");
   return RINGATTR_OK;

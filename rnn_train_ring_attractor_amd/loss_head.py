@@ -111,8 +111,6 @@ class RingRnnLossFunc(Function):
         needs_grad = grad_mode is not False and any(ctx.needs_input_grad[i] for i in (0, 1, 4, 5))
         ctx.extra_inputs = 0 if grad_mode is None else 1
         saved = torch.empty(saved_nbytes(N, k, T, B), dtype=torch.uint8, device=dev) if needs_grad else None
-        fwd_cuda.fwd(A=A, Wa=Wa_c, J0=J0, J1=J1, Wo=Wo_c, r_init=r0, bump_history=hist, alpha=alpha,
-                     activation_type=act, saved=saved)
         lib = _lib.load()
         with torch.cuda.device(dev):
             nbytes = lib.ringattr_loss_workspace_bytes(N, T, B)
@@ -120,12 +118,13 @@ class RingRnnLossFunc(Function):
                 _lib.check(1)
             lws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
             out = torch.empty(3, dtype=torch.float32, device=dev)
-            _lib.check(lib.ringattr_loss_fwd(hist.data_ptr(), angle.data_ptr(), amp.data_ptr() if amp is not None else None,
-                                             float(bump_weight), out.data_ptr(), N, T, B, lws.data_ptr(), nbytes,
-                                             torch.cuda.current_stream(dev).cuda_stream))
+        # time loop and loss head in one call: the weight-resident forward kernel forms the loss's row sums itself
+        fwd_cuda.fwd(A=A, Wa=Wa_c, J0=J0, J1=J1, Wo=Wo_c, r_init=r0, bump_history=hist, alpha=alpha,
+                     activation_type=act, saved=saved, loss=(angle, amp, float(bump_weight), out, lws))
         ctx.save_for_backward(A, Wa_c, Wo_c, hist, r0, saved, lws, angle, amp)
         ctx.J0, ctx.J1, ctx.alpha, ctx.act, ctx.bump_weight = J0, J1, alpha, act, float(bump_weight)
         ctx.mark_non_differentiable(out, hist)
+        ctx.set_materialize_grads(False)         # no [T,B,N] tensor of zeros for the history's unused gradient
         return out[0].clone(), out, hist
 
     @staticmethod
@@ -134,6 +133,8 @@ class RingRnnLossFunc(Function):
         grad_Wa, grad_Wo = torch.empty_like(Wa), torch.empty_like(Wo)    # written, not accumulated into
         grad_A = torch.empty_like(A) if ctx.needs_input_grad[0] else None
         grad_r0 = torch.empty_like(r0) if ctx.needs_input_grad[5] else None
+        if grad_total is None:                   # (gradients are not materialised: the total went unused)
+            grad_total = torch.zeros((), device=hist.device)
         up = grad_total.to(torch.float32).reshape(1).contiguous()
         T, B, N = hist.shape
         lib = _lib.load()

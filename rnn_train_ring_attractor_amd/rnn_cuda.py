@@ -97,7 +97,9 @@ class _Fwd:
     """Stand-in for the reference's `fwd` extension module (cpp/fwd.cpp:49-55)."""
 
     @staticmethod
-    def fwd(A, Wa, J0, J1, Wo, r_init, bump_history, alpha, activation_type, saved=None, stream=None):
+    def fwd(A, Wa, J0, J1, Wo, r_init, bump_history, alpha, activation_type, saved=None, stream=None, loss=None):
+        # loss (not in the reference): (target_angle [B,T], target_amplitude [B] or None, bump_weight, loss_out [3],
+        # loss_workspace uint8) -- the loss head's forward runs in the same call (ringattr_fwd_loss)
         for name, t in (("A", A), ("Wa", Wa), ("Wo", Wo), ("r_init", r_init), ("bump_history", bump_history)):
             _contig(name, t)
         B, T, k, N = _shapes(A, Wa)
@@ -117,8 +119,15 @@ class _Fwd:
             if ws_bytes == 0:
                 _lib.check(1)
             ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
-            rc = lib.ringattr_fwd(_ptr(A), _ptr(Wa), J0, J1, _ptr(Wo), _ptr(r_init), _ptr(bump_history), alpha,
-                                  N, k, T, B, act, _ptr(saved), _ptr(ws), ws_bytes, _stream_ptr(stream, dev))
+            if loss is None:
+                rc = lib.ringattr_fwd(_ptr(A), _ptr(Wa), J0, J1, _ptr(Wo), _ptr(r_init), _ptr(bump_history), alpha,
+                                      N, k, T, B, act, _ptr(saved), _ptr(ws), ws_bytes, _stream_ptr(stream, dev))
+            else:
+                angle, amp, bump_weight, loss_out, lws = loss
+                rc = lib.ringattr_fwd_loss(_ptr(A), _ptr(Wa), J0, J1, _ptr(Wo), _ptr(r_init), _ptr(bump_history), alpha,
+                                           N, k, T, B, act, _ptr(saved), _ptr(ws), ws_bytes, _ptr(angle), _ptr(amp),
+                                           float(bump_weight), _ptr(loss_out), _ptr(lws), lws.numel(),
+                                           _stream_ptr(stream, dev))
         _lib.check(rc)
         return None
 

@@ -99,7 +99,7 @@ def test_hot_kernels_use_no_scratch(res256_asm):
     for b in blocks[1:]:
         name = b.split()[0]
         m = re.search(r"ScratchSize \[bytes/lane\]: (\d+)", b)
-        full_fwd = re.match(r"_Z22ring_fwd_res256_kernelILi\dELb[01]ELb1EE", name)
+        full_fwd = re.match(r"_Z22ring_fwd_res256_kernelILi\dELb[01]ELb1ELb[01]EE", name)
         full_bptt = name.startswith("_Z23ring_bptt_res256_kernelILb1E")
         if full_fwd or full_bptt:
             seen += 1

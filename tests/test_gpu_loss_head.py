@@ -110,7 +110,11 @@ def test_time_loop_and_loss_as_one_operator(B, T, k, N, act, own, streaming, wei
         res[fused] = (float(total), float(lc), float(la), hist.detach().cpu().numpy(), Wo.grad.cpu().numpy(),
                       Wa.grad.cpu().numpy(), r0.grad.cpu().numpy())
     f, s = res[True], res[False]
-    assert f[0] == s[0] and f[1] == s[1] and f[2] == s[2] and np.array_equal(f[3], s[3])     # same forward kernels
+    # the same trajectory; the loss values agree to rounding (the weight-resident forward kernel forms the loss
+    # head's row sums itself, in another order than the pass over the history that the two-operator chain runs)
+    assert np.array_equal(f[3], s[3])
+    for x, y in zip(f[:3], s[:3]):
+        assert abs(x - y) <= 2e-6 * max(1.0, abs(y))
     for a, b in zip(f[4:], s[4:]):
         assert np.isfinite(a).all()
         assert O.max_rel_err(a, b) <= 2e-3 and O.cosine(a, b) >= 0.99999
