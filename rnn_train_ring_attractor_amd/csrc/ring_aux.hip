@@ -38,46 +38,83 @@ __device__ __forceinline__ float rand_unit(unsigned long long seed, unsigned str
 
 }  // namespace
 
-// One thread per trial.  av [B,T], angle [B,T], action [B,T,k].
+// av [B,T], angle [B,T], action [B,T,k].  A workgroup takes GEN_TRIALS trials through the sequence in chunks of
+// GEN_TCH steps, in three phases per chunk: all threads draw the chunk's random numbers (the generator is stateless,
+// so every (trial, step) draw is independent), one thread per trial walks its steps in order (selection sampling and
+// the running angle are the only sequential parts: a compare, a subtract and an add per step), and all threads write
+// the chunk out with consecutive threads on consecutive addresses.
+namespace {
+constexpr int GEN_TRIALS = 16;
+constexpr int GEN_TCH = 128;
+}  // namespace
+
 __global__ __launch_bounds__(256) void ring_generate_trials_kernel(RingGenArgs p) {
-  const int b = blockIdx.x * blockDim.x + threadIdx.x;
-  if (b >= p.B) return;
+  __shared__ float draw[GEN_TCH][GEN_TRIALS + 1];   // selection draw * positions left;  then the step's angle
+  __shared__ float cand[GEN_TCH][GEN_TRIALS + 1];   // candidate velocity;               then the step's velocity
+  const int tid = threadIdx.x, b0 = blockIdx.x * GEN_TRIALS;
   const int T = p.T, k = p.k;
   const int n0 = (int)((float)T * p.start_ratio);
   const int rest = T - n0;
   const float two_pi = 6.283185307179586f;
-  const float angle0 = rand_unit(p.seed, 0, (unsigned long long)b) * two_pi;
-  const int pick = (int)(rand_u32(p.seed, 1, (unsigned long long)b) % (unsigned)p.n_ratios);
-  int need = rest - (int)((float)rest * p.ratios[pick]);     // float32 product, truncated, as the reference
-  need = need < 0 ? 0 : (need > rest ? rest : need);
-  float run = 0.f;                                           // sum of av[s], s < t
-  float* av = p.av + (size_t)b * T;
-  float* ang = p.angle + (size_t)b * T;
-  float* act = p.action + (size_t)b * T * k;
-  for (int t = 0; t < T; ++t) {
-    float v = 0.f;
-    if (t >= n0) {
-      const int left = T - t;                                // positions still available, this one included
-      const unsigned long long c = (unsigned long long)b * T + t;
-      if (rand_unit(p.seed, 2, c) * (float)left < (float)need) {
-        v = (rand_unit(p.seed, 3, c) - 0.5f) * (2.f * p.max_av);
-        --need;
+  // per-trial state of the sequential phase (threads 0 .. GEN_TRIALS-1)
+  const int bs = b0 + tid;
+  float angle0 = 0.f, run = 0.f;                    // run: sum of av[s], s < t
+  int need = 0;
+  if (tid < GEN_TRIALS && bs < p.B) {
+    angle0 = rand_unit(p.seed, 0, (unsigned long long)bs) * two_pi;
+    const int pick = (int)(rand_u32(p.seed, 1, (unsigned long long)bs) % (unsigned)p.n_ratios);
+    need = rest - (int)((float)rest * p.ratios[pick]);         // float32 product, truncated, as the reference
+    need = need < 0 ? 0 : (need > rest ? rest : need);
+  }
+  for (int t0 = 0; t0 < T; t0 += GEN_TCH) {
+    const int nt = T - t0 < GEN_TCH ? T - t0 : GEN_TCH;
+    for (int idx = tid; idx < nt * GEN_TRIALS; idx += 256) {
+      const int tl = idx / GEN_TRIALS, j = idx % GEN_TRIALS, b = b0 + j, t = t0 + tl;
+      if (b < p.B) {
+        const unsigned long long c = (unsigned long long)b * T + t;
+        draw[tl][j] = rand_unit(p.seed, 2, c) * (float)(T - t);   // T - t positions are still available, this one included
+        cand[tl][j] = (rand_unit(p.seed, 3, c) - 0.5f) * (2.f * p.max_av);
       }
     }
-    float a = angle0 + run;
-    a -= floorf(a / two_pi) * two_pi;                         // Python's %: result in [0, 2 pi)
-    if (t == 0) a = angle0;
-    av[t] = v;
-    ang[t] = a;
-    if (p.spread) {
-      for (int c = 0; c < k; ++c) {
+    __syncthreads();
+    if (tid < GEN_TRIALS && bs < p.B) {
+      for (int tl = 0; tl < nt; ++tl) {
+        const int t = t0 + tl;
+        float v = 0.f;
+        if (t >= n0 && draw[tl][tid] < (float)need) {
+          v = cand[tl][tid];
+          --need;
+        }
+        float a = angle0 + run;
+        a -= floorf(a / two_pi) * two_pi;                       // Python's %: result in [0, 2 pi)
+        if (t == 0) a = angle0;
+        cand[tl][tid] = v;
+        draw[tl][tid] = a;
+        run += v;
+      }
+    }
+    __syncthreads();
+    for (int idx = tid; idx < nt * GEN_TRIALS; idx += 256) {
+      const int j = idx / nt, tl = idx % nt, b = b0 + j;
+      if (b < p.B) {
+        p.av[(size_t)b * T + t0 + tl] = cand[tl][j];
+        p.angle[(size_t)b * T + t0 + tl] = draw[tl][j];
+      }
+    }
+    for (int idx = tid; idx < nt * GEN_TRIALS * k; idx += 256) {
+      const int c = idx % k, tl = (idx / k) % nt, j = idx / (k * nt), b = b0 + j;
+      if (b >= p.B) continue;
+      const float v = cand[tl][j];
+      float out;
+      if (p.spread) {
         const float scale = k > 1 ? -1.f + 2.f * (float)c / (float)(k - 1) : -1.f;   // linspace(-1, 1, k)
-        act[(size_t)t * k + c] = fmaxf(v * scale, 0.f);
+        out = fmaxf(v * scale, 0.f);
+      } else {
+        out = c == 0 ? fmaxf(-v, 0.f) : (c == 1 ? fmaxf(v, 0.f) : 0.f);
       }
-    } else {
-      for (int c = 0; c < k; ++c) act[(size_t)t * k + c] = c == 0 ? fmaxf(-v, 0.f) : (c == 1 ? fmaxf(v, 0.f) : 0.f);
+      p.action[((size_t)b * T + t0 + tl) * k + c] = out;
     }
-    run += v;
+    __syncthreads();
   }
 }
 
@@ -115,7 +152,7 @@ __global__ __launch_bounds__(256) void ring_generate_bump_kernel(RingGenArgs p) 
 }
 
 hipError_t ring_launch_generate(const RingGenArgs& a, hipStream_t st) {
-  hipLaunchKernelGGL(ring_generate_trials_kernel, dim3((a.B + 255) / 256), dim3(256), 0, st, a);
+  hipLaunchKernelGGL(ring_generate_trials_kernel, dim3((a.B + GEN_TRIALS - 1) / GEN_TRIALS), dim3(256), 0, st, a);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess || !a.r_init) return e;
   hipLaunchKernelGGL(ring_generate_bump_kernel, dim3(a.B), dim3(256), 0, st, a);

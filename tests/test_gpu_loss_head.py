@@ -158,3 +158,24 @@ def test_one_operator_also_returns_the_action_signal_gradient(B, T, k, N, act, g
     for a, b in zip(res[True], res[False]):
         assert np.isfinite(a).all() and np.abs(b).max() > 0
         assert O.max_rel_err(a, b) <= 2e-3 and O.cosine(a, b) >= 0.99999
+
+
+@pytest.mark.parametrize("B,N", [(32, 256), (21, 200)], ids=["n256_full", "n200_masked"])
+def test_one_operator_without_a_backward_returns_the_same_losses(B, N, gpu_device):
+    """Under torch.no_grad() the forward keeps no saved record (another variant of the forward kernel forms the loss
+    head's row sums); losses and trajectory equal those of the call that prepares a backward."""
+    from rnn_train_ring_attractor_amd import ring_rnn_loss_func
+    from tests.ring_cases import make_problem
+    T, k = 11, 2
+    print(f"[case] time loop + loss operator under no_grad B={B} T={T} N={N}", flush=True)
+    p = make_problem(77 + N, B, T, k, N, weights="perfect")
+    t = lambda x: torch.tensor(np.ascontiguousarray(x), device=gpu_device)
+    args = lambda grad: (t(p["A"]), t(p["Wa"]).requires_grad_(grad), -1.0 / N, 2.0 / N, t(p["Wo"]).requires_grad_(grad),
+                         t(p["r0"]), 0.15, "gelu", t(p["angle"]), 0.2, None)
+    with_grad = ring_rnn_loss_func(*args(True))
+    with torch.no_grad():
+        without = ring_rnn_loss_func(*args(True))
+    torch.cuda.synchronize()
+    for a, b in zip(with_grad, without):
+        assert torch.equal(a.detach(), b)
+    assert not without[0].requires_grad
