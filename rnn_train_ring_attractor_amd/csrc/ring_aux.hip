@@ -177,7 +177,18 @@ __global__ __launch_bounds__(OPT_BLOCK) void ring_gradnorm_partial_kernel(RingOp
   const float* g = p.grad[ti];
   const size_t lo = (size_t)blk * OPT_CHUNK, hi = lo + OPT_CHUNK < p.numel[ti] ? lo + OPT_CHUNK : p.numel[ti];
   float s = 0.f;
-  for (size_t i = lo + threadIdx.x; i < hi; i += OPT_BLOCK) s = fmaf(g[i], g[i], s);
+  {
+    constexpr int U = 4;                       // loads of a trip issued together; the sum keeps its element order
+    size_t i = lo + threadIdx.x;
+    for (; i + (U - 1) * OPT_BLOCK < hi; i += U * OPT_BLOCK) {
+      float x[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) x[u] = g[i + u * OPT_BLOCK];
+#pragma unroll
+      for (int u = 0; u < U; ++u) s = fmaf(x[u], x[u], s);
+    }
+    for (; i < hi; i += OPT_BLOCK) s = fmaf(g[i], g[i], s);
+  }
   s = row16_sum_dpp(s);
   const int si = __builtin_bit_cast(int, s);
   s = (__builtin_bit_cast(float, __builtin_amdgcn_readlane(si, 0)) + __builtin_bit_cast(float, __builtin_amdgcn_readlane(si, 16))) +
@@ -220,22 +231,38 @@ __global__ __launch_bounds__(OPT_BLOCK) void ring_clip_adam_kernel(RingOptArgs p
   if (ti >= p.n) return;
   float clip = 1.f;
   if (p.max_norm > 0.f) clip = fminf(p.max_norm / (norm[0] + 1e-6f), 1.f);
-  float* g = p.grad[ti];
-  float* w = p.param[ti];
-  float* m = p.exp_avg[ti];
-  float* v = p.exp_avg_sq[ti];
+  // the four arrays of a tensor are distinct allocations: all loads of a trip can be in flight together
+  float* __restrict__ g = p.grad[ti];
+  float* __restrict__ w = p.param[ti];
+  float* __restrict__ m = p.exp_avg[ti];
+  float* __restrict__ v = p.exp_avg_sq[ti];
   const size_t lo = (size_t)blk * OPT_CHUNK, hi = lo + OPT_CHUNK < p.numel[ti] ? lo + OPT_CHUNK : p.numel[ti];
   const float step_size = p.step_counter ? norm[1] : p.step_size;
   const float inv_sqrt_bc2 = p.step_counter ? norm[2] : p.inv_sqrt_bc2;
-  for (size_t i = lo + threadIdx.x; i < hi; i += OPT_BLOCK) {
-    const float gi = g[i] * clip;
-    const float mi = p.beta1 * m[i] + (1.f - p.beta1) * gi;
-    const float vi = p.beta2 * v[i] + (1.f - p.beta2) * gi * gi;
+  auto update = [&](size_t i, float gr, float mo, float vo, float wo) {
+    const float gi = gr * clip;
+    const float mi = p.beta1 * mo + (1.f - p.beta1) * gi;
+    const float vi = p.beta2 * vo + (1.f - p.beta2) * gi * gi;
     g[i] = gi;
     m[i] = mi;
     v[i] = vi;
-    w[i] -= step_size * (mi / (sqrtf(vi) * inv_sqrt_bc2 + p.eps));
+    w[i] = wo - step_size * (mi / (sqrtf(vi) * inv_sqrt_bc2 + p.eps));
+  };
+  constexpr int U = 4;
+  size_t i = lo + threadIdx.x;
+  for (; i + (U - 1) * OPT_BLOCK < hi; i += U * OPT_BLOCK) {
+    float gr[U], mo[U], vo[U], wo[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      gr[u] = g[i + u * OPT_BLOCK];
+      mo[u] = m[i + u * OPT_BLOCK];
+      vo[u] = v[i + u * OPT_BLOCK];
+      wo[u] = w[i + u * OPT_BLOCK];
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) update(i + u * OPT_BLOCK, gr[u], mo[u], vo[u], wo[u]);
   }
+  for (; i < hi; i += OPT_BLOCK) update(i, g[i], m[i], v[i], w[i]);
 }
 
 int ring_opt_chunks(size_t numel) { return (int)((numel + OPT_CHUNK - 1) / OPT_CHUNK); }
