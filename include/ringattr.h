@@ -128,9 +128,9 @@ RINGATTR_API int ringattr_loss_bwd(const void* bump_history, const void* target_
 
 /* ringattr_fwd followed by ringattr_loss_fwd in one call (same arguments, the time loop's first): the forward of
  *   total = loss_pair(bump_history),  bump_history = forward(...)
- * Where the weight-resident forward kernel serves the shape (128 < N <= 256, a_dim = 2) it forms the loss head's three
- * sums per history row itself, right after the activation, and the loss needs no pass of its own over the history
- * (-4N bytes read per sample-step); other shapes run the two stages back to back.  Either way loss_workspace ends up
+ * The persistent forward kernels (N <= 512, except small-batch forwards that are split over workgroups) form the loss
+ * head's three sums per history row themselves, right after the activation, and the loss needs no pass of its own
+ * over the history (-4N bytes read per sample-step); other shapes run the two stages back to back.  Either way loss_workspace ends up
  * as ringattr_loss_fwd leaves it (for ringattr_loss_bwd / ringattr_bwd_loss).  No counterpart in the reference. */
 RINGATTR_API int ringattr_fwd_loss(const void* A, const void* Wa, float J0, float J1, const void* Wo, const void* r_init,
                       void* bump_history, float alpha, int N, int a_dim, int seq_len, int batch_size,

@@ -295,6 +295,42 @@ __device__ __forceinline__ void read_rowsum(const float* psum, int q, float (&s)
     s[e] = ((psum[0 * 16 + 4 * q + e] + psum[1 * 16 + 4 * q + e]) + psum[2 * 16 + 4 * q + e]) + psum[3 * 16 + 4 * q + e];
 }
 
+// The loss head's three sums per row (sum_i v_i cos(phi_i), sum_i v_i sin(phi_i), sum_i |v_i|, phi_i = 2 pi i / N)
+// over the wave's neurons: per-wave partials to lsum[kind][w * 16 + row].  The lane's NC consecutive angles come from
+// its first one by the angle-addition recurrence (c0, s0 = cos, sin of phi_{i0}; cd, sd = cos, sin of 2 pi / N).
+template <int NC>
+__device__ __forceinline__ void publish_loss_sums(float* lsum, const float (&v)[4][NC], float c0, float s0, float cd,
+                                                  float sd, int w, int q, int n) {
+  float C[4] = {0.f, 0.f, 0.f, 0.f}, S[4] = {0.f, 0.f, 0.f, 0.f}, A[4] = {0.f, 0.f, 0.f, 0.f};
+  float cc = c0, ss = s0;
+#pragma unroll
+  for (int c = 0; c < NC; ++c) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      C[e] = fmaf(v[e][c], cc, C[e]);
+      S[e] = fmaf(v[e][c], ss, S[e]);
+      A[e] += fabsf(v[e][c]);
+    }
+    const float cn = fmaf(cc, cd, -ss * sd);
+    ss = fmaf(ss, cd, cc * sd);
+    cc = cn;
+  }
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    C[e] = row16_sum(C[e]);
+    S[e] = row16_sum(S[e]);
+    A[e] = row16_sum(A[e]);
+  }
+  if (n == 0) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      lsum[0 * 64 + w * 16 + 4 * q + e] = C[e];
+      lsum[1 * 64 + w * 16 + 4 * q + e] = S[e];
+      lsum[2 * 64 + w * 16 + 4 * q + e] = A[e];
+    }
+  }
+}
+
 // ------------------------------------------------------------------------------------------------
 // Forward: one workgroup = RT tiles of 16 batch rows for all T steps.  r lives in fp32 registers; its
 // bf16 copy is exchanged between the four waves through a double-buffered LDS operand buffer (one
@@ -321,7 +357,10 @@ constexpr size_t fwd_state_lds_bytes() { return RT > 1 ? (size_t)RT * 4 * NC * 2
 
 // WL: the packed weights of all 1 + a_dim matrices fit in LDS next to the operand buffers (small N): the workgroup
 // copies them there once and the per-step "stream" reads LDS instead of L2.
-template <int NC, int ACT, int RT, bool WL>
+// STATS: also leave the loss head's three sums of every history row in p.loss_stats[t * B + b] (the waves' shares
+// meet in LDS by step parity and are added in wave order behind the step's barrier), so that the loss needs no pass
+// of its own over the history.
+template <int NC, int ACT, int RT, bool WL, bool STATS>
 __global__ __launch_bounds__(256) void ring_fwd_kernel(RingFwdArgs p) {
   using TL = Tile<NC>;
   extern __shared__ __attribute__((aligned(16))) char stream_lds[];
@@ -335,6 +374,7 @@ __global__ __launch_bounds__(256) void ring_fwd_kernel(RingFwdArgs p) {
   }
   __shared__ float psum[2][RT][64];
   __shared__ float gl[2][RT * 16 * GATE_KMAX];
+  __shared__ float lsum[STATS ? 2 : 1][RT][3 * 64];
 
   const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, q = lane >> 4, n = lane & 15;
   const int bt0 = blockIdx.x * RT;             // tile rt is batch tile bt0 + rt (past the last one: all rows masked)
@@ -343,6 +383,23 @@ __global__ __launch_bounds__(256) void ring_fwd_kernel(RingFwdArgs p) {
   const int N = p.N, B = p.B, T = p.T;
   const float oma = 1.f - p.alpha;
   const bool staged = p.k <= GATE_KMAX;
+  float lc0 = 0.f, ls0 = 0.f, lcd = 0.f, lsd = 0.f;
+  if constexpr (STATS) {
+    sincosf(6.283185307179586f * (float)i0 / (float)N, &ls0, &lc0);
+    sincosf(6.283185307179586f / (float)N, &lsd, &lcd);
+  }
+  // row sums of history row `row_t` from the shares in lsum[buf] (complete behind a barrier): threads 0 .. 64 RT - 1
+  auto flush_loss_sums = [&](int row_t, int buf) {
+    if (tid < 64 * RT) {
+      const int rt = tid >> 6, kind = (tid >> 4) & 3, row = tid & 15, b = 16 * (bt0 + rt) + row;
+      float v = 0.f;
+      if (kind < 3) {
+        const float* src = lsum[buf][rt] + kind * 64 + row;
+        v = ((src[0] + src[16]) + src[32]) + src[48];
+      }
+      if (b < B) reinterpret_cast<float*>(p.loss_stats + (size_t)row_t * B + b)[kind] = v;
+    }
+  };
   auto xb = [&](int buf, int rt) { return xbuf + (size_t)(buf * RT + rt) * TL::SLOTS; };
 
   constexpr bool LDS_STATE = RT > 1;
@@ -382,6 +439,9 @@ __global__ __launch_bounds__(256) void ring_fwd_kernel(RingFwdArgs p) {
   bf16x8 wf[StreamCfg<NC, RT>::PD][StreamCfg<NC, RT>::KG];
   for (int t = 0; t < T; ++t) {
     const int cur = t & 1;
+    if constexpr (STATS) {
+      if (t > 0) flush_loss_sums(t - 1, cur);    // row t-1's shares were left in lsum[(t-1)&1 ^ 1] = lsum[cur]
+    }
     f32x4 acc[RT][NC];
     // next step's gates: loaded now, written to LDS after the products (nothing waits for them before that).
     // Two paired tiles at the widest tiling have no registers to hold them and stage them in one go.
@@ -424,6 +484,7 @@ __global__ __launch_bounds__(256) void ring_fwd_kernel(RingFwdArgs p) {
       const bool live = bt0 + rt < p.nbt;
       rows_store<NC>(p.hist + (size_t)t * B * N, N, B, bq, i0, r);
       if (p.dfrag && live) side_store<NC, f16x4, _Float16>(p.dfrag + side_offset<NC>(t, p.nbt, bt0 + rt, w, lane), d);
+      if constexpr (STATS) publish_loss_sums<NC>(lsum[cur ^ 1][rt], r, lc0, ls0, lcd, lsd, w, q, n);
       if (t + 1 < T) {
         state_put(rt, r);
         write_operand<NC>(xb(cur ^ 1, rt), r, w, q, n);
@@ -433,6 +494,7 @@ __global__ __launch_bounds__(256) void ring_fwd_kernel(RingFwdArgs p) {
     }
     lds_barrier();
   }
+  if constexpr (STATS) flush_loss_sums(T - 1, T & 1);   // the last row's shares: lsum[((T-1)&1) ^ 1]
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -1007,6 +1069,17 @@ static bool step_prefers_wide(int NCv, int nbt, int k) {
   return (long)nbt * NCv > 512;
 }
 
+// Does ring_launch_fwd fill a.loss_stats for this problem?  The persistent kernels do; the step-per-launch ones
+// (wide rings, and the split forward of small batches) do not.
+bool ring_fwd_forms_loss_sums(const RingFwdArgs& a, int NCv) {
+  if (ring_uses_step_kernels(a.N, a.k, NCv, a.nbt)) return false;
+  if (!a.dfrag && !a.rfrag && NCv >= 4 && a.nbt <= 64 && !ring_uses_resident(a.N, a.k)) {
+    const char* v = getenv("RINGATTR_SPLIT_FORWARD");
+    if (!(v && v[0] == '0')) return false;
+  }
+  return true;
+}
+
 hipError_t ring_launch_fwd(const RingFwdArgs& a, int NCv, hipStream_t st) {
   // the kernels write the derivative record and the operand copy together: both or neither
   if ((a.dfrag != nullptr) != (a.rfrag != nullptr)) return hipErrorInvalidValue;
@@ -1028,12 +1101,23 @@ hipError_t ring_launch_fwd(const RingFwdArgs& a, int NCv, hipStream_t st) {
   const int rt = stream_row_tiles(NCv, a.nbt, false);
   hipError_t e = hipErrorInvalidValue;
   if (weights_fit_lds(NCv, a.k, 8 * 1024)) {
+    if (a.loss_stats) {
+      RING_DISPATCH_NC(NCv, RING_DISPATCH_ACT(a.act, if constexpr (NC <= 2)
+          e = launch_stream(ring_fwd_kernel<NC, ACT, 1, true, true>, dim3(a.nbt), stream_lds_bytes<NC, 1>() + packed_weight_bytes<NC>(a.k), st, a)));
+      return e;
+    }
     RING_DISPATCH_NC(NCv, RING_DISPATCH_ACT(a.act, if constexpr (NC <= 2)
-        e = launch_stream(ring_fwd_kernel<NC, ACT, 1, true>, dim3(a.nbt), stream_lds_bytes<NC, 1>() + packed_weight_bytes<NC>(a.k), st, a)));
+        e = launch_stream(ring_fwd_kernel<NC, ACT, 1, true, false>, dim3(a.nbt), stream_lds_bytes<NC, 1>() + packed_weight_bytes<NC>(a.k), st, a)));
+    return e;
+  }
+  if (a.loss_stats) {
+    RING_DISPATCH_NC(NCv, RING_DISPATCH_ACT(a.act, RING_DISPATCH_RT(rt,
+        e = launch_stream(ring_fwd_kernel<NC, ACT, RT, false, true>, dim3((a.nbt + RT - 1) / RT),
+                          stream_lds_bytes<NC, RT>() + fwd_state_lds_bytes<NC, RT>(), st, a))));
     return e;
   }
   RING_DISPATCH_NC(NCv, RING_DISPATCH_ACT(a.act, RING_DISPATCH_RT(rt,
-      e = launch_stream(ring_fwd_kernel<NC, ACT, RT, false>, dim3((a.nbt + RT - 1) / RT),
+      e = launch_stream(ring_fwd_kernel<NC, ACT, RT, false, false>, dim3((a.nbt + RT - 1) / RT),
                         stream_lds_bytes<NC, RT>() + fwd_state_lds_bytes<NC, RT>(), st, a))));
   return e;
 }

@@ -60,6 +60,7 @@ hipError_t ring_launch_pack2(const float* Wo, const float* Wa, int N, int k, int
                              int split_k, float scale0, float shift0, void* out2, int transposed2, int split_k2,
                              float scale2, float shift2, hipStream_t st);
 hipError_t ring_launch_fwd(const RingFwdArgs& a, int NC, hipStream_t st);
+bool ring_fwd_forms_loss_sums(const RingFwdArgs& a, int NC);   // will that launch fill a.loss_stats?
 hipError_t ring_launch_rebuild(const RingFwdArgs& a, int NC, hipStream_t st);
 hipError_t ring_launch_bptt(const RingBpttArgs& a, int NC, hipStream_t st);
 hipError_t ring_launch_dw(const RingDwArgs& a, int NC, hipStream_t st);

@@ -247,8 +247,8 @@ static int fwd_impl(const void* A, const void* Wa, float J0, float J1, const voi
   a.B = batch_size;
   a.nbt = g.nbt;
   a.act = activation_type;
-  // only the weight-resident forward kernel forms the loss head's row sums
-  a.loss_stats = (resident && !ring_uses_step_kernels(N, a_dim, g.NC, g.nbt)) ? loss_stats : nullptr;
+  // the persistent forward kernels form the loss head's row sums themselves
+  a.loss_stats = ring_fwd_forms_loss_sums(a, g.NC) ? loss_stats : nullptr;
   if (stats_done) *stats_done = a.loss_stats != nullptr;
   e = ring_launch_fwd(a, g.NC, st);
   if (e != hipSuccess) return hip_fail(e, "forward launch");
