@@ -255,6 +255,19 @@ class GeneralizedRingAttractor(nn.Module):
         return ring_rnn_cuda_func(action_signal=self.gated_action_signal(action_signal), Wa=self.Wa, J0=self.J0,
                                   J1=self.J1, Wo=self.Wo, r_init=r_init, alpha=0.15, activation=self.activation_name)
 
+    def loss_pair(self, action_signal, target_angle, r_init=None, bump_weight=0.2):
+        """(total, cos_loss, amp_loss, bump_history) of the training objective with gain networks, time loop and loss
+        head chained as HIP operators (see GeneralizedRingAttractorNoGain.loss_pair); the gain networks train through
+        dL/d action_signal, which the fused backward returns."""
+        from .loss_head import ring_rnn_loss_func
+        batch_size, _, action_dim = action_signal.shape
+        assert action_dim == self.action_dim, f"Expected action_dim {self.action_dim}, got {action_dim}"
+        if r_init is None:
+            angle = torch.full((batch_size,), math.pi, device=self.Wo.device)
+            r_init = create_initial_bump(angle, self.num_neurons, device=self.Wo.device)
+        return ring_rnn_loss_func(self.gated_action_signal(action_signal), self.Wa, self.J0, self.J1, self.Wo, r_init,
+                                  0.15, self.activation_name, target_angle, bump_weight)
+
     def forward(self, action_signal, r_init=None):
         bump = self.forward_history(action_signal, r_init).permute(1, 0, 2)
         proj = bump @ self.W_delta7
@@ -323,6 +336,18 @@ class LeakyRingAttractor(nn.Module):
         return ring_rnn_cuda_func(action_signal=self.action_signal(av_signal), Wa=torch.stack([self.Wl, self.Wr]),
                                   J0=self.J0, J1=self.J1, Wo=self.Wo, r_init=r_init, alpha=0.15,
                                   activation=self.activation_name)
+
+    def loss_pair(self, av_signal, target_angle, r_init=None, bump_weight=0.2):
+        """(total, cos_loss, amp_loss, bump_history) of the training objective (train/train_ring_attractor.py:275-298 of
+        the reference: cosine-similarity loss of the read-out + bump_weight * bump-amplitude loss) with gain networks,
+        time loop and loss head as HIP operators; the gain networks train through dL/d action_signal."""
+        from .loss_head import ring_rnn_loss_func
+        batch_size = av_signal.shape[0]
+        if r_init is None:
+            angle = torch.full((batch_size,), math.pi, device=self.Wo.device)
+            r_init = create_initial_bump(angle, self.num_neurons, device=self.Wo.device)
+        return ring_rnn_loss_func(self.action_signal(av_signal), torch.stack([self.Wl, self.Wr]), self.J0, self.J1,
+                                  self.Wo, r_init, 0.15, self.activation_name, target_angle, bump_weight)
 
     def forward(self, av_signal, r_init=None):
         bump = self.forward_history(av_signal, r_init).permute(1, 0, 2)

@@ -433,6 +433,18 @@ def test_gain_network_model_trains_through_the_operator(gpu_device):
         assert np.isfinite(got).all(), n
         assert O.cosine(got, ref) >= 0.999, n
         assert O.max_rel_err(got, ref) <= 2e-2, n
+    # the same objective as chained HIP operators (gain networks, time loop + loss head in one): same loss, and the
+    # same gradients for every parameter, the gain networks' included
+    model.zero_grad()
+    total, _, _, hist = model.loss_pair(av.to(gpu_device), angle.to(gpu_device), r0.to(gpu_device), bump_weight=0.2)
+    total.backward()
+    torch.cuda.synchronize()
+    assert hist.shape == (T, B, N)
+    assert abs(float(total) - float(loss_cpu)) <= 1e-2 * abs(float(loss_cpu))
+    for n, p in model.named_parameters():
+        got, ref = p.grad.cpu().numpy(), want[n].numpy()
+        assert O.cosine(got, ref) >= 0.999, n
+        assert O.max_rel_err(got, ref) <= 2e-2, n
 
 
 @pytest.mark.parametrize("N,k,B,T", [(256, 4, 48, 24), (640, 6, 24, 10)], ids=["n256_k4", "n640_k6_step"])
@@ -472,6 +484,16 @@ def test_general_ring_with_per_channel_gains(N, k, B, T, gpu_device):
     for n, p in model.named_parameters():
         got, ref = p.grad.cpu().numpy(), want[n].numpy()
         assert np.isfinite(got).all(), n
+        assert O.cosine(got, ref) >= 0.999, n
+        assert O.max_rel_err(got, ref) <= 2e-2, n
+    # the same objective with time loop and loss head as one operator
+    model.zero_grad()
+    total, _, _, _ = model.loss_pair(action.to(gpu_device), angle.to(gpu_device), r0.to(gpu_device), bump_weight=0.2)
+    total.backward()
+    torch.cuda.synchronize()
+    assert abs(float(total) - float(loss_cpu)) <= 1e-2 * abs(float(loss_cpu))
+    for n, p in model.named_parameters():
+        got, ref = p.grad.cpu().numpy(), want[n].numpy()
         assert O.cosine(got, ref) >= 0.999, n
         assert O.max_rel_err(got, ref) <= 2e-2, n
 
