@@ -157,6 +157,8 @@ def main():
     ap.add_argument("--prewarm-ms", type=float, default=500.0,
                     help="untimed steps of the workload run for at least this long before --warmup (clock settling)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the host-CPU baseline legs")
+    ap.add_argument("--no-training-step", action="store_true",
+                    help="skip the whole-training-step figure that training workloads report beside the metric")
     ap.add_argument("--cpu-sample-batch", type=int, default=128)
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run three 1 GiB device-to-device copies (known HBM traffic) for scaling rocprofv3's "
@@ -237,6 +239,33 @@ def main():
     dt = time.perf_counter() - t0
     prof = _lib.profile_read()
     _lib.profile_enable(False)
+    training_step = None
+    if mode == "train" and k == 2 and N <= 512 and not args.no_training_step:
+        # Beside the metric (not part of it): a whole training step around the same time loop -- a fresh batch from the
+        # device generator, forward + loss head as one operator, its backward, gradient clipping + Adam.
+        from rnn_train_ring_attractor_amd import FusedClipAdam, generate_inputs, ring_rnn_loss_func
+        opt = FusedClipAdam([Wa, Wo], lr=1e-4, max_norm=1.0)
+
+        def train_once(i):
+            _, angle_i, action_i, r0_i = generate_inputs(1000 + i, B, T, N, k, bump="vm")
+            total = ring_rnn_loss_func(action_i, Wa, cfg["J0"], cfg["J1"], Wo, r0_i, 0.15, cfg["act"], angle_i, 0.2)[0]
+            Wa.grad = None
+            Wo.grad = None
+            total.backward()
+            opt.step()
+            return total
+
+        n_tr = max(20, min(200, args.steps))
+        for i in range(10):
+            train_once(i)
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        for i in range(n_tr):
+            last = train_once(10 + i)
+        torch.cuda.synchronize()
+        training_step = {"ms": (time.perf_counter() - t1) / n_tr * 1e3, "steps": n_tr, "final_loss": float(last),
+                         "what": "device input generator + forward and loss head as one operator + backward + fused "
+                                 "gradient clipping and Adam; reported beside the metric, not part of it"}
     if args.copy_calibration:
         src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
         dst = torch.empty_like(src)
@@ -275,6 +304,8 @@ def main():
                      "algorithmic_bytes_per_launch": (4 * N + 4 * k) * B * T},
         "kernel_ms": kern,
     }
+    if training_step:
+        out["training_step"] = training_step
     if traffic:
         out["traffic_bytes_per_launch"] = traffic
         out["traffic_over_algorithmic"] = sum(traffic.values()) / (bytes_per_ss * B * T) if train else None
