@@ -73,6 +73,19 @@ def test_c_abi_rejects_bad_arguments_with_codes_not_exit():
     assert lib.ringattr_fwd_noalloc(p, p, 0.0, 1.0, p, p, p, 0.15, 512, 8, 4, 16, 0, None, None) == 2
     assert "built-in scratch" in _lib.last_error()
     assert lib.ringattr_fwd_noalloc(p, p, 0.0, 1.0, p, p, p, 0.15, 64, 2, 4, 16, 9, None, None) == 1
+    # forward + loss head in one call: the loss arguments are checked before the time loop is touched
+    fl = ok_args + [0, None, p, 1 << 20]
+    assert lib.ringattr_fwd_loss(*fl, None, None, 0.2, p, p, 1 << 20, None) == 1 and "null" in _lib.last_error()
+    assert lib.ringattr_fwd_loss(*fl, p, None, 0.2, p, p, 16, None) == 2 and "loss workspace" in _lib.last_error()
+    assert lib.ringattr_fwd_loss(*fl, p, None, 0.2, p, p + 4, 1 << 20, None) == 1 and "aligned" in _lib.last_error()
+    # clip + Adam: host-counted steps start at 1; the device-counted variant needs its counter
+    one = (ctypes.c_void_p * 1)(p)
+    numel = (ctypes.c_size_t * 1)(16)
+    adam = [1, one, one, one, one, numel, 1e-3, 0.9, 0.999, 1e-8, 1.0]
+    assert lib.ringattr_clip_adam(*adam, 0, p, 1 << 12, None) == 1 and "counts from 1" in _lib.last_error()
+    assert lib.ringattr_clip_adam_counted(*adam, None, p, 1 << 12, None) == 1 and "step counter" in _lib.last_error()
+    assert lib.ringattr_clip_adam_counted(*adam, p + 2, p, 1 << 12, None) == 1
+    assert lib.ringattr_clip_adam_counted(*adam, p, p, 8, None) == 2 and "workspace" in _lib.last_error()
     with pytest.raises(ValueError):
         _lib.check(1)
     with pytest.raises(RuntimeError):
