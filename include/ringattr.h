@@ -153,9 +153,9 @@ RINGATTR_API int ringattr_bwd_loss(const void* loss_workspace, const void* upstr
                       const void* saved, void* grad_A, void* grad_r_init,
                       void* workspace, size_t workspace_bytes, void* stream);
 
-/* 1 when ringattr_bwd_loss can serve this shape (the persistent kernel families: N <= 512 unless RINGATTR_BLOCK=1
- * moves the shape to the step-per-launch kernels), 0 when the caller has to run ringattr_loss_bwd and hand its
- * [T,B,N] result to ringattr_bwd instead (the host-side operator does).  No counterpart in the reference. */
+/* 1 when ringattr_bwd_loss can serve this shape: every shape the time loop itself accepts (all kernel families form
+ * the loss gradient themselves); 0 only for shapes ringattr_bwd rejects as well.  A caller that finds 0 runs
+ * ringattr_loss_bwd and hands its [T,B,N] result to ringattr_bwd.  No counterpart in the reference. */
 RINGATTR_API int ringattr_bwd_loss_available(int N, int a_dim, int seq_len, int batch_size);
 
 /* Gain networks of the action signal, forward and backward.  Replaces the per-channel nn.Sequential(Linear(1,h), GELU,

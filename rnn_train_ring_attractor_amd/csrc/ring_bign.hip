@@ -165,6 +165,7 @@ __global__ __launch_bounds__(256) void ring_wide_fwd_kernel(RingFwdArgs p, int N
 // One BPTT step t: G = grad_output[t] + carry_in, g = (alpha F') * G (operand, all neurons, every workgroup of the batch
 // tile), carry_out = (1-alpha) G + J0 sum(g) + J1 (g Wo) + sum_c A_c (g Wa_c) for the workgroup's own 256 neurons.
 // carry_in == nullptr at the last time step (zero carry); at t == 0 the host points carry_out at grad_r_init or scratch.
+template <bool LOSS>
 __global__ __launch_bounds__(256) void ring_wide_bptt_kernel(RingBpttArgs p, int NC, int t, const float* carry_in,
                                                              float* carry_out, int xcd_map) {
   extern __shared__ __attribute__((aligned(16))) char wide_lds[];
@@ -177,13 +178,16 @@ __global__ __launch_bounds__(256) void ring_wide_bptt_kernel(RingBpttArgs p, int
   const int N = p.N, B = p.B, T = p.T, NPAD = 64 * NC;
   const bool staged = p.k <= BN_GATE_KMAX;
   const size_t rows_pad = (size_t)16 * p.nbt;
-  const float* gout = p.grad_out + (size_t)t * B * N;
+  const float* gout = LOSS ? nullptr : p.grad_out + (size_t)t * B * N;
   const _Float16* drow = p.dfrag + (size_t)t * rows_pad * NPAD;
+  // LOSS: grad_output is not read; it is formed from the state history and the loss head's row coefficients
+  const float up = LOSS ? (p.loss_upstream ? p.loss_upstream[0] : 1.f) * p.loss_inv_rows : 0.f;
 
   // g of (row, j..j+3): carry rows live in a padded [16*nbt][NPAD] buffer
   auto g4 = [&](int row, int j, f32x4& G) {
     const int b = 16 * bt + row;
-    G = load4_masked(gout, N, B, b, j);
+    if constexpr (LOSS) G = loss_grad4(p, t, b, j, up);
+    else G = load4_masked(gout, N, B, b, j);
     if (carry_in) {
       const f32x4 cin = *reinterpret_cast<const f32x4*>(carry_in + ((size_t)16 * bt + row) * NPAD + j);
       G += cin;
@@ -287,16 +291,34 @@ hipError_t ring_launch_wide_fwd(const RingFwdArgs& a, int NC, bool rebuild, int 
 }
 
 // carry: 2 * 16 * nbt * NPAD floats of scratch (ring_wide_carry_bytes), used as two alternating buffers
+__global__ __launch_bounds__(256) void ring_trig_table_kernel(float* out, int N, int NPAD) {
+  const int j = blockIdx.x * 256 + threadIdx.x;
+  if (j >= NPAD) return;
+  float s = 0.f, c = 0.f;
+  if (j < N) sincosf(6.283185307179586f * (float)j / (float)N, &s, &c);
+  out[2 * j] = c;
+  out[2 * j + 1] = s;
+}
+
+hipError_t ring_launch_trig_table(float* out, int N, int NPAD, hipStream_t st) {
+  hipLaunchKernelGGL(ring_trig_table_kernel, dim3((NPAD + 255) / 256), dim3(256), 0, st, out, N, NPAD);
+  return hipGetLastError();
+}
+
 hipError_t ring_launch_wide_bptt(const RingBpttArgs& a, int NC, float* carry, hipStream_t st) {
   const size_t dyn = wide_lds_bytes(NC);
-  hipError_t e = wide_attr(ring_wide_bptt_kernel, dyn);
+  const bool loss = a.loss_coef != nullptr;
+  if (loss && (!a.loss_trig || !a.hist)) return hipErrorInvalidValue;
+  if (!loss && !a.grad_out) return hipErrorInvalidValue;
+  hipError_t e = loss ? wide_attr(ring_wide_bptt_kernel<true>, dyn) : wide_attr(ring_wide_bptt_kernel<false>, dyn);
   if (e != hipSuccess) return e;
   const size_t half = (size_t)16 * a.nbt * 64 * NC;
   const unsigned ncb = (unsigned)(NC / 4);
   for (int t = a.T - 1, u = 0; t >= 0; --t, ++u) {
     const float* cin = (u == 0) ? nullptr : carry + (size_t)((u - 1) & 1) * half;
     float* cout = carry + (size_t)(u & 1) * half;
-    hipLaunchKernelGGL(ring_wide_bptt_kernel, dim3(a.nbt, ncb), dim3(256), dyn, st, a, NC, t, cin, cout, step_xcd_map());
+    if (loss) hipLaunchKernelGGL(ring_wide_bptt_kernel<true>, dim3(a.nbt, ncb), dim3(256), dyn, st, a, NC, t, cin, cout, step_xcd_map());
+    else hipLaunchKernelGGL(ring_wide_bptt_kernel<false>, dim3(a.nbt, ncb), dim3(256), dyn, st, a, NC, t, cin, cout, step_xcd_map());
     e = hipGetLastError();
     if (e != hipSuccess) return e;
   }

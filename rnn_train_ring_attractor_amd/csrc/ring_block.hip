@@ -236,7 +236,7 @@ __global__ __launch_bounds__(256) void ring_block_fwd_kernel(RingFwdArgs p, int 
 }
 
 // One BPTT step t for RT batch tiles x 64*TPW neurons per workgroup (see ring_wide_bptt_kernel for the recurrence).
-template <int RT, int TPW>
+template <int RT, int TPW, bool LOSS>
 __global__ __launch_bounds__(256) void ring_block_bptt_kernel(RingBpttArgs p, int NC, int t, const float* carry_in,
                                                               float* carry_out, int xcd_map) {
   extern __shared__ __attribute__((aligned(16))) char block_lds[];
@@ -250,8 +250,10 @@ __global__ __launch_bounds__(256) void ring_block_bptt_kernel(RingBpttArgs p, in
   const bool staged = p.k <= BN_GATE_KMAX;
   float* gl = reinterpret_cast<float*>(xb + (size_t)RT * slots);
   const size_t rows_pad = (size_t)16 * p.nbt;
-  const float* gout = p.grad_out + (size_t)t * B * N;
+  const float* gout = LOSS ? nullptr : p.grad_out + (size_t)t * B * N;
   const _Float16* drow = p.dfrag + (size_t)t * rows_pad * NPAD;
+  // LOSS: grad_output is not read; it is formed from the state history and the loss head's row coefficients
+  const float up = LOSS ? (p.loss_upstream ? p.loss_upstream[0] : 1.f) * p.loss_inv_rows : 0.f;
 
   // g of (row within the block, j..j+V-1); carry rows live in a padded [16*nbt][NPAD] buffer.  Rows of batch tiles
   // past the last one (a partial last block) read as zero.
@@ -259,7 +261,8 @@ __global__ __launch_bounds__(256) void ring_block_bptt_kernel(RingBpttArgs p, in
     const size_t prow = (size_t)16 * bt0 + row;
     G = f32x4{0.f, 0.f, 0.f, 0.f};
     if (prow >= rows_pad) return G;
-    G = load4_masked(gout, N, B, (int)prow, j);
+    if constexpr (LOSS) G = loss_grad4(p, t, (int)prow, j, up);
+    else G = load4_masked(gout, N, B, (int)prow, j);
     if (carry_in) G += *reinterpret_cast<const f32x4*>(carry_in + prow * NPAD + j);
     const f16x4 d = *reinterpret_cast<const f16x4*>(drow + prow * NPAD + j);
     return f32x4{(float)d[0] * G[0], (float)d[1] * G[1], (float)d[2] * G[2], (float)d[3] * G[3]};
@@ -480,10 +483,10 @@ hipError_t ring_launch_block_fwd(const RingFwdArgs& a, int NC, bool rebuild, hip
   }
 }
 
-template <int RT, int TPW>
+template <int RT, int TPW, bool LOSS>
 static hipError_t block_bptt_shape(const RingBpttArgs& a, int NC, float* carry, hipStream_t st) {
   const size_t dyn = block_lds_bytes(NC, RT, a.k);
-  hipError_t e = block_attr(ring_block_bptt_kernel<RT, TPW>, dyn);
+  hipError_t e = block_attr(ring_block_bptt_kernel<RT, TPW, LOSS>, dyn);
   if (e != hipSuccess) return e;
   const size_t half = (size_t)16 * a.nbt * 64 * NC;
   const dim3 grid((a.nbt + RT - 1) / RT, NC / TPW);
@@ -491,7 +494,7 @@ static hipError_t block_bptt_shape(const RingBpttArgs& a, int NC, float* carry, 
   for (int t = a.T - 1, u = 0; t >= 0; --t, ++u) {
     const float* cin = (u == 0) ? nullptr : carry + (size_t)((u - 1) & 1) * half;
     float* cout = carry + (size_t)(u & 1) * half;
-    hipLaunchKernelGGL((ring_block_bptt_kernel<RT, TPW>), grid, dim3(256), dyn, st, a, NC, t, cin, cout, xm);
+    hipLaunchKernelGGL((ring_block_bptt_kernel<RT, TPW, LOSS>), grid, dim3(256), dyn, st, a, NC, t, cin, cout, xm);
     e = hipGetLastError();
     if (e != hipSuccess) return e;
   }
@@ -503,8 +506,14 @@ hipError_t ring_launch_block_bptt(const RingBpttArgs& a, int NC, float* carry, h
   if (NC % 2 != 0) return hipErrorInvalidValue;
   int rt, tpw;
   ring_block_geometry(NC, a.nbt, a.k, &rt, &tpw);
-  if (rt == 2) return tpw == 2 ? block_bptt_shape<2, 2>(a, NC, carry, st) : block_bptt_shape<2, 1>(a, NC, carry, st);
-  return tpw == 2 ? block_bptt_shape<1, 2>(a, NC, carry, st) : block_bptt_shape<1, 1>(a, NC, carry, st);
+  if (a.loss_coef) {
+    if (!a.loss_trig || !a.hist) return hipErrorInvalidValue;
+    if (rt == 2) return tpw == 2 ? block_bptt_shape<2, 2, true>(a, NC, carry, st) : block_bptt_shape<2, 1, true>(a, NC, carry, st);
+    return tpw == 2 ? block_bptt_shape<1, 2, true>(a, NC, carry, st) : block_bptt_shape<1, 1, true>(a, NC, carry, st);
+  }
+  if (!a.grad_out) return hipErrorInvalidValue;
+  if (rt == 2) return tpw == 2 ? block_bptt_shape<2, 2, false>(a, NC, carry, st) : block_bptt_shape<2, 1, false>(a, NC, carry, st);
+  return tpw == 2 ? block_bptt_shape<1, 2, false>(a, NC, carry, st) : block_bptt_shape<1, 1, false>(a, NC, carry, st);
 }
 
 // a.grad_A, a.gfrag (complete), a.hist, a.r_init; Wf: forward-orientation packed weights (matrix 0 is not read)

@@ -1152,7 +1152,7 @@ hipError_t ring_launch_bptt(const RingBpttArgs& a, int NCv, hipStream_t st) {
   ProfScope prof(3, st);
   hipError_t e = hipErrorInvalidValue;
   if (ring_uses_step_kernels(a.N, a.k, NCv, a.nbt)) {
-    if (a.grad_A || a.loss_coef || !a.wide_carry) return hipErrorInvalidValue;   // the C ABI rejects these before
+    if (a.grad_A || !a.wide_carry) return hipErrorInvalidValue;   // (dL/dA comes from a pass of its own, see the C ABI)
     return step_prefers_wide(NCv, a.nbt, a.k) ? ring_launch_wide_bptt(a, NCv, a.wide_carry, st)
                                   : ring_launch_block_bptt(a, NCv, a.wide_carry, st);
   }

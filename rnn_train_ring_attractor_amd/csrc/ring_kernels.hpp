@@ -35,6 +35,7 @@ struct RingBpttArgs {
   const ring_f32x4* loss_coef;
   const float* loss_upstream;   // one float on the device, or null for 1
   float loss_inv_rows;          // 1 / (T * B)
+  const float* loss_trig = nullptr;   // step-per-launch kernels with loss_coef: (cos, sin)(2 pi j / N) pairs, j < NPAD
   float* wide_carry;     // N > 512 only: 2 x [16*nbt][NPAD] fp32 scratch for the carried gradient between step launches
   float J0, J1, alpha;
   int N, k, T, B, nbt;
@@ -83,6 +84,8 @@ hipError_t ring_launch_block_fwd(const RingFwdArgs& a, int NC, bool rebuild, hip
 hipError_t ring_launch_block_bptt(const RingBpttArgs& a, int NC, float* carry, hipStream_t st);
 bool ring_block_many_matrices(int k);   // the weight stream dominates a step: the block kernels lead at any batch size
 // dL/dA of the step-per-launch families: a separate pass after the BPTT steps (Wf: forward-orientation packed weights)
+// (cos, sin)(2 pi j / N) for j < N, zero up to NPAD: what the step-per-launch BPTT kernels read with the fused loss head
+hipError_t ring_launch_trig_table(float* out, int N, int NPAD, hipStream_t st);
 hipError_t ring_launch_block_grad_A(const RingBpttArgs& a, const void* Wf, int NC, hipStream_t st);
 // which kernel family runs a problem with a saved record: 0 persistent, 1 step-per-launch (wide or block)
 bool ring_uses_step_kernels(int N, int k, int NC, int nbt);

@@ -74,6 +74,26 @@ __device__ __forceinline__ f32x4 load4_masked(const float* slab, int N, int B, i
   return v;
 }
 
+// The loss head's gradient in place of grad_output (step-per-launch BPTT kernels): four neurons j..j+3 of history row
+// (t, b),  up * (kc cos(phi_j) + ks sin(phi_j) + beta sign(r_j)),  (kc, ks, beta) = loss_coef[t * B + b], the state r
+// read where grad_output would have been (same bytes), (cos, sin) from the table of ring_launch_trig_table.
+__device__ __forceinline__ f32x4 loss_grad4(const RingBpttArgs& p, int t, int b, int j, float up) {
+  f32x4 g = {0.f, 0.f, 0.f, 0.f};
+  if (b >= p.B || j >= p.N) return g;
+  const f32x4 c = p.loss_coef[(size_t)t * p.B + b];
+  const f32x4 r = load4_masked(p.hist + (size_t)t * p.B * p.N, p.N, p.B, b, j);
+  const float kc = c[0] * up, ks = c[1] * up, beta = c[2] * up;
+  const f32x4 t0 = *reinterpret_cast<const f32x4*>(p.loss_trig + 2 * j);        // j is a multiple of 4
+  const f32x4 t1 = *reinterpret_cast<const f32x4*>(p.loss_trig + 2 * j + 4);
+  const float cs[4] = {t0[0], t0[2], t1[0], t1[2]}, sn[4] = {t0[1], t0[3], t1[1], t1[3]};
+#pragma unroll
+  for (int x = 0; x < 4; ++x) {
+    const float sb = r[x] > 0.f ? beta : (r[x] < 0.f ? -beta : 0.f);              // beta * sign(r), sign(0) = 0
+    g[x] = j + x < p.N ? fmaf(kc, cs[x], fmaf(ks, sn[x], sb)) : 0.f;
+  }
+  return g;
+}
+
 __device__ __forceinline__ void store4_masked(float* slab, int N, int B, int b, int j, f32x4 v) {
   if (b >= B || j >= N) return;
   float* dst = slab + (size_t)b * N + j;

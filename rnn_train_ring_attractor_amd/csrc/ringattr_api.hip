@@ -40,6 +40,7 @@ struct Geo {
   size_t pair_bytes;     // one bf16 operand copy, time steps paired: [ceil(T/2)*2,16*nbt,NPAD]
   size_t partial_bytes;  // split-K partials of the weight gradient
   size_t carry_bytes;    // N > 512: the carried gradient between the per-step BPTT launches
+  size_t trig_bytes;     // step-per-launch kernels with the fused loss head: (cos, sin) of every neuron's angle
 };
 
 // Smallest supported neuron tiling with 64*NC >= N: the persistent kernels up to N = 512, the step-per-launch
@@ -78,6 +79,7 @@ int make_geo(int N, int k, int T, int B, Geo& g) {
   g.nz = ring_dw_tiled_applicable(nc) ? ring_dw_tiled_nz(nc, k, nchunk) : (int)nz;
   g.partial_bytes = align_up((size_t)g.nz * (1 + k) * g.NPAD * g.NPAD * 4);
   g.carry_bytes = nc >= 4 ? align_up(ring_wide_carry_bytes(nc, g.nbt)) : 0;   // (small; sized whichever family runs)
+  g.trig_bytes = nc >= 4 ? align_up((size_t)g.NPAD * 2 * sizeof(float)) : 0;
   return RINGATTR_OK;
 }
 
@@ -162,7 +164,7 @@ size_t ringattr_fwd_workspace_bytes(int N, int a_dim, int seq_len, int batch_siz
 size_t ringattr_bwd_workspace_bytes(int N, int a_dim, int seq_len, int batch_size, int have_saved) {
   Geo g;
   if (make_geo(N, a_dim, seq_len, batch_size, g) != RINGATTR_OK) return 0;
-  size_t s = g.wpack_bytes + g.pair_bytes + g.partial_bytes + g.carry_bytes;
+  size_t s = g.wpack_bytes + g.pair_bytes + g.partial_bytes + g.carry_bytes + g.trig_bytes;
   if (!have_saved) s += g.wpack_bytes + g.side_bytes + g.pair_bytes;
   return s;
 }
@@ -309,8 +311,7 @@ int ringattr_bwd_loss(const void* loss_workspace, const void* upstream, const vo
 
 int ringattr_bwd_loss_available(int N, int a_dim, int seq_len, int batch_size) {
   Geo g;
-  if (make_geo(N, a_dim, seq_len, batch_size, g) != RINGATTR_OK) return 0;
-  return ring_uses_step_kernels(N, a_dim, g.NC, g.nbt) ? 0 : 1;
+  return make_geo(N, a_dim, seq_len, batch_size, g) == RINGATTR_OK ? 1 : 0;
 }
 
 static int bwd_impl(const char* who, const void* grad_output, const void* loss_workspace, const void* upstream, const void* A,
@@ -327,9 +328,6 @@ static int bwd_impl(const char* who, const void* grad_output, const void* loss_w
   if (grad_A && (size_t)2 * a_dim * 64 * sizeof(float) > 24 * 1024)
     return fail(RINGATTR_ERR_INVALID, "%s: grad_A is supported for a_dim <= 48 (got %d)", who, a_dim);
   const bool step_family = ring_uses_step_kernels(N, a_dim, g.NC, g.nbt);
-  if (step_family && loss_workspace)
-    return fail(RINGATTR_ERR_INVALID, "%s: the fused loss backward is not available on the step-per-launch kernels "
-                "(N = %d > 512, or RINGATTR_BLOCK=1); run ringattr_loss_bwd and pass its result to ringattr_bwd", who, N);
   if (step_family && grad_A && seq_len > 65535)
     return fail(RINGATTR_ERR_INVALID, "%s: grad_A on the step-per-launch kernels supports seq_len <= 65535", who);
   if (!aligned16(grad_output) || !aligned16(A) || !aligned16(Wa) || !aligned16(Wo) || !aligned16(bump_history) ||
@@ -351,6 +349,8 @@ static int bwd_impl(const char* who, const void* grad_output, const void* loss_w
   ws += g.partial_bytes;
   float* carry = g.carry_bytes ? (float*)ws : nullptr;
   ws += g.carry_bytes;
+  float* trig = g.trig_bytes ? (float*)ws : nullptr;
+  ws += g.trig_bytes;
 
   const _Float16* dfrag;
   const __bf16* rfrag;
@@ -422,6 +422,12 @@ static int bwd_impl(const char* who, const void* grad_output, const void* loss_w
   b.loss_coef = loss_workspace ? ring_loss_row_coefficients(loss_workspace) : nullptr;
   b.loss_upstream = (const float*)upstream;
   b.loss_inv_rows = 1.f / ((float)seq_len * (float)batch_size);
+  if (step_family && loss_workspace) {
+    if (!trig) return fail(RINGATTR_ERR_INVALID, "%s: no room for the angle table in this geometry", who);
+    e = ring_launch_trig_table(trig, N, g.NPAD, st);
+    if (e != hipSuccess) return hip_fail(e, "angle table launch");
+    b.loss_trig = trig;
+  }
   b.J0 = J0;
   b.J1 = J1;
   b.alpha = alpha;

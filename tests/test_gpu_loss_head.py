@@ -179,3 +179,37 @@ def test_one_operator_without_a_backward_returns_the_same_losses(B, N, gpu_devic
     for a, b in zip(with_grad, without):
         assert torch.equal(a.detach(), b)
     assert not without[0].requires_grad
+
+
+@pytest.mark.parametrize("family", ["wide", "block11", "block22"])
+@pytest.mark.parametrize("B,T,k,N,act", [(40, 5, 3, 640, "silu"), (19, 4, 2, 1100, "tanh")], ids=["n640_k3", "n1100_ragged"])
+def test_loss_gradient_inside_the_step_per_launch_backward(B, T, k, N, act, family, gpu_device, monkeypatch):
+    """Wide rings: each of the step-per-launch BPTT kernels forms the loss gradient itself (state history rows, the
+    loss head's row coefficients and a table of the neurons' angles in place of grad_output); against the chain that
+    writes the [T,B,N] gradient and reads it back."""
+    from rnn_train_ring_attractor_amd import ring_loss_pair, ring_rnn_cuda_func, ring_rnn_loss_func
+    from tests.ring_cases import make_problem
+    print(f"[case] fused loss backward, {family} kernels, B={B} T={T} k={k} N={N} {act}", flush=True)
+    if family == "wide":
+        monkeypatch.setenv("RINGATTR_WIDE", "1")
+    else:
+        monkeypatch.setenv("RINGATTR_WIDE", "0")
+        monkeypatch.setenv("RINGATTR_BLOCK_SHAPE", family[-2:])
+    p = make_problem(41 + N, B, T, k, N, action="dense")
+    t = lambda x: torch.tensor(np.ascontiguousarray(x), device=gpu_device)
+    angle = t(p["angle"])
+    res = {}
+    for fused in (True, False):
+        A = t(p["A"]).requires_grad_(True)
+        Wa, Wo, r0 = t(p["Wa"]).requires_grad_(True), t(p["Wo"]).requires_grad_(True), t(p["r0"]).requires_grad_(True)
+        if fused:
+            total = ring_rnn_loss_func(A, Wa, -0.05, 0.4, Wo, r0, 0.15, act, angle, 0.2)[0]
+        else:
+            total = ring_loss_pair(ring_rnn_cuda_func(A, Wa, -0.05, 0.4, Wo, r0, 0.15, act), angle, 0.2)[0]
+        (1.7 * total).backward()
+        torch.cuda.synchronize()
+        res[fused] = [float(total)] + [x.grad.cpu().numpy() for x in (Wo, Wa, r0, A)]
+    assert abs(res[True][0] - res[False][0]) <= 2e-6 * max(1.0, abs(res[False][0]))
+    for name, a, b in zip(("grad_Wo", "grad_Wa", "grad_r_init", "grad_A"), res[True][1:], res[False][1:]):
+        assert np.isfinite(a).all() and np.abs(b).max() > 0, name
+        assert O.max_rel_err(a, b) <= 2e-3 and O.cosine(a, b) >= 0.99999, name
