@@ -100,6 +100,44 @@ def test_headline_size_properties(gpu_device):
     assert torch.isfinite(full[0]).all()
 
 
+def test_headline_size_training_objective_as_one_operator(gpu_device):
+    """N=256, B=4096, T=120, gelu: time loop and loss head as one operator (row sums formed inside the forward kernel,
+    loss gradient inside the BPTT kernel) against the two-operator chain at the full size; the fp64 oracle prices a
+    64-row slice of the loss; sample independence: the loss of the full batch is the mean of its shards' losses."""
+    from rnn_train_ring_attractor_amd import ring_loss_pair, ring_rnn_cuda_func, ring_rnn_loss_func
+    print("[case] headline one-operator objective N=256 B=4096 T=120 gelu", flush=True)
+    B, T, k, N = 4096, 120, 2, 256
+    J0, J1 = -1.0 / N, 1.0
+    p = make_problem(43, B, T, k, N, bump="vm")
+    A, r0, angle = _t(p["A"], gpu_device), _t(p["r0"], gpu_device), _t(p["angle"], gpu_device)
+
+    def run(fused, rows=slice(0, B)):
+        Wa = _t(p["Wa"], gpu_device).requires_grad_(True)
+        Wo = _t(p["Wo"], gpu_device).requires_grad_(True)
+        a, r, ang = A[rows].contiguous(), r0[rows].contiguous(), angle[rows].contiguous()
+        if fused:
+            total = ring_rnn_loss_func(a, Wa, J0, J1, Wo, r, 0.15, "gelu", ang, 0.2)[0]
+        else:
+            total = ring_loss_pair(ring_rnn_cuda_func(a, Wa, J0, J1, Wo, r, 0.15, "gelu"), ang, 0.2)[0]
+        total.backward()
+        return float(total.detach()), Wa.grad, Wo.grad
+
+    one, two, again = run(True), run(False), run(True)
+    assert np.isfinite(one[0]) and torch.isfinite(one[1]).all() and float(one[2].abs().max()) > 0
+    assert one[0] == again[0] and torch.equal(one[1], again[1]) and torch.equal(one[2], again[2])   # repeatable
+    assert abs(one[0] - two[0]) <= 2e-6 * max(1.0, abs(two[0]))
+    for a, b in zip(one[1:], two[1:]):
+        assert O.max_rel_err(a.cpu().numpy(), b.cpu().numpy()) <= 2e-3 and O.cosine(a.cpu().numpy(), b.cpu().numpy()) >= 0.99999
+    sl = slice(2048, 2112)
+    ref, _ = O.forward_dense(p["A"][sl], p["Wa"], J0, J1, p["Wo"], p["r0"][sl], 0.15, "gelu")
+    want = O.loss_pair_rank2(ref, p["angle"][sl], 0.2, None)[0]
+    part = run(True, sl)
+    assert abs(part[0] - want) <= 1e-2 * max(1.0, abs(want))
+    lo, hi = run(True, slice(0, B // 2)), run(True, slice(B // 2, B))
+    assert abs(0.5 * (lo[0] + hi[0]) - one[0]) <= 1e-5 * max(1.0, abs(one[0]))
+    assert O.max_rel_err((0.5 * (lo[2] + hi[2])).cpu().numpy(), one[2].cpu().numpy()) <= 1e-4
+
+
 def test_long_sequence_shape_at_full_size(gpu_device):
     """N=512, B=8192, T=512, tanh at its real size (inputs generated on the device): bitwise repeatable, a 32-row
     slice run alone reproduces its rows of the full batch bit for bit and agrees with the fp64 oracle, the
