@@ -140,6 +140,11 @@ class AVIntegrationDataset(torch.utils.data.Dataset):
         self.current_index = 0
         self.shuffled_indices = torch.randperm(self.num_samples, device=self.device)
 
+    def get_memory_usage_mb(self):
+        """Megabytes held by the pre-generated trials (utils/generate_av_integration_data.py:206-211)."""
+        return (self.av_data.element_size() * self.av_data.nelement()
+                + self.angle_data.element_size() * self.angle_data.nelement()) / (1024 * 1024)
+
     def generate_batch(self, batch_size):
         if batch_size > self.num_samples:
             raise ValueError(f"Batch size {batch_size} cannot be larger than dataset size {self.num_samples}")

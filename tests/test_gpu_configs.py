@@ -693,6 +693,28 @@ def test_training_and_evaluation_entry_point(gpu_device):
     assert abs(float(res["aligned_target"][0, 0]) - np.pi) <= 1e-5
 
 
+def test_reference_sanity_check_and_gain_model_entry_points(gpu_device):
+    """The reference's own acceptance bound (train/train_ring_attractor.py:327-348: fixed cosine weights, N = 360, gelu,
+    cosine-similarity loss below 0.5) through the HIP path, and its two gain-model training entry points
+    (train.train_ring_attractor / train.train_general_ring_attractor `run_training_and_evaluation`) at a reduced size,
+    with the torch loss chain and with the objective as chained HIP operators."""
+    import train.train_general_ring_attractor as TG
+    import train.train_ring_attractor as TL
+    print("[case] sanity check N=360 gelu; gain-model training entry points N=120 B=32 T=40", flush=True)
+    assert TL.sanity_check_loss(batch_size=128, seq_len=120) < 0.5
+    small = dict(num_neurons=120, training_steps=24, batch_size=32, seq_len=40, lr=3e-3, log_every=0, eval_seq_len=50)
+    for fused in (False, True):
+        model, hist, ev = TL.run_training_and_evaluation(fused=fused, sanity_check=False, **small)
+        assert len(hist) == 24 and all(np.isfinite(hist)) and np.mean(hist[-4:]) < np.mean(hist[:4])
+        assert ev["decoded_pv"].shape == (1, 50) and np.isfinite(ev["mean_abs_error_pv"])
+        assert [n for n, _ in model.named_parameters()][:3] == ["Wo", "Wl", "Wr"]
+        model, hist, ev = TG.run_training_and_evaluation(action_dim=2, fused=fused, **small)
+        assert len(hist) == 24 and all(np.isfinite(hist)) and np.mean(hist[-4:]) < np.mean(hist[:4])
+        assert ev["cos_activity"].shape == (1, 50, 120) and len(model.gain_nets) == 2
+    with pytest.raises(ValueError):
+        TG.run_training_and_evaluation(action_dim=3, **small)
+
+
 def test_reference_signature_entry_points(gpu_device):
     """fwd_cuda / bwd_cuda with the reference's exact C argument lists (null stream, own scratch)."""
     import ctypes

@@ -20,6 +20,11 @@ def test_module_paths_and_star_import_export_the_reference_names():
                  "decode_angle_from_population_vector", "decode_angle_from_argmax", "plot_ring_matrices"):
         assert callable(getattr(T, name))
     from utils.generate_av_integration_data import AVIntegrationDataset  # noqa: F401
+    # the training entry points of the three models, each under the reference's module path and name
+    import train.train_general_ring_attractor as TG
+    import train.train_general_ring_no_gain as TN
+    assert callable(T.run_training_and_evaluation) and callable(TG.run_training_and_evaluation)
+    assert callable(TN.run_training_and_evaluation)
 
 
 def test_helpers_match_oracle():
@@ -55,6 +60,7 @@ def test_dataset_structure_and_batch_cursor():
     assert set(nz.tolist()) <= {36 - int(np.float32(36) * np.float32(z)) for z in (0.2, 0.5, 0.8)}
     seen = torch.cat([ds.generate_batch(20)[0] for _ in range(2)])
     assert seen.shape == (40, 40)
+    assert abs(ds.get_memory_usage_mb() - 2 * 50 * 40 * 4 / 2 ** 20) < 1e-9
     b3 = ds.generate_batch(20)[0]              # wraps around the 50 samples
     assert b3.shape == (20, 40)
     with pytest.raises(ValueError):
