@@ -15,7 +15,8 @@
  *   r_init       [B,N]     initial state (never modified)
  *   bump_history [T,B,N]   state after every step (forward output)
  *   grad_output  [T,B,N]   dL/d bump_history
- *   grad_Wa [k,N,N], grad_Wo [N,N]   ACCUMULATED into (caller zeroes them)
+ *   grad_Wa [k,N,N], grad_Wo [N,N]   accumulate = 1: added to (the reference's contract, cpp/ring_rnn_cuda.py:98-99:
+ *                                    the caller zeroes them); accumulate = 0: overwritten (may be uninitialised)
  *
  * Math per sample b and step t (r_prev = r_init at t = 0):
  *   re  = J0*sum_j r_prev[j] + J1*(Wo r_prev) + sum_c A[b,t,c]*(Wa[c] r_prev)
