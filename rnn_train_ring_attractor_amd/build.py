@@ -72,5 +72,26 @@ def build_library(verbose: bool = False, extra_flags=(), out_path: str = LIB_PAT
     return out_path
 
 
+C_CONSUMER_SRC = os.path.join(os.path.dirname(PKG_DIR), "tests", "c_abi", "ring_c_consumer.c")
+C_CONSUMER_LIB = os.path.join(os.path.dirname(PKG_DIR), "tests", "c_abi", "libring_c_consumer.so")
+
+
+def build_c_consumer() -> str:
+    """The plain-C consumer of the C ABI that the GPU tests run in-process: C99, compiled by the host C compiler
+    against include/ringattr.h, the built library and the HIP runtime (no C++, no torch)."""
+    cc = shutil.which("gcc") or shutil.which("cc")
+    if not cc:
+        raise RuntimeError("no C compiler found for tests/c_abi/ring_c_consumer.c")
+    rocm = os.environ.get("ROCM_PATH", "/opt/rocm")
+    cmd = [cc, "-std=c99", "-Wall", "-Wextra", "-O2", "-fPIC", "-shared", "-fvisibility=hidden", f"-I{INCLUDE}",
+           f"-I{rocm}/include", C_CONSUMER_SRC, "-o", C_CONSUMER_LIB, f"-L{PKG_DIR}", "-lringattr", f"-L{rocm}/lib",
+           "-lamdhip64", "-lm", "-Wl,-rpath,$ORIGIN/../../rnn_train_ring_attractor_amd", f"-Wl,-rpath,{rocm}/lib"]
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError("C consumer build failed:\n" + " ".join(cmd) + "\n" + proc.stdout + proc.stderr)
+    return C_CONSUMER_LIB
+
+
 if __name__ == "__main__":
     print(build_library(verbose=True, extra_flags=sys.argv[1:]))
+    print(build_c_consumer())
