@@ -120,66 +120,70 @@ __global__ __launch_bounds__(256) void ring_loss_stats_kernel(const float* __res
   }
 }
 
-// Per batch row: target amplitude, sum over t of the deviations (what flows into the target) and of their
-// squares.  A workgroup takes 32 batch rows; eight threads per row stride over t and are combined in a
-// fixed order.
-__global__ __launch_bounds__(256) void ring_loss_rows_kernel(const f32x4* __restrict__ stats,
-                                                             const float* __restrict__ target_amp, float* __restrict__ tgt,
-                                                             float* __restrict__ dsum, float* __restrict__ sq, int T, int B) {
-  __shared__ float pd[8][32], ps[8][32];
-  const int bi = threadIdx.x & 31, tl = threadIdx.x >> 5;
-  const int b = blockIdx.x * 32 + bi, bc = b < B ? b : B - 1;
-  const float target = target_amp ? target_amp[bc] : stats[bc][2];   // row t = 0 is stats[0*B + b]
-  float d = 0.f, s = 0.f;
-  for (int t = tl; t < T; t += 8) {
-    const float dev = stats[(size_t)t * B + bc][2] - target;
-    d += dev;
-    s = fmaf(dev, dev, s);
-  }
-  pd[tl][bi] = d;
-  ps[tl][bi] = s;
-  __syncthreads();
-  if (tl == 0 && b < B) {
-    float dd = 0.f, ss = 0.f;
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      dd += pd[j][bi];
-      ss += ps[j][bi];
-    }
-    tgt[b] = target;
-    dsum[b] = dd;
-    sq[b] = ss;
-  }
-}
-
-// One thread per (t, b): the decode and everything transcendental.  Replaces stats[row] by the row's
-// gradient coefficients (kc, ks, beta, theta), all still without the 1/(T*B) and upstream factors:
-//   d total / d r_i = kc cos(phi_i) + ks sin(phi_i) + beta sign(r_i).
-// partial[block] = sum of the block's cos-sim terms (fixed order).
+// Per batch row, then per (t, b), in one launch.  A workgroup takes 32 batch rows at a time (eight threads per row
+// stride over t):
+//  1. target amplitude of the row, sum over t of the deviations (what flows into the target) and of their squares,
+//     combined over the eight threads in a fixed order;
+//  2. the decode and everything transcendental for the same rows: stats[row] is replaced by the row's gradient
+//     coefficients (kc, ks, beta, theta), all still without the 1/(T*B) and upstream factors:
+//       d total / d r_i = kc cos(phi_i) + ks sin(phi_i) + beta sign(r_i).
+// partial[block] = sum of the block's cos-sim terms (fixed order); sq[b] = the row's sum of squared deviations.
 __global__ __launch_bounds__(256) void ring_loss_decode_kernel(f32x4* __restrict__ stats, const float* __restrict__ angle,
-                                                               const float* __restrict__ tgt, const float* __restrict__ dsum,
+                                                               const float* __restrict__ target_amp, float* __restrict__ sq,
                                                                float* __restrict__ partial, LossConsts k, float bump_weight,
-                                                               int own_target, int T, int B) {
+                                                               int T, int B) {
+  __shared__ float pd[8][32], ps[8][32];
+  __shared__ float tg[32], ds[32];
   __shared__ float red[256];
-  const long rows = (long)T * B;
+  const int bi = threadIdx.x & 31, tl = threadIdx.x >> 5;
+  const int groups = (B + 31) / 32;
   float acc = 0.f;
-  for (long row = (long)blockIdx.x * 256 + threadIdx.x; row < rows; row += (long)gridDim.x * 256) {
-    const int t = (int)(row / B), b = (int)(row - (long)t * B);
-    const f32x4 st = stats[row];
-    const float C = st[0], S = st[1];
-    const float X = C * k.a1 + S * k.a2, Y = C * k.b1 + S * k.b2;
-    const float theta = atan2f(Y, X);
-    const float a = angle[(size_t)b * T + t];
-    float sth, cth, sa, ca;
-    sincosf(theta, &sth, &cth);
-    sincosf(a, &sa, &ca);
-    acc += (cth - ca) * (cth - ca) + (sth - sa) * (sth - sa);
-    // d/dtheta of (cos theta - cos a)^2 + (sin theta - sin a)^2 = 2 sin(theta - a)
-    const float dth = 2.f * (sth * ca - cth * sa) / fmaxf(X * X + Y * Y, 1e-30f);
-    // amplitude term: 2 (amp_t - target); the target (first step, unless given) collects minus the sum over t
-    float beta = 2.f * (st[2] - tgt[b]);
-    if (own_target && t == 0) beta -= 2.f * dsum[b];
-    stats[row] = f32x4{dth * (X * k.b1 - Y * k.a1), dth * (X * k.b2 - Y * k.a2), bump_weight * beta, theta};
+  for (int bg = blockIdx.x; bg < groups; bg += gridDim.x) {
+    const int b = bg * 32 + bi, bc = b < B ? b : B - 1;
+    const float target = target_amp ? target_amp[bc] : stats[bc][2];   // row t = 0 is stats[0*B + b]
+    float d = 0.f, s = 0.f;
+    for (int t = tl; t < T; t += 8) {
+      const float dev = stats[(size_t)t * B + bc][2] - target;
+      d += dev;
+      s = fmaf(dev, dev, s);
+    }
+    pd[tl][bi] = d;
+    ps[tl][bi] = s;
+    __syncthreads();
+    if (tl == 0) {
+      float dd = 0.f, ss = 0.f;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        dd += pd[j][bi];
+        ss += ps[j][bi];
+      }
+      tg[bi] = target;
+      ds[bi] = dd;
+      if (b < B) sq[b] = ss;
+    }
+    __syncthreads();
+    if (b < B) {
+      const float tgt = tg[bi], dsum = ds[bi];
+      for (int t = tl; t < T; t += 8) {
+        const size_t row = (size_t)t * B + b;
+        const f32x4 st = stats[row];
+        const float C = st[0], S = st[1];
+        const float X = C * k.a1 + S * k.a2, Y = C * k.b1 + S * k.b2;
+        const float theta = atan2f(Y, X);
+        const float a = angle[(size_t)b * T + t];
+        float sth, cth, sa, ca;
+        sincosf(theta, &sth, &cth);
+        sincosf(a, &sa, &ca);
+        acc += (cth - ca) * (cth - ca) + (sth - sa) * (sth - sa);
+        // d/dtheta of (cos theta - cos a)^2 + (sin theta - sin a)^2 = 2 sin(theta - a)
+        const float dth = 2.f * (sth * ca - cth * sa) / fmaxf(X * X + Y * Y, 1e-30f);
+        // amplitude term: 2 (amp_t - target); the target (first step, unless given) collects minus the sum over t
+        float beta = 2.f * (st[2] - tgt);
+        if (!target_amp && t == 0) beta -= 2.f * dsum;
+        stats[row] = f32x4{dth * (X * k.b1 - Y * k.a1), dth * (X * k.b2 - Y * k.a2), bump_weight * beta, theta};
+      }
+    }
+    __syncthreads();          // pd / ps / tg / ds are reused by the next group of rows
   }
   red[threadIdx.x] = acc;
   __syncthreads();
@@ -335,11 +339,9 @@ hipError_t ring_launch_loss_fwd(const float* hist, const float* angle, const flo
   if (!have_row_sums) {
     LOSS_DISPATCH(hipLaunchKernelGGL((ring_loss_stats_kernel<NCH, VEC>), dim3(grid), dim3(256), 0, st, hist, w.stats, N, T, B));
   }
-  hipLaunchKernelGGL(ring_loss_rows_kernel, dim3((B + 31) / 32), dim3(256), 0, st, w.stats, target_amp, w.tgt, w.dsum, w.sq,
-                     T, B);
-  const int dgrid = (int)((rows + 255) / 256 < 2048 ? (rows + 255) / 256 : 2048);
-  hipLaunchKernelGGL(ring_loss_decode_kernel, dim3(dgrid), dim3(256), 0, st, w.stats, angle, w.tgt, w.dsum, w.partial, k,
-                     bump_weight, target_amp ? 0 : 1, T, B);
+  const int dgrid = (B + 31) / 32 < 2048 ? (B + 31) / 32 : 2048;      // the workspace holds 2048 partial sums
+  hipLaunchKernelGGL(ring_loss_decode_kernel, dim3(dgrid), dim3(256), 0, st, w.stats, angle, target_amp, w.sq, w.partial, k,
+                     bump_weight, T, B);
   hipLaunchKernelGGL(ring_loss_final_kernel, dim3(1), dim3(256), 0, st, w.partial, dgrid, w.sq, B, 1.f / (float)rows,
                      bump_weight, loss_out);
   return hipGetLastError();
