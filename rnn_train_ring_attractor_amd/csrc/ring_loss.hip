@@ -120,10 +120,10 @@ __global__ __launch_bounds__(256) void ring_loss_stats_kernel(const float* __res
   }
 }
 
-// Per batch row, then per (t, b), in one launch.  A workgroup takes 32 batch rows at a time (eight threads per row
+// Per batch row, then per (t, b), in one launch.  A workgroup takes 16 batch rows at a time (sixteen threads per row
 // stride over t):
 //  1. target amplitude of the row, sum over t of the deviations (what flows into the target) and of their squares,
-//     combined over the eight threads in a fixed order;
+//     combined over the sixteen threads in a fixed order;
 //  2. the decode and everything transcendental for the same rows: stats[row] is replaced by the row's gradient
 //     coefficients (kc, ks, beta, theta), all still without the 1/(T*B) and upstream factors:
 //       d total / d r_i = kc cos(phi_i) + ks sin(phi_i) + beta sign(r_i).
@@ -132,17 +132,17 @@ __global__ __launch_bounds__(256) void ring_loss_decode_kernel(f32x4* __restrict
                                                                const float* __restrict__ target_amp, float* __restrict__ sq,
                                                                float* __restrict__ partial, LossConsts k, float bump_weight,
                                                                int T, int B) {
-  __shared__ float pd[8][32], ps[8][32];
-  __shared__ float tg[32], ds[32];
+  __shared__ float pd[16][16], ps[16][16];
+  __shared__ float tg[16], ds[16];
   __shared__ float red[256];
-  const int bi = threadIdx.x & 31, tl = threadIdx.x >> 5;
-  const int groups = (B + 31) / 32;
+  const int bi = threadIdx.x & 15, tl = threadIdx.x >> 4;
+  const int groups = (B + 15) / 16;
   float acc = 0.f;
   for (int bg = blockIdx.x; bg < groups; bg += gridDim.x) {
-    const int b = bg * 32 + bi, bc = b < B ? b : B - 1;
+    const int b = bg * 16 + bi, bc = b < B ? b : B - 1;
     const float target = target_amp ? target_amp[bc] : stats[bc][2];   // row t = 0 is stats[0*B + b]
     float d = 0.f, s = 0.f;
-    for (int t = tl; t < T; t += 8) {
+    for (int t = tl; t < T; t += 16) {
       const float dev = stats[(size_t)t * B + bc][2] - target;
       d += dev;
       s = fmaf(dev, dev, s);
@@ -153,7 +153,7 @@ __global__ __launch_bounds__(256) void ring_loss_decode_kernel(f32x4* __restrict
     if (tl == 0) {
       float dd = 0.f, ss = 0.f;
 #pragma unroll
-      for (int j = 0; j < 8; ++j) {
+      for (int j = 0; j < 16; ++j) {
         dd += pd[j][bi];
         ss += ps[j][bi];
       }
@@ -164,7 +164,7 @@ __global__ __launch_bounds__(256) void ring_loss_decode_kernel(f32x4* __restrict
     __syncthreads();
     if (b < B) {
       const float tgt = tg[bi], dsum = ds[bi];
-      for (int t = tl; t < T; t += 8) {
+      for (int t = tl; t < T; t += 16) {
         const size_t row = (size_t)t * B + b;
         const f32x4 st = stats[row];
         const float C = st[0], S = st[1];
@@ -339,7 +339,7 @@ hipError_t ring_launch_loss_fwd(const float* hist, const float* angle, const flo
   if (!have_row_sums) {
     LOSS_DISPATCH(hipLaunchKernelGGL((ring_loss_stats_kernel<NCH, VEC>), dim3(grid), dim3(256), 0, st, hist, w.stats, N, T, B));
   }
-  const int dgrid = (B + 31) / 32 < 2048 ? (B + 31) / 32 : 2048;      // the workspace holds 2048 partial sums
+  const int dgrid = (B + 15) / 16 < 2048 ? (B + 15) / 16 : 2048;      // the workspace holds 2048 partial sums
   hipLaunchKernelGGL(ring_loss_decode_kernel, dim3(dgrid), dim3(256), 0, st, w.stats, angle, target_amp, w.sq, w.partial, k,
                      bump_weight, T, B);
   hipLaunchKernelGGL(ring_loss_final_kernel, dim3(1), dim3(256), 0, st, w.partial, dgrid, w.sq, B, 1.f / (float)rows,
