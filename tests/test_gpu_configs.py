@@ -138,6 +138,41 @@ def test_headline_size_training_objective_as_one_operator(gpu_device):
     assert O.max_rel_err((0.5 * (lo[2] + hi[2])).cpu().numpy(), one[2].cpu().numpy()) <= 1e-4
 
 
+def test_widest_ring_at_a_training_batch(gpu_device):
+    """N = 2048 (the reference's widest published ring), B = 512, T = 16, forward + backward on the step-per-launch
+    kernels: bitwise repeatable, samples independent (a half-batch shard reproduces its rows bit for bit), gradients
+    additive over shards; the fp64 oracle checks a 16-row slice."""
+    from rnn_train_ring_attractor_amd import ring_rnn_cuda_func
+    print("[case] widest ring N=2048 B=512 T=16 tanh", flush=True)
+    B, T, k, N = 512, 16, 2, 2048
+    J0, J1 = -1.0 / N, 1.0
+    p = make_problem(44, B, T, k, N)
+    A, r0, G = _t(p["A"], gpu_device), _t(p["r0"], gpu_device), _t(p["G"], gpu_device)
+
+    def run(rows):
+        Wa = _t(p["Wa"], gpu_device).requires_grad_(True)
+        Wo = _t(p["Wo"], gpu_device).requires_grad_(True)
+        h = ring_rnn_cuda_func(A[rows].contiguous(), Wa, J0, J1, Wo, r0[rows].contiguous(), 0.15, "tanh")
+        h.backward(G[:, rows].contiguous())
+        return h.detach(), Wa.grad, Wo.grad
+
+    full, again = run(slice(0, B)), run(slice(0, B))
+    assert all(torch.equal(a, b) for a, b in zip(full, again)) and torch.isfinite(full[0]).all()
+    lo, hi = run(slice(0, B // 2)), run(slice(B // 2, B))
+    assert torch.equal(lo[0], full[0][:, :B // 2]) and torch.equal(hi[0], full[0][:, B // 2:])
+    for i in (1, 2):
+        # (the half batch runs on the other step-per-launch kernel family; the two agree to rounding, not bit for
+        # bit: see test_step_per_launch_families_agree)
+        assert O.max_rel_err((lo[i] + hi[i]).cpu().numpy(), full[i].cpu().numpy()) <= 3e-3
+    sl = slice(256, 272)
+    part = run(sl)
+    ref, _ = O.forward_dense(p["A"][sl], p["Wa"], J0, J1, p["Wo"], p["r0"][sl], 0.15, "tanh")
+    assert O.max_rel_err(part[0].cpu().numpy(), ref) <= TRAJ_TOL
+    g = O.backward_dense(p["G"][:, sl], p["A"][sl], p["Wa"], J0, J1, p["Wo"], ref, p["r0"][sl], 0.15, "tanh")
+    assert O.cosine(part[2].cpu().numpy(), g["grad_Wo"]) >= GRAD_COS
+    assert O.max_rel_err(part[2].cpu().numpy(), g["grad_Wo"]) <= GRAD_TOL
+
+
 def test_long_sequence_shape_at_full_size(gpu_device):
     """N=512, B=8192, T=512, tanh at its real size (inputs generated on the device): bitwise repeatable, a 32-row
     slice run alone reproduces its rows of the full batch bit for bit and agrees with the fp64 oracle, the
