@@ -265,7 +265,14 @@ __global__ __launch_bounds__(256) void ring_block_bptt_kernel(RingBpttArgs p, in
     else G = load4_masked(gout, N, B, (int)prow, j);
     if (carry_in) G += *reinterpret_cast<const f32x4*>(carry_in + prow * NPAD + j);
     const f16x4 d = *reinterpret_cast<const f16x4*>(drow + prow * NPAD + j);
-    return f32x4{(float)d[0] * G[0], (float)d[1] * G[1], (float)d[2] * G[2], (float)d[3] * G[3]};
+    // products rounded on their own (never contracted into the row sum that follows), so that both step-per-launch
+    // families form bit-identical g and row sums whatever the compiler does with the surrounding code
+    f32x4 g;
+    {
+#pragma clang fp contract(off)
+      g = f32x4{(float)d[0] * G[0], (float)d[1] * G[1], (float)d[2] * G[2], (float)d[3] * G[3]};
+    }
+    return g;
   };
   stage_tiles<RT>(xb, slots, rs, NPAD, tid, [&](int row, int j) { f32x4 G; return g4(row, j, G); });
   if (staged) stage_gates_rt<RT>(gl, p.A, p.k, T, B, t, bt0, tid);

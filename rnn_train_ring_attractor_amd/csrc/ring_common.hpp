@@ -91,9 +91,9 @@ __device__ __forceinline__ void act_fast(float x, float& F, float& D) {
   } else if constexpr (ACT == ACT_TANH) {
     const float xc = fminf(fmaxf(x, -15.f), 15.f);
     const float e2 = __builtin_amdgcn_exp2f(xc * 2.88539008f);      // exp(2x)
-    const float th = 1.f - 2.f * __builtin_amdgcn_rcpf(e2 + 1.f);
+    const float th = fmaf(-2.f, __builtin_amdgcn_rcpf(e2 + 1.f), 1.f);
     F = th;
-    D = 1.f - th * th;
+    D = fmaf(-th, th, 1.f);                       // written as one fused operation: the same bits in every kernel
   } else {
     const float xc = fmaxf(x, -87.f);
     const float s = __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(xc * -1.44269504f));

@@ -161,9 +161,9 @@ def test_widest_ring_at_a_training_batch(gpu_device):
     lo, hi = run(slice(0, B // 2)), run(slice(B // 2, B))
     assert torch.equal(lo[0], full[0][:, :B // 2]) and torch.equal(hi[0], full[0][:, B // 2:])
     for i in (1, 2):
-        # (the half batch runs on the other step-per-launch kernel family; the two agree to rounding, not bit for
-        # bit: see test_step_per_launch_families_agree)
-        assert O.max_rel_err((lo[i] + hi[i]).cpu().numpy(), full[i].cpu().numpy()) <= 3e-3
+        # (the half batch runs on the other step-per-launch kernel family, which gives the same bits: only the order
+        # of the sum over the batch differs between one call and two)
+        assert O.max_rel_err((lo[i] + hi[i]).cpu().numpy(), full[i].cpu().numpy()) <= 1e-4
     sl = slice(256, 272)
     part = run(sl)
     ref, _ = O.forward_dense(p["A"][sl], p["Wa"], J0, J1, p["Wo"], p["r0"][sl], 0.15, "tanh")
@@ -293,8 +293,9 @@ def test_paired_batch_tiles_equal_single_tiles(B, T, k, N, act, saved, gpu_devic
 ])
 def test_step_per_launch_families_agree(B, T, k, N, act, force, saved, gpu_device, monkeypatch):
     """The step-per-launch kernels (block, one-tile) and the persistent streaming kernels evaluate the same recurrence
-    on the same bf16 operands; they differ in accumulation order only.  Each forced pair must agree to rounding, and
-    the second run is also held to the oracle."""
+    on the same bf16 operands.  The two step-per-launch families must agree bit for bit; the persistent streaming
+    kernels differ from them in accumulation order and must agree to rounding.  The second run is also held to the
+    oracle."""
     from rnn_train_ring_attractor_amd import rnn_cuda
     print(f"[case] step families B={B} T={T} k={k} N={N} {act} {force} saved={saved}", flush=True)
     p = make_problem(31 + N + k, B, T, k, N)
@@ -317,6 +318,11 @@ def test_step_per_launch_families_agree(B, T, k, N, act, force, saved, gpu_devic
         torch.cuda.synchronize()
         outs[mode] = [x.cpu().numpy() for x in (hist, gWa, gWo, gr0)]
     a, b = outs[modes[0]], outs[modes[1]]
+    if var == "RINGATTR_WIDE":
+        # block and one-tile kernels share layouts and the order of every sum: the same bits, so that which of them
+        # the launcher picks for a batch size never shows in a result
+        for x, y in zip(a, b):
+            assert np.array_equal(x, y)
     assert O.max_rel_err(a[0], b[0]) <= 1e-4
     for x, y in zip(a[1:], b[1:]):
         # a last-bit difference in fp32 can flip the bf16 rounding of an operand copy (or a relu kink)
