@@ -429,10 +429,6 @@ __global__ __launch_bounds__(256) void ring_fwd_kernel(RingFwdArgs p) {
     write_operand<NC>(xb(0, rt), r, w, q, n);
     publish_rowsum<NC>(psum[0][rt], r, w, q, n);
     if (staged) gates_stage(gl[0] + rt * 16 * GATE_KMAX, p.A, p.k, T, B, 0, bt0 + rt, tid);
-    if (p.rfrag && bt0 + rt < p.nbt) {
-      pair_store<NC>(p.rfrag, 0, p.nbt, bt0 + rt, w, lane, r);
-      pair_zero_tail<NC>(p.rfrag, T, p.nbt, bt0 + rt, w, lane);
-    }
   }
   lds_barrier();
 
@@ -469,10 +465,18 @@ __global__ __launch_bounds__(256) void ring_fwd_kernel(RingFwdArgs p) {
       read_rowsum(psum[cur][rt], q, s);
       float r[4][NC], d[4][NC];
       state_get(rt, r);
+      const bool live = bt0 + rt < p.nbt;
+      // The bf16 operand copy pairs steps 2j and 2j+1 in one 16-byte slot per lane and tile.  At an even step both
+      // halves are in registers, this step's operand (r before the update) and the next one's (r after it): they
+      // leave as one 16-byte store, whole 32-byte sectors per lane pair, where two 8-byte stores a time step apart
+      // reach memory as two partial writes once a step outlasts the line's stay in L2 (wide tilings).
+      const bool pair_now = p.rfrag && live && (t & 1) == 0;
+      const bool tail = t + 1 == T;                // odd length: the last slot's second half has no step and reads as zero
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
+      for (int c = 0; c < NC; ++c) {
+        bf16x4 lo = {(__bf16)r[0][c], (__bf16)r[1][c], (__bf16)r[2][c], (__bf16)r[3][c]};
 #pragma unroll
-        for (int c = 0; c < NC; ++c) {
+        for (int e = 0; e < 4; ++e) {
           const float x = acc[rt][c][e] + p.J0 * s[e];
           float F, D;
           act_fast<ACT>(x, F, D);
@@ -480,8 +484,13 @@ __global__ __launch_bounds__(256) void ring_fwd_kernel(RingFwdArgs p) {
           r[e][c] = ok ? (oma * r[e][c] + p.alpha * F) : 0.f;
           d[e][c] = ok ? p.alpha * D : 0.f;   // the saved record is alpha * F'(re)
         }
+        if (pair_now) {
+          bf16x4 hi = {(__bf16)r[0][c], (__bf16)r[1][c], (__bf16)r[2][c], (__bf16)r[3][c]};
+          if (tail) hi = bf16x4{(__bf16)0.f, (__bf16)0.f, (__bf16)0.f, (__bf16)0.f};
+          *reinterpret_cast<bf16x8*>(p.rfrag + pair_offset<NC>(t, p.nbt, bt0 + rt, w * NC + c, lane)) =
+              __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        }
       }
-      const bool live = bt0 + rt < p.nbt;
       rows_store<NC>(p.hist + (size_t)t * B * N, N, B, bq, i0, r);
       if (p.dfrag && live) side_store<NC, f16x4, _Float16>(p.dfrag + side_offset<NC>(t, p.nbt, bt0 + rt, w, lane), d);
       if constexpr (STATS) publish_loss_sums<NC>(lsum[cur ^ 1][rt], r, lc0, ls0, lcd, lsd, w, q, n);
@@ -489,7 +498,6 @@ __global__ __launch_bounds__(256) void ring_fwd_kernel(RingFwdArgs p) {
         state_put(rt, r);
         write_operand<NC>(xb(cur ^ 1, rt), r, w, q, n);
         publish_rowsum<NC>(psum[cur ^ 1][rt], r, w, q, n);
-        if (p.rfrag && live) pair_store<NC>(p.rfrag, t + 1, p.nbt, bt0 + rt, w, lane, r);
       }
     }
     lds_barrier();
@@ -607,7 +615,6 @@ __global__ __launch_bounds__(256) void ring_bptt_kernel(RingBpttArgs p) {
     for (int e = 0; e < 4; ++e)
 #pragma unroll
       for (int c = 0; c < NC; ++c) carry[rt][e][c] = 0.f;
-    if (bt0 + rt < p.nbt) pair_zero_tail<NC>(p.gfrag, T, p.nbt, bt0 + rt, w, lane);
   }
   // the lane's cos(phi_i), sin(phi_i): in registers, or (paired tiles, where registers are short) in LDS
   constexpr bool CS_LDS = LOSS && RT > 1;
@@ -669,6 +676,22 @@ __global__ __launch_bounds__(256) void ring_bptt_kernel(RingBpttArgs p) {
 
   // The weight pipeline restarts every step here; carrying its buffers over would cost registers.
   bf16x8 wf[StreamCfg<NC, RT>::PD][StreamCfg<NC, RT>::KG];
+  // The bf16 operand copy of g pairs steps 2j and 2j+1 in one 16-byte slot per lane and tile: the odd step's half
+  // waits in registers for the even step that follows it here, and the two leave as one 16-byte store (whole
+  // 32-byte sectors per lane pair instead of two partial writes a time step apart).  An odd sequence length starts
+  // on an even step, whose slot's second half has no step and is written as zero.
+  // (paired tiles at the widest tiling have no registers left for it and park it in LDS, each thread its own words)
+  constexpr bool HOLD_LDS = NC == 8 && RT > 1;
+  __shared__ bf16x4 held_lds[HOLD_LDS ? RT * NC * 256 : 1];
+  bf16x4 held[HOLD_LDS ? 1 : RT][HOLD_LDS ? 1 : NC];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+    for (int c = 0; c < NC; ++c) {
+      const bf16x4 z = {(__bf16)0.f, (__bf16)0.f, (__bf16)0.f, (__bf16)0.f};
+      if constexpr (HOLD_LDS) held_lds[(rt * NC + c) * 256 + tid] = z;
+      else held[rt][c] = z;
+    }
   for (int t = T - 1; t >= 0; --t) {
     const int cur = (T - 1 - t) & 1;
     // The accumulators start at (1-alpha) G, so that G itself is dead before the products begin.
@@ -712,7 +735,20 @@ __global__ __launch_bounds__(256) void ring_bptt_kernel(RingBpttArgs p) {
       }
       write_operand<NC>(xb(cur, rt), g, w, q, n);
       publish_rowsum<NC>(psum[cur][rt], g, w, q, n);
-      if (live) pair_store<NC>(p.gfrag, t, p.nbt, bt0 + rt, w, lane, g);
+#pragma unroll
+      for (int c = 0; c < NC; ++c) {
+        const bf16x4 pk = {(__bf16)g[0][c], (__bf16)g[1][c], (__bf16)g[2][c], (__bf16)g[3][c]};
+        if (t & 1) {
+          if constexpr (HOLD_LDS) held_lds[(rt * NC + c) * 256 + tid] = pk;
+          else held[rt][c] = pk;
+        } else if (live) {
+          bf16x4 hi;
+          if constexpr (HOLD_LDS) hi = held_lds[(rt * NC + c) * 256 + tid];
+          else hi = held[rt][c];
+          *reinterpret_cast<bf16x8*>(p.gfrag + pair_offset<NC>(t, p.nbt, bt0 + rt, w * NC + c, lane)) =
+              __builtin_shufflevector(pk, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        }
+      }
     }
     lds_barrier();
     const float* glt = staged ? gl[cur] : nullptr;
