@@ -126,7 +126,7 @@ __global__ __launch_bounds__(256) void ring_wide_fwd_kernel(RingFwdArgs p, int N
 
   const float oma = 1.f - p.alpha;
   const size_t rows_pad = (size_t)16 * p.nbt;
-  bf16x4 rcopy[TPW];
+  bf16x4 rcopy[TPW], ncopy[TPW];
 #pragma unroll
   for (int e = 0; e < 4; ++e) {
     const int b = b0 + e;
@@ -141,6 +141,12 @@ __global__ __launch_bounds__(256) void ring_wide_fwd_kernel(RingFwdArgs p, int N
       rn[cl] = ok ? fmaf(p.alpha, F, oma * rp[cl]) : 0.f;
       dd[cl] = ok ? p.alpha * D : 0.f;
       rcopy[cl][e] = (__bf16)rp[cl];
+      ncopy[cl][e] = (__bf16)rn[cl];
+    }
+    if constexpr (REBUILD) {   // the copy is of the history as given, not of the state recomputed here
+      const f32x4 rh = loadv_masked<TPW>(p.hist + (size_t)t * B * N, N, B, b, j0);
+#pragma unroll
+      for (int cl = 0; cl < TPW; ++cl) ncopy[cl][e] = (__bf16)rh[cl];
     }
     if (!REBUILD) storev_masked<TPW>(p.hist + (size_t)t * B * N, N, B, b, j0, rn);
     if (p.dfrag) {
@@ -149,15 +155,16 @@ __global__ __launch_bounds__(256) void ring_wide_fwd_kernel(RingFwdArgs p, int N
       for (int cl = 0; cl < TPW; ++cl) dst[cl] = (_Float16)dd[cl];
     }
   }
-  if (p.rfrag) {
-    // bf16 copy of this step's operand r_prev for the weight-gradient kernel (slot t of the paired buffer)
+  if (p.rfrag && (t & 1) == 0) {
+    // bf16 copies of the operands of this step and the next (r_prev and the new r) for the weight-gradient kernel:
+    // the paired buffer holds steps 2j and 2j+1 in one 16-byte slot, and an even step has both halves in registers,
+    // so they leave as one store (odd steps write none); past an odd sequence's last step the second half is zero
+    const bool tail = t + 1 == T;
 #pragma unroll
-    for (int cl = 0; cl < TPW; ++cl)
-      *reinterpret_cast<bf16x4*>(p.rfrag + pair_off_rt(NC, t, p.nbt, bt, tg0 + cl, lane)) = rcopy[cl];
-    if (t == T - 1 && (T & 1)) {
-      const bf16x4 z = {(__bf16)0.f, (__bf16)0.f, (__bf16)0.f, (__bf16)0.f};
-#pragma unroll
-      for (int cl = 0; cl < TPW; ++cl) *reinterpret_cast<bf16x4*>(p.rfrag + pair_off_rt(NC, T, p.nbt, bt, tg0 + cl, lane)) = z;
+    for (int cl = 0; cl < TPW; ++cl) {
+      const bf16x4 hi = tail ? bf16x4{(__bf16)0.f, (__bf16)0.f, (__bf16)0.f, (__bf16)0.f} : ncopy[cl];
+      *reinterpret_cast<bf16x8*>(p.rfrag + pair_off_rt(NC, t, p.nbt, bt, tg0 + cl, lane)) =
+          __builtin_shufflevector(rcopy[cl], hi, 0, 1, 2, 3, 4, 5, 6, 7);
     }
   }
 }

@@ -198,7 +198,7 @@ __global__ __launch_bounds__(256) void ring_block_fwd_kernel(RingFwdArgs p, int 
 #pragma unroll
   for (int i = 0; i < RT; ++i) {
     if (bt0 + i >= p.nbt) break;                           // a partial last block of batch tiles
-    bf16x4 rcopy[TPW];
+    bf16x4 rcopy[TPW], ncopy[TPW];
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
       const int b = b0 + 16 * i + e;
@@ -213,6 +213,12 @@ __global__ __launch_bounds__(256) void ring_block_fwd_kernel(RingFwdArgs p, int 
         rn[cl] = ok ? fmaf(p.alpha, F, oma * rp[cl]) : 0.f;
         dd[cl] = ok ? p.alpha * D : 0.f;
         rcopy[cl][e] = (__bf16)rp[cl];
+        ncopy[cl][e] = (__bf16)rn[cl];
+      }
+      if constexpr (REBUILD) {   // the copy is of the history as given, not of the state recomputed here
+        const f32x4 rh = loadv_masked<TPW>(p.hist + (size_t)t * B * N, N, B, b, j0);
+#pragma unroll
+        for (int cl = 0; cl < TPW; ++cl) ncopy[cl][e] = (__bf16)rh[cl];
       }
       if (!REBUILD) storev_masked<TPW>(p.hist + (size_t)t * B * N, N, B, b, j0, rn);
       if (p.dfrag) {
@@ -221,15 +227,15 @@ __global__ __launch_bounds__(256) void ring_block_fwd_kernel(RingFwdArgs p, int 
         for (int cl = 0; cl < TPW; ++cl) dst[cl] = (_Float16)dd[cl];
       }
     }
-    if (p.rfrag) {
+    if (p.rfrag && (t & 1) == 0) {
+      // both halves of the pair slot (this step's operand and the next one's) as one 16-byte store, as in
+      // ring_wide_fwd_kernel; odd steps write none
+      const bool tail = t + 1 == T;
 #pragma unroll
-      for (int cl = 0; cl < TPW; ++cl)
-        *reinterpret_cast<bf16x4*>(p.rfrag + pair_off_rt(NC, t, p.nbt, bt0 + i, tg0 + cl, lane)) = rcopy[cl];
-      if (t == T - 1 && (T & 1)) {
-        const bf16x4 z = {(__bf16)0.f, (__bf16)0.f, (__bf16)0.f, (__bf16)0.f};
-#pragma unroll
-        for (int cl = 0; cl < TPW; ++cl)
-          *reinterpret_cast<bf16x4*>(p.rfrag + pair_off_rt(NC, T, p.nbt, bt0 + i, tg0 + cl, lane)) = z;
+      for (int cl = 0; cl < TPW; ++cl) {
+        const bf16x4 hi = tail ? bf16x4{(__bf16)0.f, (__bf16)0.f, (__bf16)0.f, (__bf16)0.f} : ncopy[cl];
+        *reinterpret_cast<bf16x8*>(p.rfrag + pair_off_rt(NC, t, p.nbt, bt0 + i, tg0 + cl, lane)) =
+            __builtin_shufflevector(rcopy[cl], hi, 0, 1, 2, 3, 4, 5, 6, 7);
       }
     }
   }
