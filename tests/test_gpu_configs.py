@@ -335,6 +335,40 @@ def test_step_per_launch_families_agree(B, T, k, N, act, force, saved, gpu_devic
     assert O.cosine(b[3], ref["grad_r_init"]) >= floor
 
 
+@pytest.mark.parametrize("B,T,k,N,act,wide", [(40, 5, 2, 1024, "tanh", "1"), (40, 6, 2, 1024, "gelu", "0"),
+                                                (24, 7, 3, 700, "silu", "1"), (24, 1, 2, 640, "tanh", "0")])
+def test_step_per_launch_rebuild_equals_saved_record_bitwise(B, T, k, N, act, wide, gpu_device, monkeypatch):
+    """Without the forward's saved buffer the step-per-launch families recompute the derivative record and the operand
+    copies from bump_history with the forward's own kernel (all steps in one launch), so the backward must give the
+    same bits as with the buffer.  Even and odd sequence lengths: the operand copies are written a pair of steps at a
+    time, and an odd length leaves half a pair."""
+    from rnn_train_ring_attractor_amd import rnn_cuda
+    print(f"[case] step rebuild == saved B={B} T={T} k={k} N={N} {act} wide={wide}", flush=True)
+    monkeypatch.setenv("RINGATTR_WIDE", wide)
+    p = make_problem(57 + N + T, B, T, k, N)
+    acts = {"relu": 0, "gelu": 1, "tanh": 2, "silu": 3}
+    J0, J1 = -1.0 / N, 0.3
+    A, Wa, Wo, r0, G = (_t(p[x], gpu_device) for x in ("A", "Wa", "Wo", "r0", "G"))
+    hist = torch.empty(T, B, N, device=gpu_device)
+    sv = torch.empty(rnn_cuda.saved_nbytes(N, k, T, B), dtype=torch.uint8, device=gpu_device)
+    rnn_cuda.fwd_cuda.fwd(A=A, Wa=Wa, J0=J0, J1=J1, Wo=Wo, r_init=r0, bump_history=hist, alpha=0.15,
+                          activation_type=acts[act], saved=sv)
+    outs = []
+    for saved in (sv, None):
+        gWa, gWo, gr0 = torch.zeros_like(Wa), torch.zeros_like(Wo), torch.empty_like(r0)
+        rnn_cuda.bwd_cuda.bwd(grad_output=G, A=A, Wa=Wa, J0=J0, J1=J1, Wo=Wo, bump_history=hist, r_init=r0,
+                              grad_Wa=gWa, grad_Wo=gWo, alpha=0.15, activation_type=acts[act], saved=saved,
+                              grad_r_init=gr0)
+        torch.cuda.synchronize()
+        outs.append((gWa, gWo, gr0))
+    for x, y in zip(*outs):
+        assert torch.isfinite(x).all() and torch.equal(x, y)
+    ref_hist, _ = O.forward_dense(p["A"], p["Wa"], J0, J1, p["Wo"], p["r0"], 0.15, act)
+    ref = O.backward_dense(p["G"], p["A"], p["Wa"], J0, J1, p["Wo"], ref_hist, p["r0"], 0.15, act)
+    assert O.cosine(outs[1][1].cpu().numpy(), ref["grad_Wo"]) >= 0.999
+    assert O.cosine(outs[1][0].cpu().numpy(), ref["grad_Wa"]) >= 0.999
+
+
 @pytest.mark.parametrize("B,T,k,N,act", [(72, 5, 3, 1024, "tanh"), (40, 4, 7, 640, "silu")], ids=["n1024_k3", "n640_k7"])
 def test_block_kernel_shapes_and_workgroup_orders_agree_bitwise(B, T, k, N, act, gpu_device, monkeypatch):
     """The block kernels come in four shapes (one or two row tiles per workgroup, one or two column tiles per wave)
