@@ -36,6 +36,18 @@ __device__ __forceinline__ bf16x8 pack_fragment(const float* __restrict__ Wo, co
   const int k0 = 32 * kc + 8 * q;
   const float* W = (mm == 0) ? Wo : Wa + (size_t)(mm - 1) * N * N;
   bf16x8 pk;
+  if (!transposed && !split_k && (N & 3) == 0 && col < N && k0 + 8 <= N) {
+    // forward orientation away from the padding: the fragment's eight values lie side by side in one row
+    const f32x4* src = reinterpret_cast<const f32x4*>(W + (size_t)col * N + k0);
+    const f32x4 a = src[0], b = src[1];
+#pragma unroll
+    for (int x = 0; x < 8; ++x) {
+      float val = x < 4 ? a[x] : b[x - 4];
+      if (mm == 0) val = fmaf(val, scale0, shift0);
+      pk[x] = (__bf16)val;
+    }
+    return pk;
+  }
 #pragma unroll
   for (int x = 0; x < 8; ++x) {
     const int kk = split_k ? split_k_neuron(k0 + x) : k0 + x;
