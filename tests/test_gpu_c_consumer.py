@@ -29,7 +29,7 @@ def test_plain_c_caller(N, B, T, gpu_device):
     assert rc == 0, msg.value.decode()
 
 
-def test_reference_side_binding_from_the_integration_guide(gpu_device, monkeypatch):
+def test_reference_side_binding_from_the_integration_guide(gpu_device, monkeypatch, default_kernels):
     """The ctypes stub that the integration guide proposes for the reference's cpp/rnn_cuda.py, executed verbatim from
     the guide: its fwd_cuda.fwd / bwd_cuda.bwd (reference keyword names, no saved buffer, gradients added to) give the
     history of the packaged operator bit for bit and its gradients to rounding."""

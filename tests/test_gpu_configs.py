@@ -637,7 +637,7 @@ def _gain_oracle(model, av, r0, G, act):
     return hist, g, gp, model_g, gp_model
 
 
-def test_gain_network_configuration_at_full_size(gpu_device):
+def test_gain_network_configuration_at_full_size(gpu_device, default_kernels):
     """The general ring with gain networks at its benchmark size: N=256, B=4096, T=240, relu, two 1 -> 16 -> 1 gain
     networks evaluated by the HIP gain operator, BPTT through the weight-resident kernel with dL/d action_signal.
     A 64-row slice is checked against the fp64 oracle (trajectory, weight gradients, gain-network gradients); the
@@ -693,7 +693,7 @@ def test_gain_network_configuration_at_full_size(gpu_device):
 
 
 @pytest.mark.parametrize("weights", ["random", "perfect"])
-def test_relu_gradients_against_fp64_at_a_realistic_batch(weights, gpu_device):
+def test_relu_gradients_against_fp64_at_a_realistic_batch(weights, gpu_device, default_kernels):
     """relu weight gradients against the fp64 oracle at B = 1024, T = 120 (122 880 samples per entry).  relu's
     derivative is a step, and rounding the operands to bf16 moves pre-activations across it: with random weights
     single entries differ from fp64 by 3-6 % even at this batch, with bump-sustaining weights (a few neurons carry

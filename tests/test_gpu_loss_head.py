@@ -161,7 +161,7 @@ def test_one_operator_also_returns_the_action_signal_gradient(B, T, k, N, act, g
 
 
 @pytest.mark.parametrize("B,N", [(32, 256), (21, 200)], ids=["n256_full", "n200_masked"])
-def test_one_operator_without_a_backward_returns_the_same_losses(B, N, gpu_device):
+def test_one_operator_without_a_backward_returns_the_same_losses(B, N, gpu_device, default_kernels):
     """Under torch.no_grad() the forward keeps no saved record (another variant of the forward kernel forms the loss
     head's row sums); losses and trajectory equal those of the call that prepares a backward."""
     from rnn_train_ring_attractor_amd import ring_rnn_loss_func
