@@ -71,6 +71,7 @@ CASES = [
     # the reference's published many-channel rows (assets/REPORT.md:11-12: 32 and 64 channels)
     ("n2048_k32_dense", 16,  2, 32, 2048, "silu", -0.01, 0.1, "dense"),
     ("n1024_k64_dense", 16,  3, 64, 1024, "tanh", -0.01, 0.1, "dense"),
+    ("n640_k66_dense",  20,  3, 66, 640, "tanh", -1 / 640, 0.3, "dense"),   # wide ring, more channels than the gate stage holds
 ]
 
 
