@@ -109,3 +109,36 @@ def test_training_driver_replays_its_step_from_a_graph(gpu_device):
     assert np.mean(replayed[-4:]) < np.mean(replayed[:4])
     with pytest.raises(ValueError):
         drv.run_training(hip_graph=True, **dict(kw, fused_loss=False))
+
+
+def test_two_streams_interleaved_give_the_sequential_results(gpu_device):
+    """The library keeps no hidden device state between calls: two callers that drive the operator from two streams at
+    the same time, their launches interleaved by one host thread and their kernels free to overlap on the device,
+    each get the bits a lone run gives (different kernel families on the two streams)."""
+    from rnn_train_ring_attractor_amd import ring_rnn_cuda_func
+    print("[case] two streams: N=256 B=1024 T=40 gelu beside N=200 B=640 T=30 tanh", flush=True)
+    jobs = [(make_problem(71, 1024, 40, 2, 256), "gelu"), (make_problem(72, 640, 30, 2, 200), "tanh")]
+
+    def dev(x):
+        return torch.tensor(x, device=gpu_device)
+
+    def run(p, act):
+        Wa, Wo = dev(p["Wa"]).requires_grad_(True), dev(p["Wo"]).requires_grad_(True)
+        r0 = dev(p["r0"]).requires_grad_(True)
+        hist = ring_rnn_cuda_func(dev(p["A"]), Wa, -0.05, 0.4, Wo, r0, 0.15, act)
+        hist.backward(dev(p["G"]))
+        return [hist.detach(), Wa.grad, Wo.grad, r0.grad]
+
+    alone = [run(p, act) for p, act in jobs]
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    together = [[], []]
+    for rep in range(3):
+        for i, (p, act) in enumerate(jobs):
+            with torch.cuda.stream(streams[i]):
+                together[i].append(run(p, act))
+    torch.cuda.synchronize()
+    for i in range(2):
+        for got in together[i]:
+            for x, y in zip(got, alone[i]):
+                assert torch.equal(x, y)
