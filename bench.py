@@ -1,6 +1,6 @@
 """Headline benchmark: fused forward + BPTT of the ring-attractor time loop on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu] [--prewarm-ms MS]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu] [--prewarm-ms MS] [--recompute]
 
 One "step" = one forward + one backward of the operator over one synthetic batch at
 N=256, B=4096, T=120, k=2, gelu (inputs resident in HBM before the timed region).
@@ -11,7 +11,8 @@ length is reported under "prewarm"), then exactly --warmup untimed steps, then e
 two torch.cuda.synchronize().
 
 Prints ONE JSON line: sample-steps/s (B*T per fwd+bwd), the roofline of the slowest kernel from HIP events recorded
-on the launch stream inside the timed region, and host-CPU baselines (torch port of the reference's per-sample-W_eff
+on the launch stream inside the timed region (around every --event-stride-th launch of each kernel: the two event
+records around a launch cost the stream 4-5 us, 23 us per step when every launch is bracketed), and host-CPU baselines (torch port of the reference's per-sample-W_eff
 formulation): the reference's own CPU configuration (N=120, B=64, T=120, tanh, fp32) exactly, and the benchmarked
 workload at a reduced batch.
 """
@@ -132,20 +133,33 @@ def cpu_baseline(N, B, T, k, act, J0, J1, budget_s, note):
             "sample": f"N={N} B={B} T={T} {act} fp32, {len(ts)} fwd+bwd iters, {mean * 1e3:.1f} ms each; {note}"}
 
 
-def measured_traffic(workload):
+def measured_traffic(workload, launched):
     """HBM bytes per launch of each kernel, from the committed rocprofv3 counter summary of this workload
     (profiles/<workload>_counters.md carries a line 'TRAFFIC_BYTES_PER_LAUNCH fwd=.. bptt=.. dw=..': FETCH_SIZE and
     WRITE_SIZE per dispatch, each scaled by what the same counter reads for a 1 GiB device copy).  Counter runs cannot
-    share a process with the timed region, so the figure is read from there; None when no summary exists."""
+    share a process with the timed region, so the figure is read from there.  The summary also names the kernels it
+    was taken from ('TRAFFIC_KERNELS fwd=<kernel>;bptt=<kernel>;...'); `launched` maps the same keys to the kernels
+    this run launched (ringattr_last_kernel_name), and a key whose names differ is dropped: a summary that predates a
+    kernel change must not pass for a measurement of the new kernel.  Returns (traffic or None, list of notes)."""
     path = os.path.join(ROOT, "profiles", f"{workload}_counters.md")
     try:
         text = open(path).read()
     except OSError:
-        return None
+        return None, ["no counter summary for this workload"]
     m = re.search(r"^TRAFFIC_BYTES_PER_LAUNCH\s+(.*)$", text, re.M)
     if not m:
-        return None
-    return {kv.split("=")[0]: float(kv.split("=")[1]) for kv in m.group(1).split()}
+        return None, ["counter summary has no TRAFFIC_BYTES_PER_LAUNCH line"]
+    traffic = {kv.split("=")[0]: float(kv.split("=")[1]) for kv in m.group(1).split()}
+    mk = re.search(r"^TRAFFIC_KERNELS\s+(.*)$", text, re.M)
+    if not mk:
+        return None, ["counter summary names no kernels (TRAFFIC_KERNELS): not used"]
+    named = dict(kv.split("=", 1) for kv in mk.group(1).strip().split(";") if "=" in kv)
+    notes = []
+    for key in list(traffic):
+        if key in launched and named.get(key) != launched[key]:
+            notes.append(f"{key}: summary is of '{named.get(key)}', this run launched '{launched[key]}': dropped")
+            del traffic[key]
+    return (traffic or None), notes
 
 
 def main():
@@ -157,6 +171,12 @@ def main():
     ap.add_argument("--prewarm-ms", type=float, default=500.0,
                     help="untimed steps of the workload run for at least this long before --warmup (clock settling)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the host-CPU baseline legs")
+    ap.add_argument("--recompute", action="store_true",
+                    help="training workloads: the forward keeps no saved record and the backward recomputes the "
+                         "derivative record and operand copy from bump_history first (activation recompute)")
+    ap.add_argument("--event-stride", type=int, default=0,
+                    help="bracket every n-th launch of each kernel with HIP events inside the timed region "
+                         "(0: steps // 4 clamped to 1..8)")
     ap.add_argument("--no-training-step", action="store_true",
                     help="skip the whole-training-step figure that training workloads report beside the metric")
     ap.add_argument("--cpu-sample-batch", type=int, default=128)
@@ -170,6 +190,8 @@ def main():
 
     import torch
     from rnn_train_ring_attractor_amd import _lib, ring_rnn_cuda_func
+    from rnn_train_ring_attractor_amd import ring_rnn_cuda as _op
+    _op.RECOMPUTE_IN_BACKWARD = bool(args.recompute)
     if not torch.cuda.is_available():
         sys.exit("bench.py: no GPU visible; the HIP path has no CPU fallback")
     dev = torch.device("cuda:0")
@@ -230,7 +252,8 @@ def main():
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
-    _lib.profile_enable(True)
+    stride = args.event_stride if args.event_stride > 0 else max(1, min(8, args.steps // 4))
+    _lib.profile_enable(stride)
     _lib.profile_read()
     t0 = time.perf_counter()
     for _ in range(args.steps):
@@ -282,7 +305,8 @@ def main():
     dom_ms = kern[dominant]
     achieved = flops_third / (dom_ms * 1e-3) / 1e12
     bytes_per_ss = 12 * N + 8 * k                           # fp32 history write + r_prev/grad_output reads + A
-    traffic = measured_traffic(args.workload)
+    traffic, traffic_notes = measured_traffic(args.workload + ("_recompute" if args.recompute else ""),
+                                              _lib.last_kernel_names())
     out = {
         "metric": ("fwd+bwd sample-steps/s (B*T/s) at N=256,B=4096,T=120; % bf16 MFMA peak"
                    if args.workload == HEADLINE else
@@ -290,7 +314,7 @@ def main():
         "value": value, "unit": "sample-steps/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": args.workload, "N": N, "B": B, "T": T, "a_dim": k, "activation": cfg["act"],
+        "config": {"workload": args.workload + ("_recompute" if args.recompute else ""), "N": N, "B": B, "T": T, "a_dim": k, "activation": cfg["act"],
                    "mode": {"train": "forward + backward", "infer": "forward only (no saved activations)",
                             "gain": "gain MLPs + forward + backward (MLP gradients through dL/d action_signal)"}[mode],
                    "grad_output": "gradient of the cos-sim + 0.2*bump-amplitude loss pair, precomputed" if train else None},
@@ -300,15 +324,18 @@ def main():
         "roofline": {"bound": "mfma", "kernel": dominant, "achieved": achieved, "peak": PEAK_BF16_TFLOPS,
                      "unit": "TFLOP/s", "frac": achieved / PEAK_BF16_TFLOPS,
                      "traffic": (traffic or {}).get(dominant),
-                     "flops_per_launch": flops_third, "avg_launch_ms": dom_ms,
+                     "flops_per_launch": flops_third, "avg_launch_ms": dom_ms, "event_stride": stride,
                      "algorithmic_bytes_per_launch": (4 * N + 4 * k) * B * T},
         "kernel_ms": kern,
     }
     if training_step:
         out["training_step"] = training_step
+    if traffic_notes:
+        out["traffic_notes"] = traffic_notes
     if traffic:
         out["traffic_bytes_per_launch"] = traffic
-        out["traffic_over_algorithmic"] = sum(traffic.values()) / (bytes_per_ss * B * T) if train else None
+        complete = all(k_ in traffic for k_ in (("fwd", "bptt", "dw") if train else ("fwd",)))
+        out["traffic_over_algorithmic"] = sum(traffic.values()) / (bytes_per_ss * B * T) if train and complete else None
     if not args.no_cpu:
         # the reference's CPU configuration exactly (what cpu_baseline means), then this workload at a reduced batch
         out["cpu_baseline"] = cpu_baseline(120, 64, 120, 2, "tanh", -1.0 / 120, 1.0, 8.0,

@@ -210,8 +210,11 @@ RINGATTR_API int ringattr_clip_adam_counted(int n_tensors, void* const* params, 
                       void* const* exp_avg_sq, const size_t* numel, float lr, float beta1, float beta2, float eps,
                       float max_norm, void* step_counter, void* workspace, size_t workspace_bytes, void* stream);
 
-/* Per-kernel timing for benchmarks; no counterpart in the reference.  While enabled, every kernel
- * launch is bracketed by two HIP events recorded on the launch stream.  ringattr_profile_read waits
+/* Per-kernel timing for benchmarks; no counterpart in the reference.  ringattr_profile_enable(n): n = 0 switches it
+ * off; n >= 1 brackets every n-th launch of each kernel (counted per kernel from this call on) by two HIP events
+ * recorded on the launch stream.  The two records cost about 4-5 us of stream time per bracketed launch (23 us per
+ * forward + backward at n = 1 on an MI355X), which is why a benchmark that also reports wall time samples with
+ * n > 1.  ringattr_profile_read waits
  * for the recorded events, adds their durations into ms[RINGATTR_NUM_KERNELS] and the launch counts
  * into launches[RINGATTR_NUM_KERNELS] (both caller arrays, not cleared first) and forgets them. */
 #define RINGATTR_NUM_KERNELS 6
@@ -222,6 +225,10 @@ RINGATTR_API int ringattr_clip_adam_counted(int n_tensors, void* const* params, 
 #define RINGATTR_K_DW 4
 #define RINGATTR_K_DW_REDUCE 5
 RINGATTR_API int ringattr_profile_enable(int on);
+/* Name of the kernel this process launched last in slot `kernel` (RINGATTR_K_*), e.g.
+ * "ring_fwd_res256_kernel<1,true,true,false>" (demangled, no return type, parameter list or blanks), or the empty
+ * string if the slot has not launched yet.  For benchmarks that pair a timing with a stored counter profile. */
+RINGATTR_API int ringattr_last_kernel_name(int kernel, char* buf, size_t buf_bytes);
 RINGATTR_API int ringattr_profile_read(double* ms, long long* launches);
 
 /* Reference-signature entry points, argument for argument (cpp/fwd.cu:21-35,

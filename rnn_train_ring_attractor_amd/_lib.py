@@ -63,6 +63,7 @@ PROTOTYPES = {
                                            c_void_p]),
     "ringattr_profile_enable": (c_int, [c_int]),
     "ringattr_profile_read": (c_int, [ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_longlong)]),
+    "ringattr_last_kernel_name": (c_int, [c_int, ctypes.c_char_p, ctypes.c_size_t]),
     "fwd_cuda": (None, [c_void_p, c_void_p, c_float, c_float, c_void_p, c_void_p, c_void_p, c_float,
                         c_int, c_int, c_int, c_int, c_int]),
     "bwd_cuda": (None, [c_void_p, c_void_p, c_void_p, c_float, c_float, c_void_p, c_void_p, c_void_p, c_void_p,
@@ -112,8 +113,21 @@ def check(rc: int) -> None:
 KERNEL_NAMES = ("pack_weights", "fwd", "rebuild_saved", "bptt", "dw", "dw_reduce")
 
 
-def profile_enable(on: bool) -> None:
-    check(load().ringattr_profile_enable(1 if on else 0))
+def profile_enable(on) -> None:
+    """False / 0: off.  True / 1: bracket every kernel launch with HIP events; n > 1: every n-th launch of each kernel
+    (the two event records cost the stream 4-5 us per bracketed launch)."""
+    check(load().ringattr_profile_enable(int(on)))
+
+
+def last_kernel_names():
+    """{kernel slot name: name of the kernel launched last in it} for the slots that have launched."""
+    out = {}
+    buf = ctypes.create_string_buffer(256)
+    for i, key in enumerate(KERNEL_NAMES):
+        check(load().ringattr_last_kernel_name(i, buf, len(buf)))
+        if buf.value:
+            out[key] = buf.value.decode()
+    return out
 
 
 def profile_read():

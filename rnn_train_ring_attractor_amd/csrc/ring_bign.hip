@@ -272,13 +272,13 @@ static hipError_t wide_fwd_tpw(const RingFwdArgs& a, int NC, bool rebuild, hipSt
   if (rebuild) {
     hipError_t e = wide_attr(ring_wide_fwd_kernel<ACT, true, TPW>, dyn);
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL((ring_wide_fwd_kernel<ACT, true, TPW>), dim3(a.nbt, ncb, a.T), dim3(256), dyn, st, a, NC, 0, step_xcd_map());
+    RING_LAUNCH((ring_wide_fwd_kernel<ACT, true, TPW>), dim3(a.nbt, ncb, a.T), dim3(256), dyn, st, a, NC, 0, step_xcd_map());
     return hipGetLastError();
   }
   hipError_t e = wide_attr(ring_wide_fwd_kernel<ACT, false, TPW>, dyn);
   if (e != hipSuccess) return e;
   for (int t = 0; t < a.T; ++t) {
-    hipLaunchKernelGGL((ring_wide_fwd_kernel<ACT, false, TPW>), dim3(a.nbt, ncb), dim3(256), dyn, st, a, NC, t, step_xcd_map());
+    RING_LAUNCH((ring_wide_fwd_kernel<ACT, false, TPW>), dim3(a.nbt, ncb), dim3(256), dyn, st, a, NC, t, step_xcd_map());
     e = hipGetLastError();
     if (e != hipSuccess) return e;
   }
@@ -315,7 +315,7 @@ __global__ __launch_bounds__(256) void ring_trig_table_kernel(float* out, int N,
 }
 
 hipError_t ring_launch_trig_table(float* out, int N, int NPAD, hipStream_t st) {
-  hipLaunchKernelGGL(ring_trig_table_kernel, dim3((NPAD + 255) / 256), dim3(256), 0, st, out, N, NPAD);
+  RING_LAUNCH(ring_trig_table_kernel, dim3((NPAD + 255) / 256), dim3(256), 0, st, out, N, NPAD);
   return hipGetLastError();
 }
 
@@ -331,8 +331,8 @@ hipError_t ring_launch_wide_bptt(const RingBpttArgs& a, int NC, float* carry, hi
   for (int t = a.T - 1, u = 0; t >= 0; --t, ++u) {
     const float* cin = (u == 0) ? nullptr : carry + (size_t)((u - 1) & 1) * half;
     float* cout = carry + (size_t)(u & 1) * half;
-    if (loss) hipLaunchKernelGGL(ring_wide_bptt_kernel<true>, dim3(a.nbt, ncb), dim3(256), dyn, st, a, NC, t, cin, cout, step_xcd_map());
-    else hipLaunchKernelGGL(ring_wide_bptt_kernel<false>, dim3(a.nbt, ncb), dim3(256), dyn, st, a, NC, t, cin, cout, step_xcd_map());
+    if (loss) RING_LAUNCH(ring_wide_bptt_kernel<true>, dim3(a.nbt, ncb), dim3(256), dyn, st, a, NC, t, cin, cout, step_xcd_map());
+    else RING_LAUNCH(ring_wide_bptt_kernel<false>, dim3(a.nbt, ncb), dim3(256), dyn, st, a, NC, t, cin, cout, step_xcd_map());
     e = hipGetLastError();
     if (e != hipSuccess) return e;
   }

@@ -464,13 +464,13 @@ static hipError_t block_fwd_shape(const RingFwdArgs& a, int NC, bool rebuild, hi
   if (rebuild) {
     hipError_t e = block_attr(ring_block_fwd_kernel<ACT, true, RT, TPW>, dyn);
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL((ring_block_fwd_kernel<ACT, true, RT, TPW>), grid, dim3(256), dyn, st, a, NC, 0, xm);
+    RING_LAUNCH((ring_block_fwd_kernel<ACT, true, RT, TPW>), grid, dim3(256), dyn, st, a, NC, 0, xm);
     return hipGetLastError();
   }
   hipError_t e = block_attr(ring_block_fwd_kernel<ACT, false, RT, TPW>, dyn);
   if (e != hipSuccess) return e;
   for (int t = 0; t < a.T; ++t) {
-    hipLaunchKernelGGL((ring_block_fwd_kernel<ACT, false, RT, TPW>), grid, dim3(256), dyn, st, a, NC, t, xm);
+    RING_LAUNCH((ring_block_fwd_kernel<ACT, false, RT, TPW>), grid, dim3(256), dyn, st, a, NC, t, xm);
     e = hipGetLastError();
     if (e != hipSuccess) return e;
   }
@@ -507,7 +507,7 @@ static hipError_t block_bptt_shape(const RingBpttArgs& a, int NC, float* carry, 
   for (int t = a.T - 1, u = 0; t >= 0; --t, ++u) {
     const float* cin = (u == 0) ? nullptr : carry + (size_t)((u - 1) & 1) * half;
     float* cout = carry + (size_t)(u & 1) * half;
-    hipLaunchKernelGGL((ring_block_bptt_kernel<RT, TPW, LOSS>), grid, dim3(256), dyn, st, a, NC, t, cin, cout, xm);
+    RING_LAUNCH((ring_block_bptt_kernel<RT, TPW, LOSS>), grid, dim3(256), dyn, st, a, NC, t, cin, cout, xm);
     e = hipGetLastError();
     if (e != hipSuccess) return e;
   }
@@ -536,6 +536,6 @@ hipError_t ring_launch_block_grad_A(const RingBpttArgs& a, const void* Wf, int N
   const size_t dyn = (size_t)2 * NC * 4 * XG * sizeof(bf16x8);
   hipError_t e = block_attr(ring_block_grad_A_kernel<2>, dyn);
   if (e != hipSuccess) return e;
-  hipLaunchKernelGGL((ring_block_grad_A_kernel<2>), dim3(a.nbt, a.T), dim3(256), dyn, st, a, (const bf16x8*)Wf, NC);
+  RING_LAUNCH((ring_block_grad_A_kernel<2>), dim3(a.nbt, a.T), dim3(256), dyn, st, a, (const bf16x8*)Wf, NC);
   return hipGetLastError();
 }

@@ -236,13 +236,13 @@ template <int NC>
 static hipError_t launch_group(const RingDwArgs& a, int mg, unsigned blocks, hipStream_t st) {
   const int nmat = (a.k + 1 - 3 * mg) < 3 ? (a.k + 1 - 3 * mg) : 3;
   if (mg == 0) {
-    if (nmat == 3) hipLaunchKernelGGL((ring_dw_direct_kernel<NC, 3, true>), dim3(blocks), dim3(256), 0, st, a, mg);
-    else if (nmat == 2) hipLaunchKernelGGL((ring_dw_direct_kernel<NC, 2, true>), dim3(blocks), dim3(256), 0, st, a, mg);
-    else hipLaunchKernelGGL((ring_dw_direct_kernel<NC, 1, true>), dim3(blocks), dim3(256), 0, st, a, mg);
+    if (nmat == 3) RING_LAUNCH((ring_dw_direct_kernel<NC, 3, true>), dim3(blocks), dim3(256), 0, st, a, mg);
+    else if (nmat == 2) RING_LAUNCH((ring_dw_direct_kernel<NC, 2, true>), dim3(blocks), dim3(256), 0, st, a, mg);
+    else RING_LAUNCH((ring_dw_direct_kernel<NC, 1, true>), dim3(blocks), dim3(256), 0, st, a, mg);
   } else {
-    if (nmat == 3) hipLaunchKernelGGL((ring_dw_direct_kernel<NC, 3, false>), dim3(blocks), dim3(256), 0, st, a, mg);
-    else if (nmat == 2) hipLaunchKernelGGL((ring_dw_direct_kernel<NC, 2, false>), dim3(blocks), dim3(256), 0, st, a, mg);
-    else hipLaunchKernelGGL((ring_dw_direct_kernel<NC, 1, false>), dim3(blocks), dim3(256), 0, st, a, mg);
+    if (nmat == 3) RING_LAUNCH((ring_dw_direct_kernel<NC, 3, false>), dim3(blocks), dim3(256), 0, st, a, mg);
+    else if (nmat == 2) RING_LAUNCH((ring_dw_direct_kernel<NC, 2, false>), dim3(blocks), dim3(256), 0, st, a, mg);
+    else RING_LAUNCH((ring_dw_direct_kernel<NC, 1, false>), dim3(blocks), dim3(256), 0, st, a, mg);
   }
   return hipGetLastError();
 }

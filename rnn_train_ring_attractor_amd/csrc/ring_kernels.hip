@@ -947,21 +947,35 @@ __global__ __launch_bounds__(256) void ring_dw_reduce_kernel(RingDwArgs p, int N
 // ------------------------------------------------------------------------------------------------
 // Optional per-launch HIP event bracketing (benchmarks only).
 // ------------------------------------------------------------------------------------------------
+#include <cxxabi.h>
 #include <stdlib.h>
+#include <string.h>
+#include <atomic>
 #include <mutex>
+#include <string>
 #include <vector>
 namespace {
+constexpr int PROF_SLOTS = 8;
+thread_local int t_kernel_slot = -1;                     // innermost open ProfScope of this thread
+std::atomic<const void*> g_last_kernel[PROF_SLOTS];      // host function of the last launch per slot
 struct ProfRec { hipEvent_t a, b; int id; };
 std::mutex g_prof_mu;
 std::vector<ProfRec> g_prof;
-bool g_prof_on = false;
+int g_prof_stride = 0;                       // 0: off; n: every n-th launch of each kernel is bracketed
+long g_prof_seen[PROF_SLOTS] = {0, 0, 0, 0, 0, 0, 0, 0};
 
 struct ProfScope {
   hipStream_t st;
   ProfRec rec;
   bool active;
-  ProfScope(int id, hipStream_t s) : st(s), active(false) {
-    if (!g_prof_on) return;
+  int outer;
+  ProfScope(int id, hipStream_t s) : st(s), active(false), outer(t_kernel_slot) {
+    t_kernel_slot = id;
+    if (g_prof_stride <= 0) return;
+    {
+      std::lock_guard<std::mutex> lk(g_prof_mu);
+      if (g_prof_seen[id]++ % g_prof_stride != 0) return;
+    }
     if (hipEventCreate(&rec.a) != hipSuccess) return;
     if (hipEventCreate(&rec.b) != hipSuccess) { (void)hipEventDestroy(rec.a); return; }
     rec.id = id;
@@ -969,6 +983,7 @@ struct ProfScope {
     (void)hipEventRecord(rec.a, st);
   }
   ~ProfScope() {
+    t_kernel_slot = outer;
     if (!active) return;
     (void)hipEventRecord(rec.b, st);
     std::lock_guard<std::mutex> lk(g_prof_mu);
@@ -977,8 +992,44 @@ struct ProfScope {
 };
 }  // namespace
 
-void ring_profile_set(bool on) { g_prof_on = on; }
-bool ring_profile_on() { return g_prof_on; }
+void ring_note_kernel(const void* host_function) {
+  const int slot = t_kernel_slot;
+  if (slot >= 0 && slot < PROF_SLOTS) g_last_kernel[slot].store(host_function, std::memory_order_relaxed);
+}
+
+int ring_last_kernel_name(int id, char* buf, size_t n) {
+  if (!buf || n == 0) return -1;
+  buf[0] = 0;
+  if (id < 0 || id >= PROF_SLOTS) return -1;
+  const void* fn = g_last_kernel[id].load(std::memory_order_relaxed);
+  if (!fn) return 0;
+  const char* mangled = hipKernelNameRefByPtr(fn, nullptr);
+  if (!mangled) return -1;
+  int status = 0;
+  char* dem = abi::__cxa_demangle(mangled, nullptr, nullptr, &status);
+  std::string name = (status == 0 && dem) ? dem : mangled;
+  free(dem);
+  if (name.rfind("void ", 0) == 0) name.erase(0, 5);
+  // cut the parameter list: the first '(' outside the template argument list
+  int depth = 0;
+  for (size_t i = 0; i < name.size(); ++i) {
+    if (name[i] == '<') ++depth;
+    else if (name[i] == '>') --depth;
+    else if (name[i] == '(' && depth == 0) { name.erase(i); break; }
+  }
+  std::string out;
+  for (char c : name) if (c != ' ') out.push_back(c);
+  strncpy(buf, out.c_str(), n - 1);
+  buf[n - 1] = 0;
+  return (int)out.size();
+}
+
+void ring_profile_set(int stride) {
+  std::lock_guard<std::mutex> lk(g_prof_mu);
+  g_prof_stride = stride > 0 ? stride : 0;
+  for (long& c : g_prof_seen) c = 0;
+}
+bool ring_profile_on() { return g_prof_stride > 0; }
 
 hipError_t ring_profile_collect(double* ms, long long* launches) {
   std::vector<ProfRec> recs;
@@ -1031,7 +1082,7 @@ hipError_t ring_launch_pack2(const float* Wo, const float* Wa, int N, int k, int
   const size_t total = (size_t)(1 + k) * 4 * NC * 2 * NC * 64 * (out2 ? 2 : 1);
   const int blocks = (int)((total + 255) / 256 < 4096 ? (total + 255) / 256 : 4096);
   ProfScope prof(0, st);
-  hipLaunchKernelGGL(ring_pack_weights_kernel, dim3(blocks), dim3(256), 0, st, Wo, Wa, (bf16x8*)out, (bf16x8*)out2, N, k,
+  RING_LAUNCH(ring_pack_weights_kernel, dim3(blocks), dim3(256), 0, st, Wo, Wa, (bf16x8*)out, (bf16x8*)out2, N, k,
                      NC, transposed, split_k, scale0, shift0, transposed2, split_k2, scale2, shift2);
   return hipGetLastError();
 }
@@ -1074,7 +1125,7 @@ static hipError_t launch_stream(K kern, dim3 grid, size_t dyn, hipStream_t st, c
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)dyn);
     if (e != hipSuccess) return e;
   }
-  hipLaunchKernelGGL(kern, grid, dim3(256), dyn, st, a);
+  RING_LAUNCH(kern, grid, dim3(256), dyn, st, a);
   return hipGetLastError();
 }
 
@@ -1239,9 +1290,9 @@ hipError_t ring_launch_dw(const RingDwArgs& a, int NCv, hipStream_t st) {
     e = ring_launch_dw_tiled(a, NCv, st);   // every group's launch status, first failure wins
   } else {
     if (NCv == 1) {
-      hipLaunchKernelGGL((ring_dw_kernel<1, 4>), dim3(blocks), dim3(256), 0, st, a);
+      RING_LAUNCH((ring_dw_kernel<1, 4>), dim3(blocks), dim3(256), 0, st, a);
     } else {
-      RING_DISPATCH_NC(NCv, if constexpr (NC >= 2) hipLaunchKernelGGL((ring_dw_kernel<NC, 8>), dim3(blocks), dim3(256), 0, st, a));
+      RING_DISPATCH_NC(NCv, if constexpr (NC >= 2) RING_LAUNCH((ring_dw_kernel<NC, 8>), dim3(blocks), dim3(256), 0, st, a));
     }
     e = hipGetLastError();
   }
@@ -1249,6 +1300,6 @@ hipError_t ring_launch_dw(const RingDwArgs& a, int NCv, hipStream_t st) {
   if (e != hipSuccess) return e;   // the reduction must not sum partials that were never written
   const size_t per_z = (size_t)(a.k + 1) * NT * NT * 64;
   ProfScope prof(5, st);
-  hipLaunchKernelGGL(ring_dw_reduce_kernel, dim3((unsigned)((per_z + 255) / 256)), dim3(256), 0, st, a, NCv);
+  RING_LAUNCH(ring_dw_reduce_kernel, dim3((unsigned)((per_z + 255) / 256)), dim3(256), 0, st, a, NCv);
   return hipGetLastError();
 }

@@ -148,7 +148,20 @@ struct RingOptArgs {
 int ring_opt_chunks(size_t numel);
 hipError_t ring_launch_clip_adam(const RingOptArgs& a, float* workspace, hipStream_t st);
 
+// Which kernel ran.  The dispatch functions open a scope that names the slot (RINGATTR_K_*) their launches belong
+// to; RING_LAUNCH remembers the kernel it launches under the innermost open slot of the calling thread, and
+// ring_last_kernel_name gives that kernel's name ("ring_fwd_res256_kernel<1,true,true,false>": demangled, without
+// return type, parameter list and blanks), so that a benchmark can tell whether a stored counter summary is of the
+// kernel it has just timed.
+void ring_note_kernel(const void* host_function);
+int ring_last_kernel_name(int id, char* buf, size_t n);
+#define RING_LAUNCH(kern, grid, block, lds, st, ...)                       \
+  do {                                                                     \
+    ring_note_kernel(reinterpret_cast<const void*>(kern));                 \
+    hipLaunchKernelGGL(kern, grid, block, lds, st, __VA_ARGS__);           \
+  } while (0)
+
 // Optional event bracketing of launches (benchmark support).
-void ring_profile_set(bool on);
+void ring_profile_set(int stride);
 bool ring_profile_on();
 hipError_t ring_profile_collect(double* ms, long long* launches);

@@ -225,14 +225,20 @@ __global__ __launch_bounds__(512) void ring_fwd_res256_kernel(RingFwdArgs p) {
     gates_publish(gbuf, tid, B, bt, gs);
   }
 
-  // The LDS-resident slice is consumed in units of (tile cc, two K chunks), eight per step in the
-  // order f = 4*ph + 2*cc + j -> chunks 4*ph + 2*j + {0,1}; while unit f is multiplied, unit f+1 is
-  // fetched into the other register buffer.
+  // The LDS-resident slice is consumed in units f = 4*ph + 2*cc + j of two fragments (tile cc, chunks
+  // 4*ph + 2*j + {0,1}), eight units per step; fragment g = 2*f + u.  An LDS read takes about 130 cycles to land
+  // and a fragment's three MFMAs 48.  The unmasked variants (which have the registers to pin the reads early)
+  // run the fragments through a ring of four registers filled three fragments ahead of the MFMAs -- across
+  // tiles, halves and time steps alike, since the slice never changes; the masked ones fetch unit f + 1 while
+  // unit f is multiplied and leave the placement of the reads to the compiler.
   constexpr int UF = 2;
-  bf16x8 w0[2][UF];
-  auto unit_slot = [&](int f, int u) { return ((((f >> 1) & 1) * R_KCH) + (f >> 2) * HK + (f & 1) * UF + u) * 64; };
+  auto frag_slot = [&](int g) {
+    const int f = g >> 1, u = g & 1;
+    return ((((f >> 1) & 1) * R_KCH) + (f >> 2) * HK + (f & 1) * UF + u) * 64;
+  };
+  bf16x8 w0[4];
 #pragma unroll
-  for (int u = 0; u < UF; ++u) w0[0][u] = wl[unit_slot(0, u)];
+  for (int g = 0; g < (FULL ? 3 : UF); ++g) w0[g] = wl[frag_slot(g)];
   lds_barrier();   // A_0
 
   // History / F' / operand-copy stores of a finished step are not issued in one burst behind its
@@ -275,15 +281,23 @@ __global__ __launch_bounds__(512) void ring_fwd_res256_kernel(RingFwdArgs p) {
 
   f32x4 P[2][3];
   auto mfma_unit = [&](int f, const bf16x8 (&af)[HK]) {
-    const int cc = (f >> 1) & 1, ph = f >> 2, j = f & 1, fn = (f + 1) & 7;
+    const int cc = (f >> 1) & 1, ph = f >> 2, j = f & 1;
+    if constexpr (!FULL) {
 #pragma unroll
-    for (int u = 0; u < UF; ++u) w0[(f + 1) & 1][u] = wl[unit_slot(fn, u)];
+      for (int u = 0; u < UF; ++u) w0[((f + 1) & 1) * UF + u] = wl[frag_slot((2 * (f + 1) + u) & 15)];
+    }
 #pragma unroll
     for (int u = 0; u < UF; ++u) {
-      const int kl = j * UF + u, kc = ph * HK + kl;
-      P[cc][0] = mfma16(af[kl], w0[f & 1][u], P[cc][0]);
+      const int g = 2 * f + u, kl = j * UF + u, kc = ph * HK + kl;
+      if constexpr (FULL) {
+        w0[(g + 3) & 3] = wl[frag_slot((g + 3) & 15)];
+        // keep the read where it is: left alone it sinks towards its use and the distance is gone
+        __builtin_amdgcn_sched_barrier(0);
+      }
       P[cc][1] = mfma16(af[kl], wreg[0][cc][kc], P[cc][1]);
       P[cc][2] = mfma16(af[kl], wreg[1][cc][kc], P[cc][2]);
+      P[cc][0] = mfma16(af[kl], w0[g & 3], P[cc][0]);
+      if constexpr (FULL) __builtin_amdgcn_sched_barrier(0);
     }
   };
   // K chunks 0..3 (ph = 0, from the E buffer of this step's parity) or 4..7 (ph = 1, from the L half);
@@ -298,11 +312,16 @@ __global__ __launch_bounds__(512) void ring_fwd_res256_kernel(RingFwdArgs p) {
 #pragma unroll
       for (int cc = 0; cc < 2; ++cc) P[cc][0] = P[cc][1] = P[cc][2] = z;
     }
+    // The two waves of a SIMD share one issue port for vector-ALU and MFMA instructions, and the arbiter serves
+    // the older wave first: without a hint a wave in its (long, dense) activation starves the other one's MFMAs
+    // and the matrix pipe idles until the activation is over.  A wave that is contracting asks for priority.
+    __builtin_amdgcn_s_setprio(3);
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       if constexpr (decltype(emit)::value) emit_store(ts, 4 * ph + j);
       mfma_unit(4 * ph + j, af);
     }
+    __builtin_amdgcn_s_setprio(0);
   };
   // x[e][cc] = P0 + a0*P1 + a1*P2 with the gates of step t (P0 already holds J0*rowsum + J1*(Wo r))
   auto preactivation = [&](int t, float (&x)[4][2]) {
@@ -619,9 +638,20 @@ __global__ __launch_bounds__(256) void ring_bptt_res256_kernel(RingBpttArgs p) {
   GateStage gs;
   gates_fetch(p.A, T, B, bt, 0, -1, tid, gs);
   gates_publish(gbuf, tid, B, bt, gs);
-  bf16x8 w0[2][R_KCH / 2];
+  // The LDS-resident slice is consumed one fragment at a time.  PAIR (the variants with registers to spare): two
+  // tiles are contracted together, fragment g of a step = tile pair g/16, K chunk (g/2)%8, tile g%2 of the pair,
+  // through a ring of eight registers filled seven fragments ahead across tiles and steps; otherwise tile by tile
+  // in half-tile units of four fragments, one unit ahead.
+  constexpr bool PAIR = FULL && !(LOSS && GA);
+  auto frag_slot = [&](int g) { return ((2 * (g >> 4) + (g & 1)) * R_KCH + ((g >> 1) & 7)) * 64; };
+  bf16x8 w0[8];
+  if constexpr (PAIR) {
 #pragma unroll
-  for (int u = 0; u < R_KCH / 2; ++u) w0[0][u] = wl[u * 64];
+    for (int g = 0; g < 7; ++g) w0[g] = wl[frag_slot(g)];
+  } else {
+#pragma unroll
+    for (int u = 0; u < R_KCH / 2; ++u) w0[u] = wl[u * 64];
+  }
   // (the first lds_barrier inside the loop also publishes the gates)
 
   bf16x4 held[R_NC];   // MERGE: the odd step's bf16 g, waiting for its even partner
@@ -709,27 +739,9 @@ __global__ __launch_bounds__(256) void ring_bptt_res256_kernel(RingBpttArgs p) {
 #pragma unroll
         for (int e = 0; e < 4; ++e) gate[e] = gb[e];
       }
-#pragma unroll
-      for (int c = 0; c < R_NC; ++c) {
-        // the ungated chain starts from the term that needs no product, (1 - alpha) * G; J0 * sum(g) comes with
-        // the product itself (the packed fragments hold J1 * Wo^T + J0)
-        f32x4 P0 = {oma * G[0][c], oma * G[1][c], oma * G[2][c], oma * G[3][c]};
-        f32x4 P1 = {0.f, 0.f, 0.f, 0.f}, P2 = P1;
-#pragma unroll
-        for (int h = 0; h < 2; ++h) {
-          // stage the next half tile of the LDS-resident matrix (wraps to tile 0 of the next step)
-          constexpr int HK = R_KCH / 2;
-          const int f = 2 * c + h, fn = (f + 1) & 7;
-#pragma unroll
-          for (int u = 0; u < HK; ++u) w0[(f + 1) & 1][u] = wl[(fn * HK + u) * 64];
-#pragma unroll
-          for (int u = 0; u < HK; ++u) {
-            const int kc = h * HK + u;
-            P0 = mfma16(af[kc], w0[f & 1][u], P0);
-            P1 = mfma16(af[kc], wreg[0][c][kc], P1);
-            P2 = mfma16(af[kc], wreg[1][c][kc], P2);
-          }
-        }
+      // the ungated chain starts from the term that needs no product, (1 - alpha) * G; J0 * sum(g) comes with
+      // the product itself (the packed fragments hold J1 * Wo^T + J0)
+      auto tile_epilogue = [&](int c, const f32x4& P0, const f32x4& P1, const f32x4& P2) {
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           float x = fmaf(gate[e][0], P1[e], P0[e]);
@@ -745,6 +757,54 @@ __global__ __launch_bounds__(256) void ring_bptt_res256_kernel(RingBpttArgs p) {
             ga[0][e] = fmaf(P1[e], rv, ga[0][e]);
             ga[1][e] = fmaf(P2[e], rv, ga[1][e]);
           }
+        }
+      };
+      if constexpr (PAIR) {
+#pragma unroll
+        for (int cp = 0; cp < R_NC / 2; ++cp) {
+          f32x4 P[2][3];
+#pragma unroll
+          for (int j = 0; j < 2; ++j) {
+            const int c = 2 * cp + j;
+            P[j][0] = f32x4{oma * G[0][c], oma * G[1][c], oma * G[2][c], oma * G[3][c]};
+            P[j][1] = f32x4{0.f, 0.f, 0.f, 0.f};
+            P[j][2] = P[j][1];
+          }
+#pragma unroll
+          for (int kc = 0; kc < R_KCH; ++kc)
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+              const int c = 2 * cp + j, g = (cp * R_KCH + kc) * 2 + j;
+              w0[(g + 7) & 7] = wl[frag_slot((g + 7) & 31)];
+              __builtin_amdgcn_sched_barrier(0);   // the read stays seven fragments ahead of its use
+              P[j][1] = mfma16(af[kc], wreg[0][c][kc], P[j][1]);
+              P[j][2] = mfma16(af[kc], wreg[1][c][kc], P[j][2]);
+              P[j][0] = mfma16(af[kc], w0[g & 7], P[j][0]);
+            }
+#pragma unroll
+          for (int j = 0; j < 2; ++j) tile_epilogue(2 * cp + j, P[j][0], P[j][1], P[j][2]);
+        }
+      } else {
+#pragma unroll
+        for (int c = 0; c < R_NC; ++c) {
+          f32x4 P0 = {oma * G[0][c], oma * G[1][c], oma * G[2][c], oma * G[3][c]};
+          f32x4 P1 = {0.f, 0.f, 0.f, 0.f}, P2 = P1;
+#pragma unroll
+          for (int h = 0; h < 2; ++h) {
+            // stage the next half tile of the LDS-resident matrix (wraps to tile 0 of the next step)
+            constexpr int HK = R_KCH / 2;
+            const int f = 2 * c + h, fn = (f + 1) & 7;
+#pragma unroll
+            for (int u = 0; u < HK; ++u) w0[((f + 1) & 1) * HK + u] = wl[(fn * HK + u) * 64];
+#pragma unroll
+            for (int u = 0; u < HK; ++u) {
+              const int kc = h * HK + u;
+              P0 = mfma16(af[kc], w0[(f & 1) * HK + u], P0);
+              P1 = mfma16(af[kc], wreg[0][c][kc], P1);
+              P2 = mfma16(af[kc], wreg[1][c][kc], P2);
+            }
+          }
+          tile_epilogue(c, P0, P1, P2);
         }
       }
       if constexpr (GA) {
@@ -788,7 +848,7 @@ static hipError_t launch_fwd_variant(const RingFwdArgs& a, hipStream_t st) {
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                                      (int)R8_LDS_BYTES);
   if (e != hipSuccess) return e;
-  hipLaunchKernelGGL(kern, dim3(a.nbt), dim3(512), R8_LDS_BYTES, st, a);
+  RING_LAUNCH(kern, dim3(a.nbt), dim3(512), R8_LDS_BYTES, st, a);
   return hipGetLastError();
 }
 
@@ -819,7 +879,7 @@ static hipError_t launch_bptt_variant(const RingBpttArgs& a, hipStream_t st) {
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                                      (int)R_LDS_BYTES);
   if (e != hipSuccess) return e;
-  hipLaunchKernelGGL(kern, dim3(a.nbt), dim3(256), R_LDS_BYTES, st, a);
+  RING_LAUNCH(kern, dim3(a.nbt), dim3(256), R_LDS_BYTES, st, a);
   return hipGetLastError();
 }
 

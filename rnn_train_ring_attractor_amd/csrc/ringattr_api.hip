@@ -663,7 +663,14 @@ static int clip_adam_impl(int n_tensors, void* const* params, void* const* grads
 }
 
 int ringattr_profile_enable(int on) {
-  ring_profile_set(on != 0);
+  ring_profile_set(on);
+  return RINGATTR_OK;
+}
+
+int ringattr_last_kernel_name(int kernel, char* buf, size_t buf_bytes) {
+  if (!buf || buf_bytes == 0) return fail(RINGATTR_ERR_INVALID, "ringattr_last_kernel_name: null buffer");
+  if (kernel < 0 || kernel >= RINGATTR_NUM_KERNELS) return fail(RINGATTR_ERR_INVALID, "ringattr_last_kernel_name: no such kernel slot");
+  if (ring_last_kernel_name(kernel, buf, buf_bytes) < 0) return fail(RINGATTR_ERR_HIP, "ringattr_last_kernel_name: the runtime does not know the kernel");
   return RINGATTR_OK;
 }
 

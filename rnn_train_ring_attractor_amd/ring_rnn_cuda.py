@@ -37,6 +37,13 @@ def ring_rnn_cuda_func(action_signal, Wa, J0, J1, Wo, r_init, alpha, activation=
     return RingRnnCudaFunc.apply(action_signal, Wa, J0, J1, Wo, r_init, alpha, activation, torch.is_grad_enabled())
 
 
+# Store or recompute.  False (default): a forward that a backward can follow also writes the derivative record and the
+# bf16 operand copy (ringattr_saved_bytes: 4 bytes per state element and step) for the backward to read.  True: the
+# forward writes only bump_history, as the reference's does (cpp/ring_rnn_cuda.py:68-78), and the backward recomputes
+# both from it before the reverse-time loop (the reference recomputes re in every backward,
+# cpp/kernels/bwd_mixed_precision_aggressive.cuh:53-269): no saved buffer is held between forward and backward.
+RECOMPUTE_IN_BACKWARD = False
+
 DRIVEN_ATTR = "_ring_driven_channels"     # set on zero-padded action signals by the host helper that builds them
 
 
@@ -100,7 +107,7 @@ class RingRnnCudaFunc(Function):
         needs_grad = grad_mode is not False and any(ctx.needs_input_grad[i] for i in (0, 1, 4, 5))
         ctx.extra_inputs = 0 if grad_mode is None else 1
         saved = None
-        if needs_grad:
+        if needs_grad and not RECOMPUTE_IN_BACKWARD:
             saved = torch.empty(saved_nbytes(N, a_dim, seq_len, batch_size), dtype=torch.uint8,
                                 device=action_signal.device)
         fwd_cuda.fwd(A=action_signal, Wa=Wa_c, J0=J0, J1=J1, Wo=Wo_c, r_init=r0, bump_history=bump_history,
