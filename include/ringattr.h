@@ -97,8 +97,13 @@ RINGATTR_API int ringattr_fwd_noalloc(const void* A, const void* Wa, float J0, f
  * recurrence again from r_init, which reproduces the forward's own numbers.
  * grad_A [B,T,k] and grad_r_init [B,N] are optional outputs (NULL = skip), written
  * rather than accumulated; the reference returns None for both
- * (cpp/ring_rnn_cuda.py:144).  Asking for grad_A (a_dim <= 48) adds one read of
- * bump_history and runs the BPTT on the weight-streaming kernel for every N.
+ * (cpp/ring_rnn_cuda.py:144).  grad_A comes out of the BPTT kernel itself up to N = 512 (the
+ * weight-resident kernel reads the bf16 operand copy of r_prev with the step's other inputs; the persistent
+ * streaming kernel stages its per-channel shares in LDS, which limits it to a_dim <= 48) and from a pass of its own
+ * after the BPTT steps on the step-per-launch kernels (wide rings and small batches; any a_dim, seq_len <= 65535).
+ * With a saved buffer, the buffer must be the one the forward filled, at the address it filled it, and the
+ * weights must be unchanged since (the forward's transposed weight copy inside it is reused on an exact match of
+ * shape, J0, J1 and weight addresses; anything else is repacked).
  * accumulate != 0: grad_Wa / grad_Wo are added to, as in the reference, whose caller zeroes them first
  * (cpp/ring_rnn_cuda.py:98-99); accumulate == 0: they are overwritten and need no zeroing. */
 RINGATTR_API int ringattr_bwd(const void* grad_output, const void* A, const void* Wa, float J0, float J1,
@@ -181,13 +186,19 @@ RINGATTR_API int ringattr_gain_bwd(const void* base_signal, const void* params, 
  * train_general_ring_no_gain.py:176-229) and create_initial_bump (train/train_ring_attractor.py:21-52).  Same
  * distributions; the random stream is the library's own counter-based generator, a function of `seed` only
  * (repeatable bit for bit, independent of launch geometry).
+ *   zero_padding_start_ratio   the first int(seq_len * ratio) steps of every trial are zero; a double, and the
+ *                     product is formed in double precision, so the count is the one Python's int() gives
  *   zero_ratios       HOST array of 1..8 floats (per trial one is picked uniformly)
  *   spread_action     0: channels 0 / 1 = relu(-av) / relu(av), others zero; 1: relu(av * linspace(-1, 1, a_dim))
  *   bump_kind, bump_param   0: Gaussian on the circular distance, width N / bump_param (the reference, 10);
  *                           1: von Mises exp(kappa cos(phi_i - angle)), kappa = bump_param; both L2-normalised
  *   av, angle [B,T]; action_signal [B,T,a_dim]; r_init [B,N] or NULL (all fp32 device pointers, outputs) */
+/* Number of leading zero steps the generator gives every trial: int(seq_len * zero_padding_start_ratio) as the
+ * reference's Python evaluates it (utils/generate_av_integration_data.py:21); -1 for arguments out of range.
+ * Host arithmetic only (callable without a GPU). */
+RINGATTR_API int ringattr_generator_initial_zeros(int seq_len, double zero_padding_start_ratio);
 RINGATTR_API int ringattr_generate_inputs(unsigned long long seed, int N, int a_dim, int seq_len, int batch_size,
-                      float zero_padding_start_ratio, const float* zero_ratios, int n_zero_ratios, float max_av,
+                      double zero_padding_start_ratio, const float* zero_ratios, int n_zero_ratios, float max_av,
                       int spread_action, int bump_kind, float bump_param,
                       void* av, void* angle, void* action_signal, void* r_init, void* stream);
 

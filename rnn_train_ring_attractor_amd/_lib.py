@@ -50,7 +50,8 @@ PROTOTYPES = {
     "ringattr_gain_fwd": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p]),
     "ringattr_gain_bwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
                                   c_void_p, c_size_t, c_void_p]),
-    "ringattr_generate_inputs": (c_int, [ctypes.c_ulonglong, c_int, c_int, c_int, c_int, c_float,
+    "ringattr_generator_initial_zeros": (c_int, [c_int, ctypes.c_double]),
+    "ringattr_generate_inputs": (c_int, [ctypes.c_ulonglong, c_int, c_int, c_int, c_int, ctypes.c_double,
                                          ctypes.POINTER(c_float), c_int, c_float, c_int, c_int, c_float,
                                          c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
     "ringattr_clip_adam_workspace_bytes": (c_size_t, [c_int, ctypes.POINTER(c_size_t)]),

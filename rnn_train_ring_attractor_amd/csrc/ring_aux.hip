@@ -4,7 +4,7 @@
 // Input generator (utils/generate_av_integration_data.py:11-58, root train_general_ring_no_gain.py:176-229,
 // train/train_ring_attractor.py:21-52 of the reference): angular-velocity trials, their integrated angle, the action
 // signal and the initial bump, written where the time loop reads them, so that a training or benchmark step stages
-// nothing from the host.  Per trial: the first int(T * start_ratio) steps are zero; of the remaining `rest` steps
+// nothing from the host.  Per trial: the first n_initial_zeros steps are zero; of the remaining `rest` steps
 // exactly rest - floor(rest * zero_ratio) randomly placed ones carry U(-max_av, max_av) draws (zero_ratio picked
 // uniformly from a list); angle[0] = U(0, 2 pi), angle[t] = (angle[0] + sum_{s<t} av[s]) mod 2 pi.  The reference
 // draws a random permutation per trial (argsort of uniform keys) and keeps the first n positions; choosing each
@@ -53,7 +53,7 @@ __global__ __launch_bounds__(256) void ring_generate_trials_kernel(RingGenArgs p
   __shared__ float cand[GEN_TCH][GEN_TRIALS + 1];   // candidate velocity;               then the step's velocity
   const int tid = threadIdx.x, b0 = blockIdx.x * GEN_TRIALS;
   const int T = p.T, k = p.k;
-  const int n0 = (int)((float)T * p.start_ratio);
+  const int n0 = p.n_initial_zeros;
   const int rest = T - n0;
   const float two_pi = 6.283185307179586f;
   // per-trial state of the sequential phase (threads 0 .. GEN_TRIALS-1)

@@ -123,7 +123,8 @@ struct RingGenArgs {
   float* r_init;         // [B,N] or null
   float ratios[8];       // zero ratios to pick from
   int n_ratios;
-  float start_ratio, max_av, bump_param;
+  int n_initial_zeros;   // leading zero steps of every trial
+  float max_av, bump_param;
   int spread;            // 0: (L, R) in channels 0, 1, zeros elsewhere; 1: relu(av * linspace(-1, 1, k))
   int bump_kind;         // 0: Gaussian of width N / bump_param on the circular distance; 1: von Mises, kappa = bump_param
   int N, k, T, B;

@@ -94,29 +94,46 @@ int hip_fail(hipError_t e, const char* what) {
   return fail(RINGATTR_ERR_HIP, "%s: %s", what, hipGetErrorString(e));
 }
 
-// Which kernel family filled a saved buffer: the transposed weight copy behind the saved activations has J0 and J1
-// folded into Wo for the weight-resident BPTT kernel and is plain for the streaming one.  The forward notes what it
-// wrote under the buffer's address; a backward that finds no matching note (another process state, a copied
-// buffer, RINGATTR_STREAMING changed in between) packs its own copy instead of trusting the one in the buffer.
+// What a forward left in a saved buffer.  The transposed weight copy behind the saved activations has J0 and J1
+// folded into Wo for the weight-resident BPTT kernel and is plain for the streaming one, and the derivative record of
+// the step-per-launch family has its own layout.  The forward notes, under the buffer's address, the family, the
+// shape, J0, J1 and the weight tensors' addresses it packed; a backward trusts the transposed copy in the buffer only
+// if every one of them matches its own arguments, and packs its own copy otherwise (no note: another process state
+// or a copied buffer; a stale note: the address was reused; RINGATTR_STREAMING / RINGATTR_BLOCK changed in between;
+// other J0, J1 or weights).  A buffer must not be copied or moved between the forward and the backward that
+// consumes it, and the weights must not change in between (pass saved = NULL to recompute instead).
 constexpr int kSavedNotes = 256;
-struct SavedNote { const void* ptr; int family; };   // family: 1 streaming, 2 weight-resident, 3 step-per-launch
+struct SavedNote {
+  const void* ptr;
+  int family;   // 1 streaming, 2 weight-resident, 3 step-per-launch
+  int N, k, T, B;
+  float J0, J1;
+  const void *Wo, *Wa;
+};
 std::mutex g_saved_mu;
 SavedNote g_saved_notes[kSavedNotes] = {};
 int g_saved_next = 0;
 
-void saved_note_put(const void* ptr, int family) {
+void saved_note_put(const SavedNote& note) {
   std::lock_guard<std::mutex> lk(g_saved_mu);
   for (auto& n : g_saved_notes)
-    if (n.ptr == ptr) { n.family = family; return; }
-  g_saved_notes[g_saved_next] = SavedNote{ptr, family};
+    if (n.ptr == note.ptr) { n = note; return; }
+  g_saved_notes[g_saved_next] = note;
   g_saved_next = (g_saved_next + 1) % kSavedNotes;
 }
 
-int saved_note_get(const void* ptr) {
+// The note under ptr (family 0 if there is none).
+SavedNote saved_note_get(const void* ptr) {
   std::lock_guard<std::mutex> lk(g_saved_mu);
   for (const auto& n : g_saved_notes)
-    if (n.ptr == ptr) return n.family;
-  return 0;
+    if (n.ptr == ptr) return n;
+  return SavedNote{};
+}
+
+bool saved_note_matches(const SavedNote& n, int family, int N, int k, int T, int B, float J0, float J1, const void* Wo,
+                        const void* Wa) {
+  return n.family == family && n.N == N && n.k == k && n.T == T && n.B == B && n.J0 == J0 && n.J1 == J1 && n.Wo == Wo &&
+         n.Wa == Wa;
 }
 
 // Device address of `scratch` on the current device, looked up once per device.
@@ -231,7 +248,9 @@ static int fwd_impl(const void* A, const void* Wa, float J0, float J1, const voi
   hipError_t e = ring_launch_pack2((const float*)Wo, (const float*)Wa, N, a_dim, g.NC, workspace, 0, resident, s0, h0,
                                    wpack_t, 1, 0, s0, h0, st);
   if (e != hipSuccess) return hip_fail(e, "pack weights");
-  if (saved) saved_note_put(saved, ring_uses_step_kernels(N, a_dim, g.NC, g.nbt) ? 3 : (resident ? 2 : 1));
+  if (saved)
+    saved_note_put(SavedNote{saved, ring_uses_step_kernels(N, a_dim, g.NC, g.nbt) ? 3 : (resident ? 2 : 1), N, a_dim,
+                             seq_len, batch_size, J0, J1, Wo, Wa});
 
   RingFwdArgs a;
   a.A = (const float*)A;
@@ -325,9 +344,12 @@ static int bwd_impl(const char* who, const void* grad_output, const void* loss_w
   if ((rc = check_act(activation_type))) return rc;
   if (!A || !Wa || !Wo || !bump_history || !r_init || !grad_Wa || !grad_Wo)
     return fail(RINGATTR_ERR_INVALID, "%s: null tensor pointer", who);
-  if (grad_A && (size_t)2 * a_dim * 64 * sizeof(float) > 24 * 1024)
-    return fail(RINGATTR_ERR_INVALID, "%s: grad_A is supported for a_dim <= 48 (got %d)", who, a_dim);
   const bool step_family = ring_uses_step_kernels(N, a_dim, g.NC, g.nbt);
+  // the persistent streaming BPTT kernel stages the per-channel shares of dL/dA in 24 KiB of LDS; the
+  // step-per-launch families form dL/dA in a pass of their own that has no such stage
+  if (grad_A && !step_family && !ring_uses_resident(N, a_dim) && (size_t)2 * a_dim * 64 * sizeof(float) > 24 * 1024)
+    return fail(RINGATTR_ERR_INVALID, "%s: grad_A on the persistent streaming kernels (N <= 512 at this batch) is "
+                "supported for a_dim <= 48 (got %d)", who, a_dim);
   if (step_family && grad_A && seq_len > 65535)
     return fail(RINGATTR_ERR_INVALID, "%s: grad_A on the step-per-launch kernels supports seq_len <= 65535", who);
   if (!aligned16(grad_output) || !aligned16(A) || !aligned16(Wa) || !aligned16(Wo) || !aligned16(bump_history) ||
@@ -394,11 +416,12 @@ static int bwd_impl(const char* who, const void* grad_output, const void* loss_w
   const bool bptt_resident = resident;
   hipError_t e = hipSuccess;
   const int family = step_family ? 3 : (bptt_resident ? 2 : 1);
-  const int noted = saved ? saved_note_get(saved) : 0;
+  const SavedNote note = saved ? saved_note_get(saved) : SavedNote{};
+  const int noted = note.family;
   if (noted != 0 && (noted == 3) != (family == 3))
     return fail(RINGATTR_ERR_INVALID, "%s: the saved buffer was filled by the other kernel family (its derivative record "
                 "has a different layout); run forward and backward under the same RINGATTR_BLOCK setting", who);
-  if (saved && noted == family) {
+  if (saved && saved_note_matches(note, family, N, a_dim, seq_len, batch_size, J0, J1, Wo, Wa)) {
     // the forward left the transposed copy, in the form this BPTT kernel expects, behind the saved activations
     wb = (char*)const_cast<void*>(saved) + g.side_bytes + g.pair_bytes;
   } else {
@@ -556,8 +579,15 @@ int ringattr_gain_bwd(const void* base_signal, const void* params, const void* g
   return RINGATTR_OK;
 }
 
+int ringattr_generator_initial_zeros(int seq_len, double zero_padding_start_ratio) {
+  // int(seq_len * ratio) with the product in double precision, as Python evaluates it
+  // (utils/generate_av_integration_data.py:21); a float product differs by one for some (length, ratio) pairs
+  if (seq_len <= 0 || !(zero_padding_start_ratio >= 0.0 && zero_padding_start_ratio <= 1.0)) return -1;
+  return (int)((double)seq_len * zero_padding_start_ratio);
+}
+
 int ringattr_generate_inputs(unsigned long long seed, int N, int a_dim, int seq_len, int batch_size,
-                             float zero_padding_start_ratio, const float* zero_ratios, int n_zero_ratios, float max_av,
+                             double zero_padding_start_ratio, const float* zero_ratios, int n_zero_ratios, float max_av,
                              int spread_action, int bump_kind, float bump_param, void* av, void* angle,
                              void* action_signal, void* r_init, void* stream) {
   if (N <= 0 || a_dim <= 0 || seq_len <= 0 || batch_size <= 0)
@@ -565,7 +595,7 @@ int ringattr_generate_inputs(unsigned long long seed, int N, int a_dim, int seq_
                 seq_len, batch_size);
   if (!zero_ratios || n_zero_ratios < 1 || n_zero_ratios > 8)
     return fail(RINGATTR_ERR_INVALID, "ringattr_generate_inputs: between 1 and 8 zero ratios (host array) are needed");
-  if (!(zero_padding_start_ratio >= 0.f && zero_padding_start_ratio <= 1.f))
+  if (!(zero_padding_start_ratio >= 0.0 && zero_padding_start_ratio <= 1.0))
     return fail(RINGATTR_ERR_INVALID, "ringattr_generate_inputs: zero_padding_start_ratio must lie in [0, 1]");
   if ((bump_kind != 0 && bump_kind != 1) || !(bump_param > 0.f))
     return fail(RINGATTR_ERR_INVALID, "ringattr_generate_inputs: bump_kind is 0 (Gaussian) or 1 (von Mises), bump_param > 0");
@@ -578,7 +608,7 @@ int ringattr_generate_inputs(unsigned long long seed, int N, int a_dim, int seq_
   a.r_init = (float*)r_init;
   for (int i = 0; i < 8; ++i) a.ratios[i] = i < n_zero_ratios ? zero_ratios[i] : 0.f;
   a.n_ratios = n_zero_ratios;
-  a.start_ratio = zero_padding_start_ratio;
+  a.n_initial_zeros = ringattr_generator_initial_zeros(seq_len, zero_padding_start_ratio);
   a.max_av = max_av;
   a.bump_param = bump_param;
   a.spread = spread_action ? 1 : 0;

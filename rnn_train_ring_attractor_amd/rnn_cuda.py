@@ -88,6 +88,20 @@ def _ptr(t):
     return None if t is None else t.data_ptr()
 
 
+def _workspace(nbytes, device, stream):
+    """Scratch for one call, from torch's caching allocator.  The allocator hands a freed block back to later
+    allocations on the stream it was ALLOCATED on (the current one) as soon as the tensor is dropped, which is at
+    the end of the call, long before the kernels have run.  On the current stream that is safe (the next user's
+    work is queued behind the kernels); when the caller passes another stream through `stream=`, the block is
+    marked as in use on that stream too, so it is not recycled before the work queued there has finished."""
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=device)
+    if stream is not None:
+        s = stream if isinstance(stream, torch.cuda.Stream) else torch.cuda.ExternalStream(int(stream), device=device)
+        if s != torch.cuda.current_stream(device):
+            ws.record_stream(s)
+    return ws
+
+
 def saved_nbytes(N, a_dim, seq_len, batch_size) -> int:
     """Size of the opaque saved-activations buffer (uint8 elements)."""
     return int(_lib.load().ringattr_saved_bytes(N, a_dim, seq_len, batch_size))
@@ -118,7 +132,7 @@ class _Fwd:
             ws_bytes = lib.ringattr_fwd_workspace_bytes(N, k, T, B)
             if ws_bytes == 0:
                 _lib.check(1)
-            ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+            ws = _workspace(ws_bytes, dev, stream)
             if loss is None:
                 rc = lib.ringattr_fwd(_ptr(A), _ptr(Wa), J0, J1, _ptr(Wo), _ptr(r_init), _ptr(bump_history), alpha,
                                       N, k, T, B, act, _ptr(saved), _ptr(ws), ws_bytes, _stream_ptr(stream, dev))
@@ -193,7 +207,7 @@ class _Bwd:
                 ws_bytes = lib.ringattr_bwd_workspace_bytes(N, k, T, B, 1 if saved is not None else 0)
                 if ws_bytes == 0:
                     _lib.check(1)
-                ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+                ws = _workspace(ws_bytes, dev, stream)
                 rc = lib.ringattr_bwd_loss(_ptr(loss_workspace), _ptr(loss_upstream), _ptr(A), _ptr(Wa), J0, J1, _ptr(Wo),
                                            _ptr(bump_history), _ptr(r_init), _ptr(grad_Wa), _ptr(grad_Wo), alpha, N, k, T,
                                            B, act, 1 if accumulate else 0, _ptr(saved), _ptr(grad_A), _ptr(grad_r_init), _ptr(ws), ws_bytes,
@@ -204,7 +218,7 @@ class _Bwd:
             ws_bytes = lib.ringattr_bwd_workspace_bytes(N, k, T, B, 1 if saved is not None else 0)
             if ws_bytes == 0:
                 _lib.check(1)
-            ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+            ws = _workspace(ws_bytes, dev, stream)
             rc = lib.ringattr_bwd(_ptr(grad_output), _ptr(A), _ptr(Wa), J0, J1, _ptr(Wo), _ptr(bump_history),
                                   _ptr(r_init), _ptr(grad_Wa), _ptr(grad_Wo), alpha, N, k, T, B, act,
                                   1 if accumulate else 0, _ptr(saved), _ptr(grad_A), _ptr(grad_r_init), _ptr(ws), ws_bytes,

@@ -132,3 +132,31 @@ def test_operator_rejects_unknown_activation_before_touching_the_gpu():
 
 def test_saved_buffer_size_helper_matches_library():
     assert rnn_cuda.saved_nbytes(256, 2, 120, 4096) == _lib.load().ringattr_saved_bytes(256, 2, 120, 4096)
+
+
+def test_generator_leading_zero_count_is_pythons_over_a_grid():
+    """The device generator's count of leading zero steps is int(seq_len * ratio) with the product in double
+    precision, as the reference's Python forms it (utils/generate_av_integration_data.py:21).  A float32 product is
+    off by one for some pairs (seq_len = 180, ratio 0.35: 63 against 62; ratio 0.7 at seq_len = 10: 6 against 7), so
+    the library takes the ratio as a double and the count is checked here against Python's own over a grid, and
+    against the host generator's output (host.generate_av_integration_data_ultra_fast, the reference's construction)."""
+    import numpy as np
+    import torch
+    from rnn_train_ring_attractor_amd import _lib, host
+    lib = _lib.load()
+    ratios = [0.0, 0.01, 0.05, 0.1, 0.15, 0.2, 0.3, 0.35, 0.5, 0.7, 0.9, 1.0]
+    float_product_differs = 0
+    for ratio in ratios:
+        for T in range(1, 4097):
+            want = int(T * ratio)
+            assert lib.ringattr_generator_initial_zeros(T, ratio) == want, (T, ratio)
+            float_product_differs += int(int(np.float32(T) * np.float32(ratio)) != want)
+    assert float_product_differs > 0          # the grid contains the pairs a float product gets wrong
+    assert lib.ringattr_generator_initial_zeros(180, 0.35) == 62 and lib.ringattr_generator_initial_zeros(10, 0.7) == 7
+    assert lib.ringattr_generator_initial_zeros(0, 0.1) == -1 and lib.ringattr_generator_initial_zeros(10, 1.5) == -1
+    torch.manual_seed(0)
+    for T, ratio in ((180, 0.35), (10, 0.7), (120, 0.1), (77, 0.3)):
+        av, _ = host.generate_av_integration_data_ultra_fast(64, T, ratio, [0.0])     # ratio 0: every later step drawn
+        n0 = lib.ringattr_generator_initial_zeros(T, ratio)
+        assert torch.all(av[:, :n0] == 0)
+        assert torch.all(av[:, n0:] != 0)

@@ -60,6 +60,18 @@ def test_generated_inputs_follow_the_reference_construction(B, T, k, N, pad, bum
         assert abs(a0.mean() - 0.5) <= 0.02 and abs(a0.var() - 1.0 / 12.0) <= 0.01
 
 
+@pytest.mark.parametrize("T,ratio", [(180, 0.35), (10, 0.7), (120, 0.01)])
+def test_generator_leading_zeros_are_pythons_count(T, ratio, gpu_device):
+    """int(T * ratio) as Python forms it (a float32 product gives 63 and 6 for the first two pairs instead of 62
+    and 7); with a zero ratio of 0 every later step is drawn, so the leading zeros are exactly the count."""
+    from rnn_train_ring_attractor_amd import generate_inputs
+    print(f"[case] generator leading zeros T={T} ratio={ratio}", flush=True)
+    av = generate_inputs(5, 256, T, 64, 2, zero_padding_start_ratio=ratio, zero_ratios_in_rest=[0.0])[0].cpu().numpy()
+    n0 = int(T * ratio)
+    assert np.all(av[:, :n0] == 0.0)
+    assert np.all(av[:, n0:] != 0.0)
+
+
 def test_generated_inputs_drive_the_operator(gpu_device):
     """Generated tensors go straight into the time loop (zero-padded action channels state the driven ones)."""
     from rnn_train_ring_attractor_amd import generate_inputs, ring_rnn_cuda_func

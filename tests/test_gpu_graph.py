@@ -142,3 +142,65 @@ def test_two_streams_interleaved_give_the_sequential_results(gpu_device):
         for got in together[i]:
             for x, y in zip(got, alone[i]):
                 assert torch.equal(x, y)
+
+
+def test_explicit_stream_keyword_with_allocator_churn_on_the_current_stream(gpu_device):
+    """`stream=` of fwd_cuda.fwd / bwd_cuda.bwd: the work goes to a stream that is NOT torch's current one.  The
+    scratch the calls take from torch's caching allocator is freed when they return, long before their kernels have
+    run; it must not be handed to allocations on the current stream meanwhile.  The side stream is kept busy so that
+    the operator's kernels are still queued while the current stream allocates, fills and frees blocks of exactly the
+    scratch sizes; results must equal those of the same calls on the current stream, bit for bit."""
+    from rnn_train_ring_attractor_amd import _lib
+    from rnn_train_ring_attractor_amd.rnn_cuda import fwd_cuda, bwd_cuda, saved_nbytes
+    B, T, k, N = 512, 24, 2, 256
+    print(f"[case] explicit stream= B={B} T={T} k={k} N={N} gelu", flush=True)
+    p = make_problem(81, B, T, k, N)
+
+    def dev(x):
+        return torch.tensor(x, device=gpu_device)
+
+    A, Wa, Wo, r0, G = dev(p["A"]), dev(p["Wa"]), dev(p["Wo"]), dev(p["r0"]), dev(p["G"])
+    lib = _lib.load()
+    sizes = [int(lib.ringattr_fwd_workspace_bytes(N, k, T, B)), int(lib.ringattr_bwd_workspace_bytes(N, k, T, B, 1))]
+
+    def run(stream, churn):
+        hist = torch.empty(T, B, N, device=gpu_device)
+        saved = torch.empty(saved_nbytes(N, k, T, B), dtype=torch.uint8, device=gpu_device)
+        gWa, gWo = torch.empty_like(Wa), torch.empty_like(Wo)
+        fwd_cuda.fwd(A=A, Wa=Wa, J0=-0.05, J1=0.4, Wo=Wo, r_init=r0, bump_history=hist, alpha=0.15,
+                     activation_type=1, saved=saved, stream=stream)
+        if churn:
+            churn()
+        bwd_cuda.bwd(grad_output=G, A=A, Wa=Wa, J0=-0.05, J1=0.4, Wo=Wo, bump_history=hist, r_init=r0, grad_Wa=gWa,
+                     grad_Wo=gWo, alpha=0.15, activation_type=1, saved=saved, accumulate=False, stream=stream)
+        if churn:
+            churn()
+        return hist, gWa, gWo
+
+    want = run(None, None)
+    torch.cuda.synchronize()
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    busy = torch.randn(4096, 4096, device=gpu_device)
+
+    def churn():
+        # blocks of the scratch sizes, written on the current stream while the side stream still works
+        for _ in range(4):
+            for nbytes in sizes:
+                torch.empty(nbytes, dtype=torch.uint8, device=gpu_device).fill_(0xFF)
+
+    with torch.cuda.stream(side):
+        for _ in range(20):
+            busy = busy @ busy * 1e-4          # ~tens of milliseconds queued in front of the operator
+    got = run(side, churn)
+    queued = not side.query()
+    torch.cuda.synchronize()
+    print(f"[measured] side stream still busy when the calls returned: {queued}", flush=True)
+    for x, y in zip(got, want):
+        assert torch.equal(x, y)
+    # the raw stream handle is accepted as well
+    got = run(side.cuda_stream, churn)
+    torch.cuda.synchronize()
+    for x, y in zip(got, want):
+        assert torch.equal(x, y)

@@ -212,10 +212,10 @@ def test_backward_without_saved_buffer_rebuilds_it(case, gpu_device):
                                                 (64, 66, 2, 256, "relu", "lr"), (24, 6, 3, 700, "silu", "dense"),
                                                 (20, 5, 2, 1024, "tanh", "lr"), (18, 4, 4, 1300, "gelu", "spread"),
                                                 (1, 3, 2, 256, "gelu", "dense"), (1, 2, 2, 2048, "tanh", "dense"),
-                                                (1, 1, 2, 40, "tanh", "dense")],
+                                                (1, 1, 2, 40, "tanh", "dense"), (16, 3, 64, 640, "silu", "dense")],
                          ids=["n120", "n256", "ragged_k3", "k16", "n256_odd_T", "n200_ragged_resident", "n256_relu_T66",
                               "n700_k3_step", "n1024_step", "n1300_k4_step",
-                              "one_sample_resident", "one_sample_n2048_step", "one_sample_one_step"])
+                              "one_sample_resident", "one_sample_n2048_step", "one_sample_one_step", "n640_k64_step"])
 def test_gradients_of_action_signal_and_initial_state(B, T, k, N, act, action, gpu_device):
     """dL/d action_signal and dL/d r_init, which the reference operator does not return (cpp/ring_rnn_cuda.py:144);
     pinned by the fp64 oracle, whose grad_A / grad_r_init are themselves checked by finite differences."""
@@ -295,3 +295,112 @@ def test_alpha_zero_and_zero_weights_closed_forms(gpu_device):
     decay = ring_rnn_cuda_func(A, torch.zeros_like(Wa), 0.0, 1.0, torch.zeros_like(Wo), r0, 0.15, "tanh")
     for t in range(T):
         torch.testing.assert_close(decay[t], r0 * 0.85 ** (t + 1), rtol=1e-5, atol=1e-8)
+
+
+@pytest.mark.parametrize("N", [256, 200], ids=["resident", "streaming"])
+def test_saved_buffer_that_was_copied_or_lands_on_a_stale_note(N, gpu_device):
+    """The forward leaves a transposed weight copy behind the saved activations and remembers, under the buffer's
+    address, what it packed (family, shape, J0, J1, weight tensors).  A backward must trust that copy only on an exact
+    match: a clone of the buffer (no note at its address) and a buffer whose address still carries the note of an
+    EARLIER forward with another J1 (whose packed Wo would be folded differently) both have to give the bits of the
+    backward that consumes the original buffer."""
+    from rnn_train_ring_attractor_amd.rnn_cuda import fwd_cuda, bwd_cuda, saved_nbytes
+    B, T, k = 48, 12, 2
+    print(f"[case] saved-buffer notes N={N} B={B} T={T}", flush=True)
+    p = _problem(300, B, T, k, N, "lr")
+    A, Wa, Wo, r0, G = (_dev(p[x], gpu_device) for x in ("A", "Wa", "Wo", "r0", "G"))
+    nbytes = saved_nbytes(N, k, T, B)
+
+    def forward(J1, saved):
+        hist = torch.empty(T, B, N, device=gpu_device)
+        fwd_cuda.fwd(A=A, Wa=Wa, J0=-0.05, J1=J1, Wo=Wo, r_init=r0, bump_history=hist, alpha=0.15,
+                     activation_type=ACTS["gelu"], saved=saved)
+        return hist
+
+    def backward(J1, hist, saved):
+        gWa, gWo = torch.empty_like(Wa), torch.empty_like(Wo)
+        bwd_cuda.bwd(grad_output=G, A=A, Wa=Wa, J0=-0.05, J1=J1, Wo=Wo, bump_history=hist, r_init=r0, grad_Wa=gWa,
+                     grad_Wo=gWo, alpha=0.15, activation_type=ACTS["gelu"], saved=saved, accumulate=False)
+        return gWa, gWo
+
+    stale = torch.empty(nbytes, dtype=torch.uint8, device=gpu_device)
+    forward(0.9, stale)                                  # leaves a note for J1 = 0.9 under stale's address
+    saved = torch.empty(nbytes, dtype=torch.uint8, device=gpu_device)
+    hist = forward(0.4, saved)
+    want = backward(0.4, hist, saved)
+    clone = saved.clone()                                # an address the library has never seen
+    got_clone = backward(0.4, hist, clone)
+    stale.copy_(saved)                                   # right contents, wrong note
+    got_stale = backward(0.4, hist, stale)
+    torch.cuda.synchronize()
+    for got in (got_clone, got_stale):
+        for x, y in zip(got, want):
+            assert torch.equal(x, y)
+    ref_hist, _ = O.forward_dense(p["A"], p["Wa"], -0.05, 0.4, p["Wo"], p["r0"], 0.15, "gelu")
+    ref = O.backward_dense(p["G"], p["A"], p["Wa"], -0.05, 0.4, p["Wo"], ref_hist, p["r0"], 0.15, "gelu")
+    assert O.max_rel_err(want[1].cpu().numpy(), ref["grad_Wo"]) <= GRAD_TOL
+
+
+def _self_check_recipe(seed, B, T, k, N):
+    """Inputs of the reference's own forward + backward comparison (legacy/bwd_fp32.py:486-507): weights, action
+    signal and initial state all ~ N(0, 1), UNSCALED (so gates and states are signed and the state grows by an order
+    of magnitude per step), and a random target for an MSE loss (:612-619)."""
+    rng = np.random.default_rng(seed)
+    return dict(Wa=rng.standard_normal((k, N, N)).astype(np.float32), Wo=rng.standard_normal((N, N)).astype(np.float32),
+                A=rng.standard_normal((B, T, k)).astype(np.float32), r0=rng.standard_normal((B, N)).astype(np.float32),
+                gt=rng.standard_normal((T, B, N)).astype(np.float32))
+
+
+SELF_CHECK = [
+    # name,                 B,  T,  k,    N, act      (J0 = -0.1, J1 = 0.1 as legacy/bwd_fp32.py:488-489)
+    ("reference_recipe",  256,  4, 16,  512, "silu"),   # the reference's own shape (legacy/bwd_fp32.py:587-594 region)
+    ("resident_signed",    64,  4,  2,  256, "silu"),   # signed dense gates on the weight-resident kernels
+    ("streaming_signed",   64,  5,  3,  200, "silu"),   # ... the persistent streaming kernels
+    ("step_signed",        32,  3,  3, 1024, "silu"),   # ... the step-per-launch kernels
+]
+
+
+@pytest.mark.parametrize("case", SELF_CHECK, ids=[c[0] for c in SELF_CHECK])
+def test_reference_self_check_recipe(case, gpu_device):
+    """The one forward + backward comparison the reference itself holds (legacy/bwd_fp32.py:486-507, 587-660): MSE
+    against a random target, gradients of Wa and Wo, on unscaled N(0, 1) weights, signed gates and signed states.
+    The trajectory meets the 1e-2 bound against fp64.  The weight gradients are held to cosine >= 0.998 against
+    fp64 (the CPU model of the bf16 operands alone reaches 0.99903 for grad_Wa at the reference's shape) and to the
+    rounding-aware model (same bf16 operands, fp64 sums): on this recipe the state grows ~10 x per
+    step and the Jacobian's norm is ~14, and bf16 operand rounding alone moves the largest gradient entries by
+    1e-2 .. 4e-1 of the largest (measured on the CPU model: grad_Wo 0.17, grad_Wa 0.36 at the reference's shape),
+    so the 2e-2 max-norm bound is not one a bf16-operand implementation can meet here -- the reference's own WMMA
+    path rounds the same operands (cpp/kernels/fwd_1loop_tc_idx.cuh:6-48) and its check is off by default with
+    loosened tolerances (legacy/bwd_fp32.py:641-660)."""
+    from rnn_train_ring_attractor_amd import ring_rnn_cuda_func
+    name, B, T, k, N, act = case
+    J0, J1 = -0.1, 0.1
+    print(f"[case] self-check {name} B={B} T={T} k={k} N={N} {act}", flush=True)
+    p = _self_check_recipe(7, B, T, k, N)
+    A, r0, gt = _dev(p["A"], gpu_device), _dev(p["r0"], gpu_device), _dev(p["gt"], gpu_device)
+    Wa, Wo = _dev(p["Wa"], gpu_device).requires_grad_(True), _dev(p["Wo"], gpu_device).requires_grad_(True)
+    hist = ring_rnn_cuda_func(A, Wa, J0, J1, Wo, r0, 0.15, act)
+    torch.nn.functional.mse_loss(hist, gt).backward()
+    torch.cuda.synchronize()
+    got = hist.detach().cpu().numpy().astype(np.float64)
+    ref, _ = O.forward_dense(p["A"], p["Wa"], J0, J1, p["Wo"], p["r0"], 0.15, act)
+    assert np.isfinite(got).all()
+    terr = O.max_rel_err(got, ref)
+    G_ref = (2.0 * (ref - p["gt"]) / ref.size)
+    rb = O.backward_dense(G_ref, p["A"], p["Wa"], J0, J1, p["Wo"], ref, p["r0"], 0.15, act)
+    G_hip = (2.0 * (got - p["gt"]) / got.size).astype(np.float32)
+    model = OB.forward_backward(p["A"], p["Wa"], J0, J1, p["Wo"], p["r0"], 0.15, act, G_hip, folded=_folded(N, k))
+    gWo, gWa = Wo.grad.cpu().numpy(), Wa.grad.cpu().numpy()
+    assert np.isfinite(gWo).all() and np.isfinite(gWa).all()
+    e_o, e_a = O.max_rel_err(gWo, rb["grad_Wo"]), O.max_rel_err(gWa, rb["grad_Wa"])
+    m_o, m_a = O.max_rel_err(gWo, model["grad_Wo"]), O.max_rel_err(gWa, model["grad_Wa"])
+    print(f"[measured] self-check {name}: trajectory {terr:.2e}; vs fp64 grad_Wo {e_o:.2e} grad_Wa {e_a:.2e} "
+          f"(cos {O.cosine(gWo, rb['grad_Wo']):.5f} {O.cosine(gWa, rb['grad_Wa']):.5f}); vs rounding model "
+          f"grad_Wo {m_o:.2e} grad_Wa {m_a:.2e}", flush=True)
+    assert terr <= TRAJ_TOL
+    for t in range(T):
+        assert O.max_rel_err(got[t], ref[t]) <= TRAJ_TOL
+    assert O.cosine(gWo, rb["grad_Wo"]) >= 0.998 and O.cosine(gWa, rb["grad_Wa"]) >= 0.998
+    assert O.max_rel_err(got, model["bump_history"]) <= MODEL_TOL
+    # measured against the model: 1.2e-2 / 2.1e-2 at the reference's shape (fp32 against fp64 sums, amplified as above)
+    assert m_o <= 2 * GRAD_TOL and m_a <= 2 * GRAD_TOL

@@ -35,6 +35,17 @@ def _run_pair(lib, dev, seed, B, T, k, N, act):
         torch.cuda.synchronize()
         outs.append((hist, saved))
     (h_ws, s_ws), (h_na, s_na) = outs
+    # What the entry point is for: a warmed call takes nothing from the device allocator and returns nothing to it.
+    # hipMemGetInfo (torch.cuda.mem_get_info) reports the device's free bytes; a hipMalloc inside the call, freed
+    # or not, would show while the call's work is still queued or after it.
+    torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info(dev)[0]
+    rc = lib.ringattr_fwd_noalloc(A.data_ptr(), Wa.data_ptr(), J0, J1, Wo.data_ptr(), r0.data_ptr(), h_na.data_ptr(),
+                                  alpha, N, k, T, B, act, s_na.data_ptr(), stream)
+    free_queued = torch.cuda.mem_get_info(dev)[0]
+    assert rc == 0, lib.ringattr_last_error()
+    torch.cuda.synchronize()
+    assert free_queued == free_before and torch.cuda.mem_get_info(dev)[0] == free_before
     assert torch.isfinite(h_na).all()
     assert torch.equal(h_na, h_ws)                 # bit-exact: same kernels, same packed weights
     assert torch.equal(s_na, s_ws)
