@@ -21,6 +21,8 @@
 #include "ring_common.hpp"
 #include "ring_kernels.hpp"
 
+#include <stdlib.h>
+
 namespace {
 
 constexpr int DW_WI = 2;      // MFMA row tiles per wave (32 neurons of g)
@@ -73,8 +75,11 @@ __device__ __forceinline__ bf16x8 gate_frag(bf16x8 x, const f32x4 (&g8)[2]) {
 
 }  // namespace
 
+// seg_begin / seg_end: the launch covers K chunks [seg_begin, seg_end) of the sequence (chunk = time-step pair *
+// batch tiles + batch tile, so a range of chunks is a range of time steps); add != 0: the wave adds its result
+// to the partial sums an earlier launch left.
 template <int NC, int NMAT, bool FIRST>
-__global__ __launch_bounds__(256) void ring_dw_direct_kernel(RingDwArgs p, int mg) {
+__global__ __launch_bounds__(256) void ring_dw_direct_kernel(RingDwArgs p, int mg, int seg_begin, int seg_end, int add) {
   constexpr int NT = 4 * NC;
   constexpr int NB = NT / 8;             // 128-neuron blocks per side
   constexpr int NG = NMAT - (FIRST ? 1 : 0);
@@ -99,8 +104,8 @@ __global__ __launch_bounds__(256) void ring_dw_direct_kernel(RingDwArgs p, int m
   const int it0 = (tile % NB) * 8 + wv * DW_WI;
   const int jt0 = (tile / NB) * 8;
 
-  const int nchunk = p.nbt * ((p.T + 1) / 2);   // the host checked that this fits an int
-  const int ch0 = (int)((long)nchunk * z / p.nz), ch1 = (int)((long)nchunk * (z + 1) / p.nz);
+  const int nchunk = seg_end - seg_begin;       // (the host checked that the sequence's chunk count fits an int)
+  const int ch0 = seg_begin + (int)((long)nchunk * z / p.nz), ch1 = seg_begin + (int)((long)nchunk * (z + 1) / p.nz);
 
   f32x4 acc[NMAT][DW_WI][DW_WJ];
 #pragma unroll
@@ -211,8 +216,10 @@ __global__ __launch_bounds__(256) void ring_dw_direct_kernel(RingDwArgs p, int m
 #pragma unroll
     for (int ii = 0; ii < DW_WI; ++ii)
 #pragma unroll
-      for (int u = 0; u < DW_WJ; ++u)
-        p.partial[((((size_t)z * (p.k + 1) + mm) * NT + it0 + ii) * NT + jt0 + u) * 64 + lane] = acc[a][ii][u];
+      for (int u = 0; u < DW_WJ; ++u) {
+        ring_f32x4* dst = p.partial + ((((size_t)z * (p.k + 1) + mm) * NT + it0 + ii) * NT + jt0 + u) * 64 + lane;
+        *dst = add ? *dst + acc[a][ii][u] : acc[a][ii][u];
+      }
   }
 }
 
@@ -233,36 +240,65 @@ int ring_dw_tiled_nz(int NC, int k, long nchunk) {
 }
 
 template <int NC>
-static hipError_t launch_group(const RingDwArgs& a, int mg, unsigned blocks, hipStream_t st) {
+static hipError_t launch_group(const RingDwArgs& a, int mg, unsigned blocks, int seg_begin, int seg_end, int add,
+                               hipStream_t st) {
   const int nmat = (a.k + 1 - 3 * mg) < 3 ? (a.k + 1 - 3 * mg) : 3;
   if (mg == 0) {
-    if (nmat == 3) RING_LAUNCH((ring_dw_direct_kernel<NC, 3, true>), dim3(blocks), dim3(256), 0, st, a, mg);
-    else if (nmat == 2) RING_LAUNCH((ring_dw_direct_kernel<NC, 2, true>), dim3(blocks), dim3(256), 0, st, a, mg);
-    else RING_LAUNCH((ring_dw_direct_kernel<NC, 1, true>), dim3(blocks), dim3(256), 0, st, a, mg);
+    if (nmat == 3) RING_LAUNCH((ring_dw_direct_kernel<NC, 3, true>), dim3(blocks), dim3(256), 0, st, a, mg, seg_begin, seg_end, add);
+    else if (nmat == 2) RING_LAUNCH((ring_dw_direct_kernel<NC, 2, true>), dim3(blocks), dim3(256), 0, st, a, mg, seg_begin, seg_end, add);
+    else RING_LAUNCH((ring_dw_direct_kernel<NC, 1, true>), dim3(blocks), dim3(256), 0, st, a, mg, seg_begin, seg_end, add);
   } else {
-    if (nmat == 3) RING_LAUNCH((ring_dw_direct_kernel<NC, 3, false>), dim3(blocks), dim3(256), 0, st, a, mg);
-    else if (nmat == 2) RING_LAUNCH((ring_dw_direct_kernel<NC, 2, false>), dim3(blocks), dim3(256), 0, st, a, mg);
-    else RING_LAUNCH((ring_dw_direct_kernel<NC, 1, false>), dim3(blocks), dim3(256), 0, st, a, mg);
+    if (nmat == 3) RING_LAUNCH((ring_dw_direct_kernel<NC, 3, false>), dim3(blocks), dim3(256), 0, st, a, mg, seg_begin, seg_end, add);
+    else if (nmat == 2) RING_LAUNCH((ring_dw_direct_kernel<NC, 2, false>), dim3(blocks), dim3(256), 0, st, a, mg, seg_begin, seg_end, add);
+    else RING_LAUNCH((ring_dw_direct_kernel<NC, 1, false>), dim3(blocks), dim3(256), 0, st, a, mg, seg_begin, seg_end, add);
   }
   return hipGetLastError();
 }
 
-// One launch per group of three matrices (a_dim = 2 needs exactly one).
+// K chunks a workgroup walks per launch, at most.  The workgroups of a K split read the same two operand streams
+// and find each other's fragments in their XCD's L2 only while they stay within about 32 chunks of one another
+// (4 MiB of L2 against 128 KiB of new operand bytes per chunk step and XCD).  Nothing synchronises them, so over a
+// long walk they drift apart and every one fetches its operands from memory for itself: at N = 512, B = 8192 the
+// kernel reads 1.02 x its operands over 512 chunks per workgroup, 1.45 x over 2048 and 2.47 x over 8192.  A long
+// sequence is therefore cut into segments in time, one launch each (a launch boundary re-aligns the workgroups);
+// the launches after the first add to the partial sums.  RINGATTR_DW_SEGMENT overrides the length (0: no cut).
+static int dw_segment_chunks() {
+  static const int v = [] {
+    const char* e = getenv("RINGATTR_DW_SEGMENT");
+    return e ? atoi(e) : 640;
+  }();
+  return v;
+}
+
+// One launch per group of three matrices (a_dim = 2 needs exactly one) and segment.
 hipError_t ring_launch_dw_tiled(const RingDwArgs& a, int NC, hipStream_t st) {
   const int NB = 4 * NC / 8;
   const unsigned blocks = (unsigned)(NB * NB * a.nz);
   const int nmg = (a.k + 3) / 3;
+  const int npairs = (a.T + 1) / 2;
+  const long nchunk = (long)a.nbt * npairs;
+  const int seg = dw_segment_chunks();
+  // whole time-step pairs per segment, so that a segment is a contiguous range of chunks
+  long pairs_per_seg = npairs;
+  if (seg > 0 && nchunk / a.nz > seg) {
+    pairs_per_seg = ((long)seg * a.nz) / a.nbt;
+    if (pairs_per_seg < 1) pairs_per_seg = 1;
+  }
   for (int mg = 0; mg < nmg; ++mg) {
-    hipError_t e = hipErrorInvalidValue;
-    switch (NC) {
-      case 4: e = launch_group<4>(a, mg, blocks, st); break;
-      case 8: e = launch_group<8>(a, mg, blocks, st); break;
-      case 16: e = launch_group<16>(a, mg, blocks, st); break;
-      case 24: e = launch_group<24>(a, mg, blocks, st); break;
-      case 32: e = launch_group<32>(a, mg, blocks, st); break;
-      default: break;
+    for (long p0 = 0; p0 < npairs; p0 += pairs_per_seg) {
+      const long p1 = p0 + pairs_per_seg < npairs ? p0 + pairs_per_seg : npairs;
+      const int b = (int)(p0 * a.nbt), e_ = (int)(p1 * a.nbt), add = p0 > 0 ? 1 : 0;
+      hipError_t e = hipErrorInvalidValue;
+      switch (NC) {
+        case 4: e = launch_group<4>(a, mg, blocks, b, e_, add, st); break;
+        case 8: e = launch_group<8>(a, mg, blocks, b, e_, add, st); break;
+        case 16: e = launch_group<16>(a, mg, blocks, b, e_, add, st); break;
+        case 24: e = launch_group<24>(a, mg, blocks, b, e_, add, st); break;
+        case 32: e = launch_group<32>(a, mg, blocks, b, e_, add, st); break;
+        default: break;
+      }
+      if (e != hipSuccess) return e;
     }
-    if (e != hipSuccess) return e;
   }
   return hipSuccess;
 }
