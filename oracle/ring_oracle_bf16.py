@@ -46,30 +46,48 @@ def round_u8_dact(x):
     return code / scale + DACT_LO
 
 
+ROUNDING_POINTS = ("r", "w", "g", "dact", "ag")
+
+
 def forward_backward(A, Wa, J0, J1, Wo, r_init, alpha, activation_name, grad_output=None, rounding=True,
-                     folded=False, dact="fp16"):
+                     folded=False, dact="fp16", only=None):
     """Returns dict(bump_history [T,B,N], and, when grad_output is given, grad_Wa, grad_Wo, grad_r_init, grad_A).
     folded: model of the weight-resident kernels, whose bf16 Wo operand is round(J1 * Wo + J0) (formed in fp32), so
     that J0 * sum_j x_j + J1 * (x Wo^T) is one product over the bf16 operand copy of x; otherwise (the streaming
     kernels) Wo is rounded alone, J1 is applied in fp32 and the J0 row sums run over the fp32 values.
-    dact: storage format of F', "fp16" or "u8"."""
-    rb16 = round_bf16 if rounding else _identity
-    rf16 = (round_u8_dact if dact == "u8" else round_fp16) if rounding else _identity
+    dact: storage format of F', "fp16" or "u8".
+    only: None rounds at every point; otherwise the subset of ROUNDING_POINTS to round at, everything else exact --
+    "r" the forward's state operand, "w" the weight operands (Wa and Wo, or the folded J1 * Wo + J0), "g" the
+    backward's operand, "dact" the stored derivative, "ag" the gated operand of the weight-gradient contraction.
+    Used to attribute a deviation from fp64 to the operand that causes it."""
+    if only is not None:
+        unknown = set(only) - set(ROUNDING_POINTS)
+        if unknown:
+            raise ValueError(f"unknown rounding points {sorted(unknown)}; choose from {ROUNDING_POINTS}")
+    on = (lambda name: rounding and (only is None or name in only))
+    rb16_r = round_bf16 if on("r") else _identity
+    rb16_w = round_bf16 if on("w") else _identity
+    rb16_g = round_bf16 if on("g") else _identity
+    rb16_ag = round_bf16 if on("ag") else _identity
+    rf16 = (round_u8_dact if dact == "u8" else round_fp16) if on("dact") else _identity
     A = np.asarray(A, np.float64)
     Wa = np.asarray(Wa, np.float64)
     Wo = np.asarray(Wo, np.float64)
     r = np.array(r_init, np.float64)
     B, T, k = A.shape
     N = Wo.shape[0]
-    Wob, Wab = rb16(Wo), rb16(Wa)
+    Wob, Wab = rb16_w(Wo), rb16_w(Wa)
     if folded:   # fp32 fused multiply-add, then one rounding to bf16
-        Wof = rb16((Wo * float(np.float32(J1)) + float(np.float32(J0))).astype(np.float32))
+        if on("w"):
+            Wof = round_bf16((Wo * float(np.float32(J1)) + float(np.float32(J0))).astype(np.float32))
+        else:
+            Wof = Wo * J1 + J0
     hist = np.empty((T, B, N))
     D = np.empty((T, B, N))
     R = np.empty((T, B, N))
     Rfull = np.empty((T, B, N))
     for t in range(T):
-        rb = rb16(r)
+        rb = rb16_r(r)
         R[t] = rb
         Rfull[t] = r
         re = rb @ Wof.T if folded else J0 * r.sum(axis=1, keepdims=True) + J1 * (rb @ Wob.T)
@@ -89,7 +107,7 @@ def forward_backward(A, Wa, J0, J1, Wo, r_init, alpha, activation_name, grad_out
     for t in range(T - 1, -1, -1):
         G = G_out[t] + carry
         g = D[t] * G
-        gb = rb16(g)
+        gb = rb16_g(g)
         if folded:
             carry = (1.0 - alpha) * G + gb @ Wof
         else:
@@ -101,6 +119,6 @@ def forward_backward(A, Wa, J0, J1, Wo, r_init, alpha, activation_name, grad_out
             grad_A[:, t, c] = (pc * (R[t] if folded else Rfull[t])).sum(axis=1)
         grad_Wo += J1 * (gb.T @ R[t])
         for c in range(k):
-            grad_Wa[c] += rb16(A[:, t, c:c + 1] * gb).T @ R[t]
+            grad_Wa[c] += rb16_ag(A[:, t, c:c + 1] * gb).T @ R[t]
     out.update(grad_Wo=grad_Wo, grad_Wa=grad_Wa, grad_r_init=carry, grad_A=grad_A)
     return out

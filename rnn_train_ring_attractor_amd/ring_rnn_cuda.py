@@ -19,7 +19,8 @@ def _activation_id(name):
     return _ACTIVATION_MAP[name]
 
 
-def ring_rnn_cuda_func(action_signal, Wa, J0, J1, Wo, r_init, alpha, activation='relu', driven_channels=None):
+def ring_rnn_cuda_func(action_signal, Wa, J0, J1, Wo, r_init, alpha, activation='relu', driven_channels=None,
+                       precise_wo=None):
     """Ring RNN forward pass on the GPU.
 
     action_signal (B,T,k); Wa (k,N,N); J0, J1 scalars; Wo (N,N); r_init (B,N); alpha float;
@@ -28,10 +29,16 @@ def ring_rnn_cuda_func(action_signal, Wa, J0, J1, Wo, r_init, alpha, activation=
     driven_channels (optional, not in the reference): the caller's statement that every action channel outside this
     list of at most two indices is identically zero (the training script's zero padding of (L, R) to a_dim = 16);
     see `_silent_channel_view`.  Tensors made by `host.av_to_action_signal_ND(zero_padding=True)` carry it themselves.
+
+    precise_wo (optional, not in the reference; None takes the module's PRECISE_WO): Wo enters the contraction as
+    two bf16 operands, its bf16 rounding and the rounding of what that leaves; see `_split_wo`.
     """
-    compact = _silent_channel_view(action_signal, Wa, driven_channels)
-    if compact is not None:
-        action_signal, Wa = compact
+    if PRECISE_WO if precise_wo is None else precise_wo:
+        action_signal, Wa = _split_wo(action_signal, Wa, J1, Wo)
+    else:
+        compact = _silent_channel_view(action_signal, Wa, driven_channels)
+        if compact is not None:
+            action_signal, Wa = compact
     # Autograd switches gradient mode off inside Function.forward, and needs_input_grad stays True under
     # torch.no_grad(): the wrapper is the place that knows whether a backward can follow.
     return RingRnnCudaFunc.apply(action_signal, Wa, J0, J1, Wo, r_init, alpha, activation, torch.is_grad_enabled())
@@ -43,6 +50,31 @@ def ring_rnn_cuda_func(action_signal, Wa, J0, J1, Wo, r_init, alpha, activation=
 # both from it before the reverse-time loop (the reference recomputes re in every backward,
 # cpp/kernels/bwd_mixed_precision_aggressive.cuh:53-269): no saved buffer is held between forward and backward.
 RECOMPUTE_IN_BACKWARD = False
+
+# Default of ring_rnn_cuda_func's precise_wo.
+PRECISE_WO = False
+
+
+def _split_wo(action_signal, Wa, J1, Wo):
+    """Wo as two bf16 MFMA operands.  The kernels round every weight to bf16 once, which makes the network they
+    simulate a fixed perturbation (2^-9 relative per weight) of the caller's.  Where the dynamics are marginally
+    stable -- the integrator regime the ring attractor is trained for, J1 = 1 with weights ~ N(0, 1/N) -- the two
+    networks' states drift apart linearly in time: at N = 512, J0 = -1/N, J1 = 1, tanh the per-step deviation from
+    fp64 reaches 1e-2 at t = 166 and 1.2e-1 at t = 511, all of it from the rounding of Wo (Wa is gated by |av| <=
+    0.31 and the state operand's rounding does not accumulate; the reference's own tensor-core path keeps Wo in fp32
+    and rounds Wa and the action signal, cpp/kernels/fwd_1loop_tc_idx.cuh:6-48).  With Wo = hi + lo, hi = bf16(Wo)
+    and lo = bf16(Wo - hi), the deviation stays under 4e-3 over the 512 steps.
+    lo rides as one more action matrix whose gate is the constant J1, so the kernels need no change: one more
+    matrix in the step's weight stream (a third more work at two action channels; with N <= 256 the call moves
+    from the weight-resident kernels to the streaming ones, whose matrix count is free).  The extra channel's weight
+    gradient repeats grad_Wo and is dropped; gradients of Wa, Wo and, if asked for, action_signal are unchanged in
+    meaning."""
+    B, T, k = action_signal.shape
+    lo = (Wo - Wo.to(torch.bfloat16).to(Wo.dtype)).detach()
+    Wa_ext = torch.cat([Wa, lo.unsqueeze(0)], dim=0)
+    gate = torch.full((B, T, 1), float(J1), dtype=action_signal.dtype, device=action_signal.device)
+    return torch.cat([action_signal, gate], dim=2), Wa_ext
+
 
 DRIVEN_ATTR = "_ring_driven_channels"     # set on zero-padded action signals by the host helper that builds them
 

@@ -180,8 +180,9 @@ def test_long_sequence_shape_at_full_size(gpu_device):
     from rnn_train_ring_attractor_amd import ring_rnn_cuda_func
     print("[case] long sequence N=512 B=8192 T=512 tanh (full size)", flush=True)
     B, T, k, N = 8192, 512, 2, 512
-    # contractive gain: with J1 = 1 random weights sit at the edge of chaos and 512 steps amplify any rounding
-    # difference, in every implementation
+    # J1 = 0.5 here: at the configuration's own J1 = 1 the dynamics are marginally stable and the bf16 rounding of Wo
+    # (a fixed perturbation of the network) accumulates past 1e-2 after ~166 steps -- shown on the CPU in
+    # tests/test_oracle_forward.py and held to what can be demanded in test_long_sequence_at_its_own_gain below
     J0, J1 = -1.0 / N, 0.5
     gen = torch.Generator(device=gpu_device).manual_seed(3)
     Wa0 = torch.randn(k, N, N, device=gpu_device, generator=gen) / N ** 0.5
@@ -223,6 +224,59 @@ def test_long_sequence_shape_at_full_size(gpu_device):
     assert O.max_rel_err(c(doubled[2]), 2.0 * c(full[2])) <= 1e-5 and O.max_rel_err(c(doubled[1]), 2.0 * c(full[1])) <= 1e-5
     lo, hi = run(slice(0, B // 2)), run(slice(B // 2, B))
     assert O.max_rel_err(c(lo[1] + hi[1]), c(full[1])) <= 1e-4 and O.max_rel_err(c(lo[2] + hi[2]), c(full[2])) <= 1e-4
+
+
+def test_long_sequence_at_its_own_gain(gpu_device):
+    """BASELINE's long-sequence configuration at its own parameters (N = 512, T = 512, tanh, J0 = -1/N, J1 = 1; a
+    32-row batch so that the fp64 oracle finishes in seconds).  bf16 operands: the kernels follow the rounding-aware
+    model over all 512 steps and the fp64 oracle over the first 150 (beyond, the rounding of Wo accumulates past
+    1e-2 in these marginally stable dynamics, in the model exactly as in the kernels).  precise_wo=True (Wo as two
+    bf16 operands): trajectory within 1e-2 of fp64 over all 512 steps, weight gradients within the gradient
+    tolerances."""
+    from rnn_train_ring_attractor_amd import ring_rnn_cuda_func
+    print("[case] long sequence at J1 = 1: N=512 B=32 T=512 tanh", flush=True)
+    B, T, k, N = 32, 512, 2, 512
+    J0, J1 = -1.0 / N, 1.0
+    p = make_problem(3, B, T, k, N, zero_ratios=(0.2,), bump="vm")
+    p["G"] = p["G"] / (T * B)
+    ref, _ = O.forward_dense(p["A"], p["Wa"], J0, J1, p["Wo"], p["r0"], 0.15, "tanh")
+    g = O.backward_dense(p["G"], p["A"], p["Wa"], J0, J1, p["Wo"], ref, p["r0"], 0.15, "tanh")
+    model = OB.forward_backward(p["A"], p["Wa"], J0, J1, p["Wo"], p["r0"], 0.15, "tanh", p["G"], folded=False)
+    c = lambda x: x.detach().cpu().numpy().astype(np.float64)
+
+    def run(precise):
+        Wa, Wo = _t(p["Wa"], gpu_device).requires_grad_(True), _t(p["Wo"], gpu_device).requires_grad_(True)
+        h = ring_rnn_cuda_func(_t(p["A"], gpu_device), Wa, J0, J1, Wo, _t(p["r0"], gpu_device), 0.15, "tanh",
+                               precise_wo=precise)
+        h.backward(_t(p["G"], gpu_device))
+        torch.cuda.synchronize()
+        return c(h), c(Wa.grad), c(Wo.grad)
+
+    def per_step(x, y):
+        return np.array([O.max_rel_err(x[t], y[t]) for t in range(T)])
+
+    h, gWa, gWo = run(False)
+    e = per_step(h, ref)
+    em = per_step(h, model["bump_history"])
+    print(f"[measured] bf16 Wo: vs fp64 per-step max over t < 150 {e[:150].max():.2e}, at t = 511 {e[-1]:.2e}; vs rounding "
+          f"model max over all steps {em.max():.2e}; grad_Wo vs fp64 {O.max_rel_err(gWo, g['grad_Wo']):.2e} (cos "
+          f"{O.cosine(gWo, g['grad_Wo']):.5f}), vs model {O.max_rel_err(gWo, model['grad_Wo']):.2e}", flush=True)
+    assert e[:150].max() <= TRAJ_TOL
+    assert em.max() <= 2e-2                       # 512 steps of fp32 against fp64 sums on top of the same operands
+    assert O.cosine(gWo, g["grad_Wo"]) >= GRAD_COS and O.cosine(gWa, g["grad_Wa"]) >= GRAD_COS
+    assert O.max_rel_err(gWo, model["grad_Wo"]) <= GRAD_TOL and O.max_rel_err(gWa, model["grad_Wa"]) <= GRAD_TOL
+    h, gWa, gWo = run(True)
+    e = per_step(h, ref)
+    whole = O.max_rel_err(h, ref)
+    print(f"[measured] Wo as hi + lo: vs fp64 whole trajectory {whole:.2e}, per-step max over all 512 steps {e.max():.2e}; grad_Wo {O.max_rel_err(gWo, g['grad_Wo']):.2e} "
+          f"(cos {O.cosine(gWo, g['grad_Wo']):.5f}), grad_Wa {O.max_rel_err(gWa, g['grad_Wa']):.2e} (cos {O.cosine(gWa, g['grad_Wa']):.5f})",
+          flush=True)
+    # in the max norm of the whole trajectory, as every other parity case; relative to each step's own largest state
+    # (which decays from 0.12 to 0.03 along the sequence) the bound is twice as wide (measured 1.1e-2 at B = 32)
+    assert whole <= TRAJ_TOL and e.max() <= 2 * TRAJ_TOL
+    assert gWa.shape == p["Wa"].shape
+    assert O.cosine(gWo, g["grad_Wo"]) >= GRAD_COS and O.max_rel_err(gWo, g["grad_Wo"]) <= GRAD_TOL
+    assert O.cosine(gWa, g["grad_Wa"]) >= GRAD_COS and O.max_rel_err(gWa, g["grad_Wa"]) <= GRAD_TOL
 
 
 def test_streaming_and_resident_kernels_agree(gpu_device, monkeypatch):
@@ -699,8 +753,11 @@ def test_relu_gradients_against_fp64_at_a_realistic_batch(weights, gpu_device, d
     single entries differ from fp64 by 3-6 % even at this batch, with bump-sustaining weights (a few neurons carry
     the gradient) by 7-9 %; the cosine holds everywhere (>= 0.9991 measured).  The CPU model that rounds the same
     operands differs from fp64 by the same amounts and agrees with the kernels to 1e-2 and better, so the deviation
-    is the operand format's, not a kernel's.  The entry-wise 2e-2 bound is therefore asserted against that model;
-    against fp64 the test asserts what was measured on the MI355X (with head room) so that a regression shows."""
+    is the operand format's, not a kernel's: the CPU model attributes all of it to the two forward operands (state
+    and weights, either of which alone exceeds 2e-2; tests/test_oracle_bf16.py), and the weights cannot be carried
+    at higher precision in a compute unit that keeps them resident.  The entry-wise 2e-2 bound is therefore asserted
+    against that model; against fp64 the test asserts what was measured on the MI355X plus 20 % (random weights
+    3.4e-2 / 5.6e-2, bump-sustaining weights 7.5e-2 / 9.1e-2 for grad_Wo / grad_Wa) so that a regression shows."""
     from rnn_train_ring_attractor_amd import ring_rnn_cuda_func
     print(f"[case] relu gradients vs fp64 at N=256 B=1024 T=120, {weights} weights", flush=True)
     B, T, k, N = 1024, 120, 2, 256
@@ -727,7 +784,8 @@ def test_relu_gradients_against_fp64_at_a_realistic_batch(weights, gpu_device, d
     assert O.max_rel_err(h.detach().cpu().numpy(), ref) <= TRAJ_TOL
     assert c_wo >= GRAD_COS and c_wa >= GRAD_COS
     assert m_wo <= GRAD_TOL and m_wa <= GRAD_TOL
-    assert e_wo <= 0.12 and e_wa <= 0.12
+    bound_wo, bound_wa = {"random": (0.041, 0.067), "perfect": (0.090, 0.109)}[weights]
+    assert e_wo <= bound_wo and e_wa <= bound_wa
 
 
 def test_training_driver_reduces_loss(gpu_device):

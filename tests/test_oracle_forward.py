@@ -169,3 +169,51 @@ def test_torch_port_forward_equals_numpy_oracle(name):
     t = lambda x: torch.tensor(x, dtype=torch.float64)
     hist_t = TP.ring_forward(t(A), t(Wa), -0.1, 0.1, t(Wo), t(r0), 0.15, name)
     np.testing.assert_allclose(hist, hist_t.numpy(), rtol=0, atol=1e-13)
+
+
+def test_long_sequence_at_its_own_gain_where_bf16_weights_leave_the_tolerance():
+    """BASELINE's long-sequence configuration at its own parameters (N = 512, T = 512, tanh, J0 = -1/N, J1 = 1,
+    weights ~ N(0, 1/N); a small batch here).  What the parity tests may and may not demand there:
+      * the dynamics are NOT chaotic: a 1e-9 perturbation of the initial state is still ~1e-9 after 512 steps, and
+        the fp32 torch port of the reference formulation (train/train_ring_attractor.py:158-177) agrees with fp64
+        to 1e-4 at every step -- an implementation that computes in fp32 has no excuse here;
+      * they are marginally stable, so a FIXED perturbation of the network accumulates: with the MFMA operands
+        rounded to bf16 the per-step deviation from fp64 (relative to the step's largest state) passes 1e-2 at
+        t ~ 166 and reaches ~1e-1 at t = 511; the GPU parity test of this configuration therefore holds the
+        kernels to fp64 over the first 150 steps and to the rounding-aware model over all 512;
+      * all of it comes from rounding Wo: rounding only Wa, or only the state operand, stays under 6e-3 to the end,
+        and Wo carried as two bf16 operands (hi + lo, the operator's precise_wo option) under 5e-3."""
+    import torch
+    from oracle import ring_oracle_bf16 as OB
+    from oracle import torch_port as TP
+    from tests.ring_cases import make_problem
+    N, B, T, k = 512, 8, 512, 2
+    J0, J1 = -1.0 / N, 1.0
+    p = make_problem(3, B, T, k, N, bump="vm")
+    args = (p["A"], p["Wa"], J0, J1, p["Wo"], p["r0"], 0.15, "tanh")
+    ref, _ = O.forward_dense(*args)
+
+    def per_step(x):
+        return np.array([O.max_rel_err(x[t], ref[t]) for t in range(T)])
+
+    bumped = p["r0"].astype(np.float64) * (1.0 + 1e-9 * np.sign(np.random.default_rng(0).standard_normal(p["r0"].shape)))
+    e_pert = per_step(O.forward_dense(p["A"], p["Wa"], J0, J1, p["Wo"], bumped, 0.15, "tanh")[0])
+    assert e_pert.max() <= 1e-8
+    t_ = lambda x: torch.tensor(x)
+    with torch.no_grad():
+        f32 = TP.ring_forward(t_(p["A"]), t_(p["Wa"]), J0, J1, t_(p["Wo"]), t_(p["r0"]), 0.15, "tanh").numpy()
+    assert per_step(f32.astype(np.float64)).max() <= 1e-4
+    e_bf16 = per_step(OB.forward_backward(*args)["bump_history"])
+    horizon = int(np.nonzero(e_bf16 > 1e-2)[0][0])
+    print(f"[measured] N=512 T=512 J1=1 tanh: bf16-operand model leaves 1e-2 at t = {horizon}, "
+          f"error at t = 511 {e_bf16[-1]:.2e}; fp32 port max {per_step(f32.astype(np.float64)).max():.1e}")
+    assert 150 <= horizon <= 250 and e_bf16[:150].max() <= 1e-2 and e_bf16[-1] > 5e-2
+    Wo_hi = OB.round_bf16(p["Wo"])
+    e_wo = per_step(O.forward_dense(p["A"], p["Wa"], J0, J1, Wo_hi, p["r0"], 0.15, "tanh")[0])
+    e_wa = per_step(O.forward_dense(p["A"], OB.round_bf16(p["Wa"]), J0, J1, p["Wo"], p["r0"], 0.15, "tanh")[0])
+    e_r = per_step(OB.forward_backward(*args, only=("r",))["bump_history"])
+    assert e_wo[-1] > 0.8 * e_bf16[-1] and e_wa.max() <= 6e-3 and e_r.max() <= 6e-3
+    # Wo = hi + lo as two bf16 operands, Wa and the state operand rounded as always
+    Wo_lo = OB.round_bf16(p["Wo"].astype(np.float64) - Wo_hi)
+    split = OB.forward_backward(p["A"], OB.round_bf16(p["Wa"]), J0, J1, Wo_hi + Wo_lo, p["r0"], 0.15, "tanh", only=("r",))
+    assert per_step(split["bump_history"]).max() <= 5e-3
