@@ -266,6 +266,7 @@ def main():
     dt = time.perf_counter() - t0
     prof = _lib.profile_read()
     _lib.profile_enable(False)
+    launched = _lib.last_kernel_names()      # the kernels of the timed region (the training-step leg below launches others)
     training_step = None
     if mode == "train" and k == 2 and N <= 512 and not args.no_training_step:
         # Beside the metric (not part of it): a whole training step around the same time loop -- a fresh batch from the
@@ -310,7 +311,7 @@ def main():
     achieved = flops_third / (dom_ms * 1e-3) / 1e12
     bytes_per_ss = 12 * N + 8 * k                           # fp32 history write + r_prev/grad_output reads + A
     traffic, traffic_notes = measured_traffic(args.workload + ("_recompute" if args.recompute else ""),
-                                              _lib.last_kernel_names())
+                                              launched)
     out = {
         "metric": ("fwd+bwd sample-steps/s (B*T/s) at N=256,B=4096,T=120; % bf16 MFMA peak"
                    if args.workload == HEADLINE else
