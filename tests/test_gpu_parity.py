@@ -404,3 +404,47 @@ def test_reference_self_check_recipe(case, gpu_device):
     assert O.max_rel_err(got, model["bump_history"]) <= MODEL_TOL
     # measured against the model: 1.2e-2 / 2.1e-2 at the reference's shape (fp32 against fp64 sums, amplified as above)
     assert m_o <= 2 * GRAD_TOL and m_a <= 2 * GRAD_TOL
+
+
+@pytest.mark.parametrize("B,T,k,N,act", [(48, 14, 2, 256, "gelu"), (40, 9, 2, 200, "tanh"), (24, 5, 3, 640, "silu")],
+                         ids=["resident", "streaming", "step"])
+def test_operator_switches_recompute_and_precise_wo(B, T, k, N, act, gpu_device):
+    """The two module-level switches of the Python operator.  RECOMPUTE_IN_BACKWARD: the forward keeps no saved
+    record and the backward rebuilds it (gradients agree with the stored-record path to summation-order noise,
+    bitwise where the rebuild re-runs the same kernel).  precise_wo: Wo as two bf16 operands through one more action
+    matrix with the constant gate J1 -- same output and gradient shapes, gradients of Wa, Wo, the action signal and
+    the initial state against the fp64 oracle, and a trajectory at least as close to fp64 as the bf16-Wo one."""
+    from rnn_train_ring_attractor_amd import ring_rnn_cuda as op
+    print(f"[case] operator switches B={B} T={T} k={k} N={N} {act}", flush=True)
+    J0, J1 = -0.05, 0.6
+    p = _problem(400, B, T, k, N, "dense")
+    ref_hist, _ = O.forward_dense(p["A"], p["Wa"], J0, J1, p["Wo"], p["r0"], 0.15, act)
+    ref = O.backward_dense(p["G"], p["A"], p["Wa"], J0, J1, p["Wo"], ref_hist, p["r0"], 0.15, act)
+
+    def run(**kw):
+        A = _dev(p["A"], gpu_device).requires_grad_(True)
+        r0 = _dev(p["r0"], gpu_device).requires_grad_(True)
+        Wa, Wo = _dev(p["Wa"], gpu_device).requires_grad_(True), _dev(p["Wo"], gpu_device).requires_grad_(True)
+        h = op.ring_rnn_cuda_func(A, Wa, J0, J1, Wo, r0, 0.15, act, **kw)
+        h.backward(_dev(p["G"], gpu_device))
+        torch.cuda.synchronize()
+        return [x.detach().cpu().numpy() for x in (h, Wa.grad, Wo.grad, A.grad, r0.grad)]
+
+    base = run()
+    assert op.RECOMPUTE_IN_BACKWARD is False and op.PRECISE_WO is False
+    op.RECOMPUTE_IN_BACKWARD = True
+    try:
+        rec = run()
+    finally:
+        op.RECOMPUTE_IN_BACKWARD = False
+    assert np.array_equal(rec[0], base[0])
+    for x, y in zip(rec[1:], base[1:]):
+        assert O.max_rel_err(x, y) <= 1e-3
+    pre = run(precise_wo=True)
+    assert [x.shape for x in pre] == [x.shape for x in base]
+    e_pre, e_base = O.max_rel_err(pre[0], ref_hist), O.max_rel_err(base[0], ref_hist)
+    print(f"[measured] trajectory vs fp64: bf16 Wo {e_base:.2e}, Wo as hi + lo {e_pre:.2e}", flush=True)
+    assert e_pre <= TRAJ_TOL and e_pre <= 1.2 * e_base + 1e-4
+    for got, key in zip(pre[1:], ("grad_Wa", "grad_Wo", "grad_A", "grad_r_init")):
+        assert O.cosine(got, ref[key]) >= GRAD_COS, key
+        assert O.max_rel_err(got, ref[key]) <= GRAD_TOL, key

@@ -1,5 +1,6 @@
 """The torch host helpers (same module paths the reference script imports) against the numpy oracle."""
 import math
+import os
 
 import numpy as np
 import pytest
@@ -119,3 +120,21 @@ def test_chunked_generator_concatenates_trials():
     assert float(av.abs().max()) <= 0.1 * 3.141593
     step = torch.remainder(ang[:, 1:] - ang[:, :-1] - av[:, :-1] + 3.141592653589793, 2 * 3.141592653589793) - 3.141592653589793
     assert float(step.abs().max()) <= 1e-4
+
+
+def test_bench_drops_counter_summaries_of_other_kernels():
+    """bench.py pairs its timings with the HBM traffic of a stored rocprofv3 counter summary; the summary names the
+    kernels it was taken from, and a slot whose kernel differs from the one the run launched is dropped with a note."""
+    import re
+    import bench
+    path = os.path.join(os.path.dirname(bench.__file__), "profiles", f"{bench.HEADLINE}_counters.md")
+    text = open(path).read()
+    named = dict(kv.split("=", 1) for kv in re.search(r"^TRAFFIC_KERNELS\s+(.*)$", text, re.M).group(1).split(";"))
+    assert {"fwd", "bptt", "dw"} <= set(named)
+    traffic, notes = bench.measured_traffic(bench.HEADLINE, dict(named))
+    assert notes == [] and traffic["fwd"] > 5e8 and traffic["bptt"] > 5e8 and traffic["dw"] > 2e8
+    other = dict(named, fwd="ring_fwd_res256_kernel<1,true,true,true>")
+    traffic, notes = bench.measured_traffic(bench.HEADLINE, other)
+    assert "fwd" not in traffic and "bptt" in traffic and len(notes) == 1 and "fwd" in notes[0]
+    traffic, notes = bench.measured_traffic("no_such_workload", named)
+    assert traffic is None and notes
