@@ -148,7 +148,8 @@ struct StreamCfg {
   using TL = Tile<NC>;
   static constexpr int KG = (RT > 1 && TL::KG == 8) ? 4 : TL::KG, NKG = TL::KCH / KG;
   static constexpr int UPM = NKG * NC;                 // units per matrix
-  static constexpr int PDMAX = (RT > 1 && TL::KG == 8) ? 8 : 4;
+  // (four tiles: every fetched fragment feeds four MFMAs, so half as many units in flight cover the same time)
+  static constexpr int PDMAX = (RT >= 4) ? 4 : ((RT > 1 && TL::KG == 8) ? 8 : 4);
   static constexpr int PD = UPM >= PDMAX ? PDMAX : UPM;
   static_assert(UPM % PD == 0, "static register-buffer indices need whole rounds per matrix");
 };
@@ -571,6 +572,68 @@ __global__ __launch_bounds__(256) void ring_rebuild_saved_kernel(RingFwdArgs p) 
       }
     }
     side_store<NC, f16x4, _Float16>(p.dfrag + side_offset<NC>(t, p.nbt, bt0 + rt, w, lane), d);
+  }
+}
+
+// The same rebuild with four row tiles per workgroup: two batch tiles x two consecutive time steps.  Nothing here
+// depends on an earlier step (every step's r_prev is a row of the history), so rows of different steps can share a
+// fetched weight fragment just as rows of different samples do: each fragment feeds four MFMAs and the workgroups
+// together stream the weights from L2 half as often as with two tiles.  Tile rt is (batch tile bt0 + rt % 2, step
+// 2 * blockIdx.y + rt / 2); the operand tiles live in dynamic shared memory (4 * SLOTS fragments).
+template <int NC, int ACT>
+__global__ __launch_bounds__(256) void ring_rebuild_saved4_kernel(RingFwdArgs p) {
+  using TL = Tile<NC>;
+  constexpr int RT = 4;
+  extern __shared__ __attribute__((aligned(16))) char rebuild_lds[];
+  bf16x8* const xbuf = reinterpret_cast<bf16x8*>(rebuild_lds);
+  __shared__ float psum[RT][64];
+  __shared__ float gl[RT * 16 * GATE_KMAX];
+
+  const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, q = lane >> 4, n = lane & 15;
+  const int bt0 = blockIdx.x * 2, t0 = blockIdx.y * 2;
+  const int i0 = 16 * NC * w + NC * n;
+  const int N = p.N, B = p.B, T = p.T;
+
+  bool live[RT];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    const int bt = bt0 + (rt & 1), t = t0 + (rt >> 1);
+    live[rt] = bt < p.nbt && t < T;
+    const int tc = t < T ? t : T - 1;                      // a step past the end re-reads the last one, unused
+    const float* prev = (tc == 0) ? p.r_init : p.hist + (size_t)(tc - 1) * B * N;
+    float r[4][NC];
+    rows_load<NC>(prev, N, B, 16 * bt + 4 * q, i0, r);
+    write_operand<NC>(xbuf + rt * TL::SLOTS, r, w, q, n);
+    publish_rowsum<NC>(psum[rt], r, w, q, n);
+    if (live[rt]) {
+      pair_store<NC>(p.rfrag, t, p.nbt, bt, w, lane, r);
+      if (t == T - 1) pair_zero_tail<NC>(p.rfrag, T, p.nbt, bt, w, lane);
+    }
+    gates_stage(gl + rt * 16 * GATE_KMAX, p.A, p.k, T, B, tc, bt, tid);
+  }
+  lds_barrier();
+
+  f32x4 acc[RT][NC];
+  bf16x8 wf[StreamCfg<NC, RT>::PD][StreamCfg<NC, RT>::KG];
+  gated_products<NC, false, RT>(xbuf, (const bf16x8*)p.Wpack, p.A, gl, gates_active(gl, p.k, lane, RT), p.k, T, B, t0,
+                                16 * bt0 + 4 * q, p.J1, w, lane, acc, wf, false, false);
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    if (!live[rt]) continue;
+    const int bt = bt0 + (rt & 1), t = t0 + (rt >> 1);
+    float s[4];
+    read_rowsum(psum[rt], q, s);
+    float d[4][NC];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+#pragma unroll
+      for (int c = 0; c < NC; ++c) {
+        float F, D;
+        act_fast<ACT>(acc[rt][c][e] + p.J0 * s[e], F, D);
+        d[e][c] = ((16 * bt + 4 * q + e < B) && (i0 + c < N)) ? p.alpha * D : 0.f;
+      }
+    }
+    side_store<NC, f16x4, _Float16>(p.dfrag + side_offset<NC>(t, p.nbt, bt, w, lane), d);
   }
 }
 
@@ -1236,6 +1299,15 @@ hipError_t ring_launch_rebuild(const RingFwdArgs& a, int NCv, hipStream_t st) {
   }
   const int rt = stream_row_tiles(NCv, a.nbt, true);
   hipError_t e = hipErrorInvalidValue;
+  // widest tiling, staged gates, more than one step and batch tile: four row tiles (two batch tiles x two steps)
+  // share every fetched weight fragment.  RINGATTR_REBUILD_TILES=2 keeps the two-tile kernel (cross-checks).
+  static const bool four = [] { const char* v = getenv("RINGATTR_REBUILD_TILES"); return !(v && v[0] == '2'); }();
+  if (four && NCv == 8 && rt == 2 && a.k <= GATE_KMAX && a.T >= 2) {
+    constexpr int NC = 8;
+    RING_DISPATCH_ACT(a.act, e = launch_stream(ring_rebuild_saved4_kernel<NC, ACT>, dim3((a.nbt + 1) / 2, (a.T + 1) / 2),
+                                               4 * Tile<NC>::SLOTS * sizeof(bf16x8), st, a));
+    return e;
+  }
   RING_DISPATCH_NC(NCv, RING_DISPATCH_ACT(a.act, RING_DISPATCH_RT(rt,
       e = launch_stream(ring_rebuild_saved_kernel<NC, ACT, RT>, dim3((a.nbt + RT - 1) / RT, a.T), 0, st, a))));
   return e;
