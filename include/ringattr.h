@@ -236,6 +236,11 @@ RINGATTR_API int ringattr_clip_adam_counted(int n_tensors, void* const* params, 
 #define RINGATTR_K_DW 4
 #define RINGATTR_K_DW_REDUCE 5
 RINGATTR_API int ringattr_profile_enable(int on);
+/* Time segments the weight-gradient kernel of a backward at this shape is launched in (1: one launch per group of three
+ * matrices; long sequences are cut so that the workgroups that share operand streams stay aligned in L2; the
+ * environment variable RINGATTR_DW_SEGMENT, K chunks of 32 samples per workgroup and launch, default 640, 0 = never
+ * cut, is read at every call).  Host arithmetic only; -1 for an unsupported shape. */
+RINGATTR_API int ringattr_dw_segments(int N, int a_dim, int seq_len, int batch_size);
 /* Name of the kernel this process launched last in slot `kernel` (RINGATTR_K_*), e.g.
  * "ring_fwd_res256_kernel<1,true,true,false>" (demangled, no return type, parameter list or blanks), or the empty
  * string if the slot has not launched yet.  For benchmarks that pair a timing with a stored counter profile. */

@@ -65,6 +65,7 @@ PROTOTYPES = {
     "ringattr_profile_enable": (c_int, [c_int]),
     "ringattr_profile_read": (c_int, [ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_longlong)]),
     "ringattr_last_kernel_name": (c_int, [c_int, ctypes.c_char_p, ctypes.c_size_t]),
+    "ringattr_dw_segments": (c_int, [c_int] * 4),
     "fwd_cuda": (None, [c_void_p, c_void_p, c_float, c_float, c_void_p, c_void_p, c_void_p, c_float,
                         c_int, c_int, c_int, c_int, c_int]),
     "bwd_cuda": (None, [c_void_p, c_void_p, c_void_p, c_float, c_float, c_void_p, c_void_p, c_void_p, c_void_p,

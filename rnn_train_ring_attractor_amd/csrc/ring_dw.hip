@@ -263,11 +263,26 @@ static hipError_t launch_group(const RingDwArgs& a, int mg, unsigned blocks, int
 // sequence is therefore cut into segments in time, one launch each (a launch boundary re-aligns the workgroups);
 // the launches after the first add to the partial sums.  RINGATTR_DW_SEGMENT overrides the length (0: no cut).
 static int dw_segment_chunks() {
-  static const int v = [] {
-    const char* e = getenv("RINGATTR_DW_SEGMENT");
-    return e ? atoi(e) : 640;
-  }();
-  return v;
+  const char* e = getenv("RINGATTR_DW_SEGMENT");   // read at every call: tests switch it between calls
+  return e ? atoi(e) : 640;
+}
+
+// Time-step pairs per segment (whole pairs, so that a segment is a contiguous range of chunks).
+static long dw_pairs_per_segment(int nbt, int T, int nz) {
+  const int npairs = (T + 1) / 2;
+  const long nchunk = (long)nbt * npairs;
+  const int seg = dw_segment_chunks();
+  long pairs_per_seg = npairs;
+  if (seg > 0 && nz > 0 && nchunk / nz > seg) {
+    pairs_per_seg = ((long)seg * nz) / nbt;
+    if (pairs_per_seg < 1) pairs_per_seg = 1;
+  }
+  return pairs_per_seg;
+}
+
+int ring_dw_tiled_segments(int nbt, int T, int nz) {
+  const long per = dw_pairs_per_segment(nbt, T, nz);
+  return (int)(((T + 1) / 2 + per - 1) / per);
 }
 
 // One launch per group of three matrices (a_dim = 2 needs exactly one) and segment.
@@ -276,14 +291,7 @@ hipError_t ring_launch_dw_tiled(const RingDwArgs& a, int NC, hipStream_t st) {
   const unsigned blocks = (unsigned)(NB * NB * a.nz);
   const int nmg = (a.k + 3) / 3;
   const int npairs = (a.T + 1) / 2;
-  const long nchunk = (long)a.nbt * npairs;
-  const int seg = dw_segment_chunks();
-  // whole time-step pairs per segment, so that a segment is a contiguous range of chunks
-  long pairs_per_seg = npairs;
-  if (seg > 0 && nchunk / a.nz > seg) {
-    pairs_per_seg = ((long)seg * a.nz) / a.nbt;
-    if (pairs_per_seg < 1) pairs_per_seg = 1;
-  }
+  const long pairs_per_seg = dw_pairs_per_segment(a.nbt, a.T, a.nz);
   for (int mg = 0; mg < nmg; ++mg) {
     for (long p0 = 0; p0 < npairs; p0 += pairs_per_seg) {
       const long p1 = p0 + pairs_per_seg < npairs ? p0 + pairs_per_seg : npairs;

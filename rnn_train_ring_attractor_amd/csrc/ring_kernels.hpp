@@ -162,6 +162,9 @@ int ring_last_kernel_name(int id, char* buf, size_t n);
     hipLaunchKernelGGL(kern, grid, block, lds, st, __VA_ARGS__);           \
   } while (0)
 
+bool ring_dw_tiled_applicable(int NC);
+int ring_dw_tiled_segments(int nbt, int T, int nz);   // launches per matrix group of the tiled weight-gradient kernel
+
 // Optional event bracketing of launches (benchmark support).
 void ring_profile_set(int stride);
 bool ring_profile_on();

@@ -697,6 +697,12 @@ int ringattr_profile_enable(int on) {
   return RINGATTR_OK;
 }
 
+int ringattr_dw_segments(int N, int a_dim, int seq_len, int batch_size) {
+  Geo g;
+  if (make_geo(N, a_dim, seq_len, batch_size, g) != RINGATTR_OK) return -1;
+  return ring_dw_tiled_applicable(g.NC) ? ring_dw_tiled_segments(g.nbt, seq_len, g.nz) : 1;
+}
+
 int ringattr_last_kernel_name(int kernel, char* buf, size_t buf_bytes) {
   if (!buf || buf_bytes == 0) return fail(RINGATTR_ERR_INVALID, "ringattr_last_kernel_name: null buffer");
   if (kernel < 0 || kernel >= RINGATTR_NUM_KERNELS) return fail(RINGATTR_ERR_INVALID, "ringattr_last_kernel_name: no such kernel slot");

@@ -160,3 +160,20 @@ def test_generator_leading_zero_count_is_pythons_over_a_grid():
         n0 = lib.ringattr_generator_initial_zeros(T, ratio)
         assert torch.all(av[:, :n0] == 0)
         assert torch.all(av[:, n0:] != 0)
+
+
+def test_weight_gradient_segment_count(monkeypatch):
+    """Host arithmetic of the weight-gradient kernel's time segments: at most RINGATTR_DW_SEGMENT (default 640) K
+    chunks of 32 samples per workgroup and launch, whole time-step pairs per segment."""
+    from rnn_train_ring_attractor_amd import _lib
+    lib = _lib.load()
+    monkeypatch.delenv("RINGATTR_DW_SEGMENT", raising=False)
+    assert lib.ringattr_dw_segments(256, 2, 120, 4096) == 1          # 240 chunks per workgroup: one launch
+    assert lib.ringattr_dw_segments(512, 2, 512, 8192) == 13         # 8192 chunks per workgroup: 20 pairs per segment
+    assert lib.ringattr_dw_segments(1024, 2, 120, 2048) == 3
+    assert lib.ringattr_dw_segments(120, 2, 120, 64) == 1            # not the tiled kernel
+    monkeypatch.setenv("RINGATTR_DW_SEGMENT", "0")
+    assert lib.ringattr_dw_segments(512, 2, 512, 8192) == 1
+    monkeypatch.setenv("RINGATTR_DW_SEGMENT", "1")
+    assert lib.ringattr_dw_segments(256, 2, 33, 256) == 5            # 64 splits x 1 chunk = 4 of the 17 time-step pairs per segment
+    assert lib.ringattr_dw_segments(4096, 2, 8, 16) == -1

@@ -870,3 +870,39 @@ def test_reference_signature_entry_points(gpu_device):
     g = O.backward_dense(p["G"], p["A"], p["Wa"], -0.1, 0.1, p["Wo"], ref, p["r0"], 0.15, "tanh")
     assert O.cosine(gWo.cpu().numpy(), g["grad_Wo"]) >= GRAD_COS
     assert O.max_rel_err(gWa.cpu().numpy(), g["grad_Wa"]) <= GRAD_TOL
+
+
+@pytest.mark.parametrize("B,T,k,N,act", [(256, 33, 2, 256, "gelu"), (96, 21, 5, 512, "tanh"), (48, 13, 3, 1024, "silu")],
+                         ids=["n256", "n512_k5", "n1024"])
+def test_weight_gradient_time_segments_add_up(B, T, k, N, act, gpu_device, monkeypatch):
+    """The weight-gradient kernel cuts long sequences into time segments, one launch each, whose partial sums add up
+    (RINGATTR_DW_SEGMENT = K chunks per workgroup and launch).  Tiny segments here (odd lengths, several matrix
+    groups, every tiled geometry): the gradients must equal those of one launch to fp32 summation order and meet the
+    fp64 oracle; 0 switches the cut off."""
+    from rnn_train_ring_attractor_amd import ring_rnn_cuda_func
+    print(f"[case] dW segments B={B} T={T} k={k} N={N} {act}", flush=True)
+    p = make_problem(77, B, T, k, N, action="dense")
+    J0, J1 = -0.05, 0.4
+
+    from rnn_train_ring_attractor_amd import _lib
+
+    def run(segment):
+        monkeypatch.setenv("RINGATTR_DW_SEGMENT", str(segment))
+        Wa, Wo = _t(p["Wa"], gpu_device).requires_grad_(True), _t(p["Wo"], gpu_device).requires_grad_(True)
+        h = ring_rnn_cuda_func(_t(p["A"], gpu_device), Wa, J0, J1, Wo, _t(p["r0"], gpu_device), 0.15, act)
+        h.backward(_t(p["G"], gpu_device))
+        torch.cuda.synchronize()
+        segments = _lib.load().ringattr_dw_segments(N, k, T, B)       # under the environment just set
+        return Wa.grad.cpu().numpy(), Wo.grad.cpu().numpy(), segments, _lib.last_kernel_names().get("dw", "")
+
+    one = run(0)
+    assert one[2] == 1 and "ring_dw_direct_kernel" in one[3]
+    for segment in (1, 3):
+        cut = run(segment)
+        assert cut[2] >= 2
+        assert O.max_rel_err(cut[0], one[0]) <= 1e-5 and O.max_rel_err(cut[1], one[1]) <= 1e-5
+    again = run(3)
+    assert np.array_equal(again[0], cut[0]) and np.array_equal(again[1], cut[1])    # and it is repeatable bit for bit
+    ref, _ = O.forward_dense(p["A"], p["Wa"], J0, J1, p["Wo"], p["r0"], 0.15, act)
+    g = O.backward_dense(p["G"], p["A"], p["Wa"], J0, J1, p["Wo"], ref, p["r0"], 0.15, act)
+    assert O.max_rel_err(cut[1], g["grad_Wo"]) <= GRAD_TOL and O.max_rel_err(cut[0], g["grad_Wa"]) <= GRAD_TOL
