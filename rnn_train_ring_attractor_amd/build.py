@@ -15,7 +15,7 @@ PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(PKG_DIR, "csrc")
 INCLUDE = os.path.join(os.path.dirname(PKG_DIR), "include")
 LIB_PATH = os.path.join(PKG_DIR, "libringattr.so")
-SOURCES = ["ring_kernels.hip", "ring_res256.hip", "ring_dw.hip", "ring_loss.hip", "ring_gain.hip", "ring_bign.hip", "ring_block.hip", "ring_aux.hip", "ringattr_api.hip"]
+SOURCES = ["ring_kernels.hip", "ring_res256.hip", "ring_cluster.hip", "ring_dw.hip", "ring_loss.hip", "ring_gain.hip", "ring_bign.hip", "ring_block.hip", "ring_aux.hip", "ringattr_api.hip"]
 ARCH = os.environ.get("RINGATTR_ARCH", "gfx950")
 
 HIPCC_FLAGS = [
@@ -36,6 +36,7 @@ def hipcc_path() -> str:
 # VGPRs (the AGPR file is full of weights there), which spares one v_accvgpr_read per result register.
 PER_SOURCE_FLAGS = {
     "ring_res256.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
+    "ring_cluster.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
 }
 
 

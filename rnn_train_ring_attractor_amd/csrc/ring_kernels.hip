@@ -18,6 +18,8 @@
 //   stays zero.
 //   split_k = 1 (NC = 4 only): contraction position kappa stands for neuron split_k_neuron(kappa) and output
 //   column n of tile c for neuron 64*w + 32*(c/2) + 2*n + c%2: the pipelined weight-resident forward's order.
+//   split_k = 2 (NC = 8 only): the same column order (neuron 128*w + 32*(c/2) + 2*n + c%2) with the contraction in
+//   neuron order: the cluster forward's.
 // ------------------------------------------------------------------------------------------------
 __device__ __forceinline__ bf16x8 pack_fragment(const float* __restrict__ Wo, const float* __restrict__ Wa, size_t u,
                                                 int N, int NC, int transposed, int split_k, float scale0, float shift0) {
@@ -32,7 +34,7 @@ __device__ __forceinline__ bf16x8 pack_fragment(const float* __restrict__ Wo, co
   const int mm = (int)(v >> 2);
   const int q = lane >> 4, n = lane & 15;
   // split_k: the output columns follow the pipelined forward's ownership as well (tile c = 2*h + cc of wave w)
-  const int col = split_k ? 64 * w + 32 * (c >> 1) + 2 * n + (c & 1) : 16 * NC * w + NC * n + c;
+  const int col = split_k ? 16 * NC * w + 32 * (c >> 1) + 2 * n + (c & 1) : 16 * NC * w + NC * n + c;
   const int k0 = 32 * kc + 8 * q;
   const float* W = (mm == 0) ? Wo : Wa + (size_t)(mm - 1) * N * N;
   bf16x8 pk;
@@ -50,7 +52,7 @@ __device__ __forceinline__ bf16x8 pack_fragment(const float* __restrict__ Wo, co
   }
 #pragma unroll
   for (int x = 0; x < 8; ++x) {
-    const int kk = split_k ? split_k_neuron(k0 + x) : k0 + x;
+    const int kk = split_k == 1 ? split_k_neuron(k0 + x) : k0 + x;
     float val = 0.f;
     if (col < N && kk < N) {
       val = transposed ? W[(size_t)kk * N + col] : W[(size_t)col * N + kk];
@@ -1141,7 +1143,8 @@ hipError_t ring_profile_collect(double* ms, long long* launches) {
 hipError_t ring_launch_pack2(const float* Wo, const float* Wa, int N, int k, int NC, void* out, int transposed,
                              int split_k, float scale0, float shift0, void* out2, int transposed2, int split_k2,
                              float scale2, float shift2, hipStream_t st) {
-  if ((split_k || (out2 && split_k2)) && NC != 4) return hipErrorInvalidValue;
+  auto order_ok = [&](int sk) { return sk == 0 || (sk == 1 && NC == 4) || (sk == 2 && NC == 8); };
+  if (!order_ok(split_k) || (out2 && !order_ok(split_k2))) return hipErrorInvalidValue;
   const size_t total = (size_t)(1 + k) * 4 * NC * 2 * NC * 64 * (out2 ? 2 : 1);
   const int blocks = (int)((total + 255) / 256 < 4096 ? (total + 255) / 256 : 4096);
   ProfScope prof(0, st);
@@ -1235,6 +1238,7 @@ static bool step_prefers_wide(int NCv, int nbt, int k) {
 // (wide rings, and the split forward of small batches) do not.
 bool ring_fwd_forms_loss_sums(const RingFwdArgs& a, int NCv) {
   if (ring_uses_step_kernels(a.N, a.k, NCv, a.nbt)) return false;
+  if (a.cluster_ws) return false;
   if (!a.dfrag && !a.rfrag && NCv >= 4 && a.nbt <= 64 && !ring_uses_resident(a.N, a.k)) {
     const char* v = getenv("RINGATTR_SPLIT_FORWARD");
     if (!(v && v[0] == '0')) return false;
@@ -1260,6 +1264,7 @@ hipError_t ring_launch_fwd(const RingFwdArgs& a, int NCv, hipStream_t st) {
     }
   }
   if (ring_uses_resident(a.N, a.k)) return ring_launch_fwd_res256(a, st);
+  if (a.cluster_ws) return ring_launch_fwd_cluster(a, st);
   const int rt = stream_row_tiles(NCv, a.nbt, false);
   hipError_t e = hipErrorInvalidValue;
   if (weights_fit_lds(NCv, a.k, 8 * 1024)) {

@@ -17,6 +17,9 @@ struct RingFwdArgs {
   // Loss head's per-row sums (sum_i r_i cos(phi_i), sum_i r_i sin(phi_i), sum_i |r_i|, -) of every history row
   // [T*B], written by the weight-resident forward kernel itself when non-null (other kernels ignore it).
   ring_f32x4* loss_stats = nullptr;
+  // Non-null: run the four-compute-unit cluster kernel (ring_cluster.hip) with this scratch area of
+  // ring_cluster_workspace_bytes(nbt) bytes; Wpack is then in that kernel's column order with J1 * Wo + J0 as matrix 0.
+  void* cluster_ws = nullptr;
 };
 
 struct RingBpttArgs {
@@ -71,6 +74,21 @@ bool ring_res256_applicable(int N, int k);
 bool ring_uses_resident(int N, int k);   // applicable and not disabled by RINGATTR_STREAMING=1
 hipError_t ring_launch_fwd_res256(const RingFwdArgs& a, hipStream_t st);
 hipError_t ring_launch_bptt_res256(const RingBpttArgs& a, hipStream_t st);
+
+// Weight-resident forward over clusters of four compute units for 256 < N <= 512, a_dim == 2 (ring_cluster.hip).
+struct RingClusterArgs {
+  void* xchg;        // [2][2 * npairs][16 K chunks][4][16 rows] x 16 bytes: the state in MFMA A-operand order
+  int* flags;        // [nclusters][ppc][16]: last state number published per (pair, member, wave)
+  int* hello;        // [nclusters][4]: XCC_ID + 1 of each member
+  int* host_err;     // word in pinned host memory, RING_CLUSTER_ERR_* when a wait ran out
+  int npairs, nclusters, ppc, spin_max;
+};
+enum { RING_CLUSTER_ERR_XCD = 1, RING_CLUSTER_ERR_START = 2, RING_CLUSTER_ERR_WAIT = 3 };
+bool ring_cluster_applicable(int N, int k);               // the shape alone
+size_t ring_cluster_workspace_bytes(int nbt);
+bool ring_uses_cluster(int N, int k, int nbt);            // applicable, switched on, and the device has the compute units
+int ring_cluster_error();                                 // the host word: non-zero once a cluster kernel gave up waiting
+hipError_t ring_launch_fwd_cluster(const RingFwdArgs& a, hipStream_t st);
 
 // Step-per-launch kernels for 512 < N <= 2048, NC in {16, 24, 32} (ring_bign.hip).
 bool ring_wide_applicable(int NC);

@@ -175,7 +175,8 @@ size_t ringattr_saved_bytes(int N, int a_dim, int seq_len, int batch_size) {
 size_t ringattr_fwd_workspace_bytes(int N, int a_dim, int seq_len, int batch_size) {
   Geo g;
   if (make_geo(N, a_dim, seq_len, batch_size, g) != RINGATTR_OK) return 0;
-  return g.wpack_bytes;
+  // (the cluster forward's exchange area is asked for wherever its shape applies, switched on or not)
+  return g.wpack_bytes + (ring_cluster_applicable(N, a_dim) ? ring_cluster_workspace_bytes(g.nbt) : 0);
 }
 
 size_t ringattr_bwd_workspace_bytes(int N, int a_dim, int seq_len, int batch_size, int have_saved) {
@@ -239,14 +240,25 @@ static int fwd_impl(const void* A, const void* Wa, float J0, float J1, const voi
     return fail(RINGATTR_ERR_WORKSPACE, "ringattr_fwd: workspace of %zu bytes needed, %zu given", g.wpack_bytes,
                 workspace ? workspace_bytes : (size_t)0);
   hipStream_t st = static_cast<hipStream_t>(stream);
+  if (const int ce = ring_cluster_error())
+    return fail(RINGATTR_ERR_HIP,
+                "an earlier cluster forward gave up waiting for a sibling workgroup (code %d: 1 members on different "
+                "XCDs, 2 members not resident together, 3 a published state never arrived); its results are invalid. "
+                "Set RINGATTR_CLUSTER=0 and restart the process",
+                ce);
 
   // With a saved buffer the same launch also writes the transposed copy the backward will need behind the saved
-  // activations.  The weight-resident kernels take Wo as J1 * Wo + J0 in both copies.
+  // activations.  The weight-resident kernels take Wo as J1 * Wo + J0 in both copies; the cluster forward takes it so
+  // in its own copy and leaves the plain transposed one the streaming BPTT expects.
   const int resident = ring_uses_resident(N, a_dim) ? 1 : 0;
+  const size_t cluster_bytes = ring_cluster_applicable(N, a_dim) ? ring_cluster_workspace_bytes(g.nbt) : 0;
+  const bool cluster = !resident && ring_uses_cluster(N, a_dim, g.nbt) && !ring_uses_step_kernels(N, a_dim, g.NC, g.nbt) &&
+                       workspace_bytes >= g.wpack_bytes + cluster_bytes;
   void* wpack_t = saved ? (char*)saved + g.side_bytes + g.pair_bytes : nullptr;
-  const float s0 = resident ? J1 : 1.f, h0 = resident ? J0 : 0.f;
-  hipError_t e = ring_launch_pack2((const float*)Wo, (const float*)Wa, N, a_dim, g.NC, workspace, 0, resident, s0, h0,
-                                   wpack_t, 1, 0, s0, h0, st);
+  const float s0 = (resident || cluster) ? J1 : 1.f, h0 = (resident || cluster) ? J0 : 0.f;
+  const float s2 = resident ? J1 : 1.f, h2 = resident ? J0 : 0.f;
+  hipError_t e = ring_launch_pack2((const float*)Wo, (const float*)Wa, N, a_dim, g.NC, workspace, 0, cluster ? 2 : resident,
+                                   s0, h0, wpack_t, 1, 0, s2, h2, st);
   if (e != hipSuccess) return hip_fail(e, "pack weights");
   if (saved)
     saved_note_put(SavedNote{saved, ring_uses_step_kernels(N, a_dim, g.NC, g.nbt) ? 3 : (resident ? 2 : 1), N, a_dim,
@@ -268,6 +280,7 @@ static int fwd_impl(const void* A, const void* Wa, float J0, float J1, const voi
   a.B = batch_size;
   a.nbt = g.nbt;
   a.act = activation_type;
+  a.cluster_ws = cluster ? (char*)workspace + g.wpack_bytes : nullptr;
   // the persistent forward kernels form the loss head's row sums themselves
   a.loss_stats = ring_fwd_forms_loss_sums(a, g.NC) ? loss_stats : nullptr;
   if (stats_done) *stats_done = a.loss_stats != nullptr;
