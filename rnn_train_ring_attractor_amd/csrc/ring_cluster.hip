@@ -1,17 +1,17 @@
-// Weight-resident forward for 256 < N <= 512 (NPAD = 512, NC = 8), a_dim = 2: the weights stay on chip, spread
-// over a cluster of four compute units.
+// Weight-resident forward for N = 512 (NC = 8), a_dim = 2: the weights stay on chip, spread over a cluster of four
+// compute units.
 //
-// [Wo|Wl|Wr] in bf16 is 1.5 MiB at NPAD = 512, four times what one compute unit can hold (the streaming kernels
+// [Wo|Wl|Wr] in bf16 is 1.5 MiB at N = 512, four times what one compute unit can hold (the streaming kernels
 // therefore pull all of it from L2 once per step and batch-tile pair, and a step is bound by that stream).  Here
 // four workgroups on four compute units of ONE XCD (one L2) form a cluster: member m keeps the slices for output
 // neurons 128 m .. 128 m + 127 for the whole sequence -- the two gated matrices in accumulation VGPRs, Wo in LDS,
-// exactly the split of the N <= 256 weight-resident kernels -- and computes those neurons for all the cluster's
-// batch rows.  What the members exchange per step is the new state in bf16, in the layout the next step's MFMA
-// A operand is read in:
-//   xchg[(t) & 1][batch tile][K chunk kc][q][row] x 16 bytes  =  r_t[row][32 kc + 8 q .. + 7],
-// written with ordinary stores (they reach the XCD's L2, vmcnt tells when) and read with device-scope loads (which
-// miss the vector L1).  A flag per (batch-tile pair, member, wave) carries the number of the last state written;
-// a reader polls the sixteen flags of a pair before it loads the pair's operand.  The buffer has two halves by step
+// the split of the N <= 256 weight-resident kernels -- and computes those neurons for all the cluster's batch rows.
+// What the members exchange per step is the new state in bf16, in the layout the next step's MFMA A operand is
+// read in:
+//   xchg[t & 1][batch tile][K chunk kc][q][row] x 16 bytes  =  r_t[row][32 kc + 8 q .. + 7],
+// written with ordinary stores (they reach the XCD's L2; vmcnt tells when) and read with device-scope loads (which
+// miss the vector L1).  A flag per (batch-tile pair, member, wave) carries the number of the last state written; a
+// reader looks at the 32 flags of a pair before it loads the pair's operand.  The buffer has two halves by step
 // parity: nobody can write state t+1 of a pair before every member has published state t of it, i.e. has finished
 // reading state t-1, which is what lives in the half being overwritten.
 //
@@ -22,10 +22,9 @@
 // workgroup's abort word and a word in host memory and all its waves leave at the next common point; the siblings
 // then run into their own time-outs.  The host finds the word set on its next call into the library.
 //
-// A cluster works on its batch-tile pairs round robin inside a step (pair-steps), so that the state a pair-step
-// needs was produced a whole round earlier and its flags are normally up when it looks; two batch tiles share every
-// LDS fetch of a Wo fragment.  Per pair-step a wave (one per SIMD, two column tiles = 32 neurons = one K chunk of the
-// next step's operand) issues 192 MFMAs.
+// A cluster works on its batch-tile pairs (32 rows) round robin inside a step -- pair-steps -- so that the state a
+// pair-step needs was produced a whole round earlier and its flags are normally up when a wave looks; two batch tiles
+// share every LDS fetch of a Wo fragment.
 #include "ring_common.hpp"
 #include "ring_kernels.hpp"
 
@@ -35,424 +34,15 @@ namespace {
 
 constexpr int C_NC = 8;
 constexpr int C_KCH = 16;
-constexpr int C_WFR = 2 * C_KCH - 1;              // Wo fragments of a wave kept in LDS (its last one stays in registers)
-constexpr int C_WSLOTS = 4 * C_WFR * 64;
 constexpr int C_TILE_UNITS = C_KCH * 4 * 16;      // 16-byte units of one batch tile's operand
 constexpr int C_XSLOTS = 2 * C_TILE_UNITS;
-constexpr size_t C_BIN_BYTES = 128 * 1024;        // target of the pipelined kernel's stores that have nothing to store
-constexpr size_t C_LDS_BYTES = (size_t)(C_WSLOTS + C_XSLOTS) * 16 + 256 + 64;   // + gates, abort word
-
-__device__ __forceinline__ f32x4 xchg_load16(const void* ptr) {
-  f32x4 v;
-  asm volatile("global_load_dwordx4 %0, %1, off sc1" : "=&v"(v) : "v"(ptr) : "memory");
-  return v;
-}
-// Stores whose instruction count the waits below rely on (one instruction each, by construction).
-__device__ __forceinline__ void store4(void* ptr, unsigned v) {
-  asm volatile("global_store_dword %0, %1, off" ::"v"(ptr), "v"(v) : "memory");
-}
-__device__ __forceinline__ void store8(void* ptr, f32x2 v) {
-  asm volatile("global_store_dwordx2 %0, %1, off" ::"v"(ptr), "v"(v) : "memory");
-}
-__device__ __forceinline__ void store16(void* ptr, f32x4 v) {
-  asm volatile("global_store_dwordx4 %0, %1, off" ::"v"(ptr), "v"(v) : "memory");
-}
-
-template <int K>
-__device__ __forceinline__ void wait_staged(f32x4 (&s)[8]) {
-  asm volatile("s_waitcnt vmcnt(%8)"
-               : "+v"(s[0]), "+v"(s[1]), "+v"(s[2]), "+v"(s[3]), "+v"(s[4]), "+v"(s[5]), "+v"(s[6]), "+v"(s[7])
-               : "n"(K)
-               : "memory");
-}
+constexpr size_t C_BIN_BYTES = 128 * 1024;        // where stores go that have nothing to store (see the kernel)
 
 __device__ __forceinline__ int flag_load(const int* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 __device__ __forceinline__ void flag_store(int* p, int v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 
-#ifdef CL_PROF
-#define CL2_DECL() long long stamp_[10]; int item_ = 0
-#define CL2_STAMP(i) stamp_[i] = clock64()
-#define CL2_FLUSH() do { if (blk == 0 && tid == 0 && item_ >= 16 && item_ < 80) { for (int i_ = 0; i_ < 10; ++i_) g_cl_prof[(item_ - 16) * 16 + i_] = stamp_[i_]; g_cl_prof[(item_ - 16) * 16 + 10] = up; } ++item_; } while (0)
-#else
-#define CL2_DECL() do { } while (0)
-#define CL2_STAMP(i) do { } while (0)
-#define CL2_FLUSH() do { } while (0)
-#endif
-#ifdef CL_PROF
-__device__ long long g_cl_prof[64 * 16];
-#define CL_STAMP(i) do { if (blk == 0 && tid == 0 && prof_row >= 0 && prof_row < 64) g_cl_prof[prof_row * 16 + (i)] = clock64(); } while (0)
-#else
-#define CL_STAMP(i) do { } while (0)
-#endif
-
 }  // namespace
 
-#ifdef CL_PROF
-extern "C" __attribute__((visibility("default"))) int ringattr_exp_cl_prof(long long* out) {
-  return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(g_cl_prof), sizeof(long long) * 64 * 16);
-}
-#endif
-
-// FULL: N == 512 and B % 32 == 0 (no masking, counted waits).
-template <int ACT, bool SAVE, bool FULL>
-__global__ __launch_bounds__(256) void ring_fwd_cluster_kernel(RingFwdArgs p, RingClusterArgs c) {
-  extern __shared__ __attribute__((aligned(16))) char smem[];
-  bf16x8* wlds = reinterpret_cast<bf16x8*>(smem);
-  bf16x8* xs = wlds + C_WSLOTS;
-  int* misc = reinterpret_cast<int*>(xs + C_XSLOTS);   // [0]: abort
-  bf16x8* const xchg = reinterpret_cast<bf16x8*>(c.xchg);
-
-  const int tid = threadIdx.x, v = tid >> 6, lane = tid & 63, q = lane >> 4, n = lane & 15;
-  const int blk = blockIdx.x, xcd = blk & 7, gi = blk >> 3, m = gi & 3, cl = (gi >> 2) * 8 + xcd;
-  if (cl >= c.nclusters) return;
-  const int N = p.N, B = p.B, T = p.T, nbt = p.nbt;
-  const int my_ppc = (c.npairs - cl + c.nclusters - 1) / c.nclusters;   // pairs cl, cl + nclusters, ...
-  const int vu = __builtin_amdgcn_readfirstlane(v);
-
-  // ---- handshake: all four members resident, on one XCD ----
-  if (tid == 0) misc[0] = 0;
-  if (v == 0) {
-    const int mine = (__builtin_amdgcn_s_getreg(20 | (0 << 6) | (3 << 11)) & 15) + 1;   // XCC_ID + 1
-    if (lane == 0) flag_store(c.hello + cl * 4 + m, mine);
-    int bad = 0;
-    for (int spins = 0;; ++spins) {
-      const int h = lane < 4 ? flag_load(c.hello + cl * 4 + lane) : mine;
-      if (__ballot(h == 0) == 0) {
-        bad = __ballot(h != mine) != 0 ? 1 : 0;
-        break;
-      }
-      if (spins > c.spin_max) {
-        bad = 2;
-        break;
-      }
-      __builtin_amdgcn_s_sleep(8);
-    }
-    if (bad && lane == 0) {
-      misc[0] = 1;
-      *c.host_err = bad == 1 ? RING_CLUSTER_ERR_XCD : RING_CLUSTER_ERR_START;
-    }
-  }
-
-  // ---- resident weights ----
-  bf16x8 wreg[2][2][C_KCH];
-  bf16x8 wo_last;
-  bf16x8* wl = wlds + (size_t)(v * C_WFR) * 64 + lane;
-  {
-    const bf16x8* Wp = reinterpret_cast<const bf16x8*>(p.Wpack);
-#pragma unroll
-    for (int cc = 0; cc < 2; ++cc)
-#pragma unroll
-      for (int kc = 0; kc < C_KCH; ++kc) {
-        const int ct = 2 * v + cc;
-        const bf16x8 f0 = Wp[((size_t)((0 * 4 + m) * C_NC + ct) * C_KCH + kc) * 64 + lane];
-        if (cc * C_KCH + kc < C_WFR) wl[(cc * C_KCH + kc) * 64] = f0;
-        else wo_last = f0;
-        wreg[0][cc][kc] = Wp[((size_t)((1 * 4 + m) * C_NC + ct) * C_KCH + kc) * 64 + lane];
-        wreg[1][cc][kc] = Wp[((size_t)((2 * 4 + m) * C_NC + ct) * C_KCH + kc) * 64 + lane];
-        asm volatile("" : "+a"(wreg[0][cc][kc]));
-        asm volatile("" : "+a"(wreg[1][cc][kc]));
-      }
-  }
-  lds_barrier();
-  if (misc[0]) return;
-
-  const float oma = 1.f - p.alpha;
-  const ActScale asc = act_scale_make(p.alpha);
-  const int i0 = 128 * m + 32 * v + 2 * n;            // this lane's two neurons (one per column tile)
-  // their place in the common tile order of the saved buffers (tile c, column n' <-> neuron 128 m + 8 n' + c)
-  const int lane_c = (lane & 48) | (4 * v + (n >> 2)), c0 = 2 * (n & 3);
-  const size_t xhalf = (size_t)2 * c.npairs * C_TILE_UNITS;   // units per parity half of the exchange buffer
-
-  f32x4 sreg[8];              // this wave's quarter of the next pair's operand, in flight
-  bool prefetched = false;
-  int pend_idx = -1, pend_val = 0;   // flag of the last pair-step whose exchange stores are not yet published
-  int nst = 0;                       // stores the last pair-step's epilogue issued (unmasked variant: exact)
-
-  auto signal_pending = [&]() {   // only behind a wait that covers the exchange stores
-    if (pend_idx >= 0 && lane == 0) flag_store(c.flags + pend_idx, pend_val);
-    pend_idx = -1;
-  };
-  auto flags_up = [&](int pl, int need) {
-    const int f = lane < 16 ? flag_load(c.flags + ((size_t)cl * c.ppc + pl) * 16 + lane) : need;
-    return __ballot(f < need) == 0;
-  };
-  auto issue_xchg_loads = [&](int t, int pr) {
-    const bf16x8* src = xchg + (size_t)(t & 1) * xhalf + (size_t)(2 * pr) * C_TILE_UNITS + v * 512 + lane;
-#pragma unroll
-    for (int j = 0; j < 8; ++j) sreg[j] = xchg_load16(src + j * 64);
-  };
-
-  for (int t = 0; t < T; ++t) {
-    for (int pl = 0; pl < my_ppc; ++pl) {
-      const int pr = cl + c.nclusters * pl;
-#ifdef CL_PROF
-      const int prof_row = (t - 4) * my_ppc + pl;   // rows 0.. from step 4 on
-      const bool was_prefetched = prefetched;
-#endif
-      CL_STAMP(0);
-      lds_barrier();   // every wave has finished reading the operand of the previous pair-step
-      CL_STAMP(1);
-      if (t == 0) {
-        // the first operand comes from r_init
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          const int u = v * 512 + j * 64 + lane;
-          const int tl = u >> 10, kc = (u >> 6) & 15, qq = (u >> 4) & 3, row = u & 15;
-          const int b = 32 * pr + 16 * tl + row, k0 = 32 * kc + 8 * qq;
-          bf16x8 pk;
-          if (FULL || (b < B && k0 + 8 <= N && (N & 3) == 0)) {
-            const f32x4* src = reinterpret_cast<const f32x4*>(p.r_init + (size_t)b * N + k0);
-            const f32x4 lo = src[0], hi = src[1];
-#pragma unroll
-            for (int x = 0; x < 4; ++x) {
-              pk[x] = (__bf16)lo[x];
-              pk[4 + x] = (__bf16)hi[x];
-            }
-          } else {
-#pragma unroll
-            for (int x = 0; x < 8; ++x) pk[x] = (__bf16)((b < B && k0 + x < N) ? p.r_init[(size_t)b * N + k0 + x] : 0.f);
-          }
-          xs[u] = pk;
-        }
-      } else {
-        if (!prefetched) {
-          asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-          signal_pending();
-          bool up = false;
-          for (int spins = 0; spins <= c.spin_max; ++spins) {
-            if ((up = flags_up(pl, t))) break;
-            __builtin_amdgcn_s_sleep(2);
-          }
-          if (up) {
-            issue_xchg_loads(t, pr);
-          } else if (lane == 0) {
-            misc[0] = 1;
-            *c.host_err = RING_CLUSTER_ERR_WAIT;
-          }
-          wait_staged<0>(sreg);
-        } else if constexpr (FULL) {
-          // the prefetch is older than the nst stores of the pair-step in between, and nothing else was issued since
-          switch (nst) {
-            case 8: wait_staged<8>(sreg); break;
-            case 10: wait_staged<10>(sreg); break;
-            case 14: wait_staged<14>(sreg); break;
-            case 16: wait_staged<16>(sreg); break;
-            case 18: wait_staged<18>(sreg); break;
-            case 22: wait_staged<22>(sreg); break;
-            case 26: wait_staged<26>(sreg); break;
-            default: wait_staged<0>(sreg); break;
-          }
-        } else {
-          wait_staged<0>(sreg);
-        }
-#pragma unroll
-        for (int j = 0; j < 8; ++j) xs[v * 512 + j * 64 + lane] = __builtin_bit_cast(bf16x8, sreg[j]);
-        prefetched = false;
-      }
-      CL_STAMP(2);
-      lds_barrier();
-      if (misc[0]) return;
-      CL_STAMP(3);
-
-      // inputs of this pair-step's epilogue: previous state (fp32) and action gates of the lane's rows
-      f32x2 rold[2][4], gate[2][4];
-#pragma unroll
-      for (int tl = 0; tl < 2; ++tl)
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const int b = 32 * pr + 16 * tl + 4 * q + e;
-          const int bc = FULL ? b : (b < B ? b : B - 1);
-          gate[tl][e] = *reinterpret_cast<const f32x2*>(p.A + ((size_t)bc * T + t) * 2);
-          const float* prev = (t == 0 ? p.r_init : p.hist + (size_t)(t - 1) * B * N) + (size_t)bc * N + i0;
-          if (FULL) {
-            rold[tl][e] = *reinterpret_cast<const f32x2*>(prev);
-          } else {
-            rold[tl][e][0] = (b < B && i0 < N) ? prev[0] : 0.f;
-            rold[tl][e][1] = (b < B && i0 + 1 < N) ? prev[1] : 0.f;
-          }
-        }
-      // the next pair-step and whether its operand can be fetched under this one's products
-      int nt = t, npl = pl + 1;
-      if (npl == my_ppc) {
-        npl = 0;
-        nt = t + 1;
-      }
-      const bool look = nt < T && nt >= 1;
-      // (always issued: its arrival is also what tells that the previous pair-step's stores have landed)
-      const int nflag = flag_load(c.flags + ((size_t)cl * c.ppc + (look ? npl : pl)) * 16 + n);
-
-      // ---- products: P[tile][cc][matrix] ----
-      f32x4 P[2][2][3];
-      {
-        const f32x4 z = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int tl = 0; tl < 2; ++tl)
-#pragma unroll
-          for (int cc = 0; cc < 2; ++cc) P[tl][cc][0] = P[tl][cc][1] = P[tl][cc][2] = z;
-      }
-      bf16x8 af[2][2], wf[2][2];
-      auto frag_fetch = [&](auto kcv, int stg) {
-        constexpr int kc = decltype(kcv)::value;
-        af[stg][0] = xs[(0 * C_KCH + kc) * 64 + lane];
-        af[stg][1] = xs[(1 * C_KCH + kc) * 64 + lane];
-        wf[stg][0] = wl[(0 * C_KCH + kc) * 64];
-        if constexpr (C_KCH + kc < C_WFR) wf[stg][1] = wl[(1 * C_KCH + kc) * 64];
-        else wf[stg][1] = wo_last;
-      };
-      auto mfma_half = [&](auto halfv) {
-        constexpr int half = decltype(halfv)::value;
-        auto body = [&](auto jv) {
-          constexpr int kc = 8 * half + decltype(jv)::value, stg = kc & 1;
-          if constexpr (kc + 1 < C_KCH) {
-            frag_fetch(std::integral_constant<int, kc + 1>{}, stg ^ 1);
-            __builtin_amdgcn_sched_barrier(0);
-          }
-#pragma unroll
-          for (int cc = 0; cc < 2; ++cc) {
-            P[0][cc][1] = mfma16(af[stg][0], wreg[0][cc][kc], P[0][cc][1]);
-            P[1][cc][1] = mfma16(af[stg][1], wreg[0][cc][kc], P[1][cc][1]);
-            P[0][cc][2] = mfma16(af[stg][0], wreg[1][cc][kc], P[0][cc][2]);
-            P[1][cc][2] = mfma16(af[stg][1], wreg[1][cc][kc], P[1][cc][2]);
-            P[0][cc][0] = mfma16(af[stg][0], wf[stg][cc], P[0][cc][0]);
-            P[1][cc][0] = mfma16(af[stg][1], wf[stg][cc], P[1][cc][0]);
-          }
-          __builtin_amdgcn_sched_barrier(0);
-        };
-        body(std::integral_constant<int, 0>{});
-        body(std::integral_constant<int, 1>{});
-        body(std::integral_constant<int, 2>{});
-        body(std::integral_constant<int, 3>{});
-        body(std::integral_constant<int, 4>{});
-        body(std::integral_constant<int, 5>{});
-        body(std::integral_constant<int, 6>{});
-        body(std::integral_constant<int, 7>{});
-      };
-      frag_fetch(std::integral_constant<int, 0>{}, 0);
-      __builtin_amdgcn_s_setprio(1);
-      CL_STAMP(4);
-      mfma_half(std::integral_constant<int, 0>{});
-      CL_STAMP(5);
-      // The flag load above is younger than every store of the previous pair-step, and vector-memory operations
-      // leave the counter in issue order: once its value is here, those stores have reached L2.
-      asm volatile("" ::"v"(nflag) : "memory");
-      signal_pending();
-      if (look && __ballot(nflag < nt) == 0) {
-        issue_xchg_loads(nt, cl + c.nclusters * npl);
-        prefetched = true;
-      }
-      CL_STAMP(6);
-      mfma_half(std::integral_constant<int, 1>{});
-      __builtin_amdgcn_s_setprio(0);
-      CL_STAMP(7);
-
-      // ---- epilogue ----
-      const bool more = t + 1 < T;
-      float rn[2][4][2], dd[2][4][2];
-#pragma unroll
-      for (int tl = 0; tl < 2; ++tl)
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const int b = 32 * pr + 16 * tl + 4 * q + e;
-#pragma unroll
-          for (int cc = 0; cc < 2; ++cc) {
-            const float x = fmaf(gate[tl][e][1], P[tl][cc][2][e], fmaf(gate[tl][e][0], P[tl][cc][1][e], P[tl][cc][0][e]));
-            float aF, aD;
-            act_scaled<ACT>(x, asc, aF, aD);
-            float r1 = fmaf(oma, rold[tl][e][cc], aF);
-            if constexpr (!FULL) {
-              const bool ok = b < B && i0 + cc < N;
-              r1 = ok ? r1 : 0.f;
-              aD = ok ? aD : 0.f;
-            }
-            rn[tl][e][cc] = r1;
-            dd[tl][e][cc] = aD;
-          }
-        }
-      nst = 0;
-      CL_STAMP(8);
-#pragma unroll
-      for (int tl = 0; tl < 2; ++tl) {
-        const int bt = 2 * pr + tl;
-        const bool live = FULL || bt < nbt;
-        // history rows
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const int b = 16 * bt + 4 * q + e;
-          float* dst = p.hist + ((size_t)t * B + b) * N + i0;
-          if constexpr (FULL) {
-            store8(dst, f32x2{rn[tl][e][0], rn[tl][e][1]});
-          } else if (b < B) {
-            if (i0 < N) dst[0] = rn[tl][e][0];
-            if (i0 + 1 < N) dst[1] = rn[tl][e][1];
-          }
-        }
-        nst += 4;
-        if (SAVE && live) {
-          // alpha F'(re): the lane's two tiles lie side by side in the record
-          typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
-          const f16x8 dk = {(_Float16)dd[tl][0][0], (_Float16)dd[tl][1][0], (_Float16)dd[tl][2][0], (_Float16)dd[tl][3][0],
-                            (_Float16)dd[tl][0][1], (_Float16)dd[tl][1][1], (_Float16)dd[tl][2][1], (_Float16)dd[tl][3][1]};
-          store16(p.dfrag + side_offset<C_NC>(t, nbt, bt, m, lane_c) + 4 * c0, __builtin_bit_cast(f32x4, dk));
-          nst += 1;
-          // bf16 operand copies for the weight gradient: slot t' holds the state before step t'; an odd length's
-          // last pair has a zero second half
-          if (t == 0) {
-#pragma unroll
-            for (int cc = 0; cc < 2; ++cc) {
-              const bf16x4 pk = {(__bf16)rold[tl][0][cc], (__bf16)rold[tl][1][cc], (__bf16)rold[tl][2][cc], (__bf16)rold[tl][3][cc]};
-              store8(p.rfrag + pair_offset<C_NC>(0, nbt, bt, m * C_NC + c0 + cc, lane_c), __builtin_bit_cast(f32x2, pk));
-            }
-            nst += 2;
-          }
-          if (more || (T & 1)) {
-#pragma unroll
-            for (int cc = 0; cc < 2; ++cc) {
-              const bf16x4 pk = {(__bf16)rn[tl][0][cc], (__bf16)rn[tl][1][cc], (__bf16)rn[tl][2][cc], (__bf16)rn[tl][3][cc]};
-              store8(p.rfrag + pair_offset<C_NC>(t + 1, nbt, bt, m * C_NC + c0 + cc, lane_c),
-                     more ? __builtin_bit_cast(f32x2, pk) : f32x2{0.f, 0.f});
-            }
-            nst += 2;
-          }
-        }
-        if (more) {
-          // the next step's operand, for all four members
-          char* dst = reinterpret_cast<char*>(xchg + (size_t)((t + 1) & 1) * xhalf + (size_t)bt * C_TILE_UNITS +
-                                              ((4 * m + vu) * 4 + (n >> 2)) * 16 + 4 * q) + (n & 3) * 4;
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            const bf16x2 pk = {(__bf16)rn[tl][e][0], (__bf16)rn[tl][e][1]};
-            store4(dst + e * 16, __builtin_bit_cast(unsigned, pk));
-          }
-          nst += 4;
-        }
-      }
-      if (more) {
-        pend_idx = (int)(((size_t)cl * c.ppc + pl) * 16 + 4 * m + v);
-        pend_val = t + 1;
-      }
-      CL_STAMP(9);
-#ifdef CL_PROF
-      if (blk == 0 && tid == 0 && prof_row >= 0 && prof_row < 64) g_cl_prof[prof_row * 16 + 10] = was_prefetched;
-#endif
-    }
-  }
-  // (the last step publishes nothing: pend_idx is unset here)
-}
-
-// ------------------------------------------------------------------------------------------------
-// The unmasked forward (N == 512, B % 32 == 0), pipelined.
-//
-// One compute unit has one address path for vector memory, shared by its four waves, and every load or store
-// instruction of a wave occupies it for tens of cycles: issued in bursts between the products (as above) the ~190
-// memory instructions of a pair-step cost more time than its 768 MFMAs.  This variant
-//  * issues every vector-memory instruction of the time loop between MFMA groups: the stores of pair-step s-1 and the
-//    loads for s and s+1 ride in the product loop of pair-step s (all through inline assembly, so that their number
-//    is known and the waits can count: vector-memory operations leave the counter in issue order);
-//  * moves whole 16-byte pieces: a quad of lanes holds [4 rows][8 neurons] of a tile as 4 x 2 per lane, and a 4x4
-//    transpose inside the quad (DPP) turns that into one row's eight neurons per lane, for the history rows, the
-//    previous state and the exchanged operand alike;
-//  * fetches the action gates of a pair-step once per workgroup (one load by wave 0, through LDS).
-// ------------------------------------------------------------------------------------------------
 namespace {
 
 // lane j's a[i] <-> lane i's a[j] among the four lanes of a quad (j = lane & 3)
@@ -515,63 +105,66 @@ __device__ __forceinline__ float sload4(const void* sbase, unsigned voff) {
 }
 
 template <int K>
-__device__ __forceinline__ void vm_wait_x(f32x4 (&s)[8]) {
-  asm volatile("s_waitcnt vmcnt(%8)"
-               : "+v"(s[0]), "+v"(s[1]), "+v"(s[2]), "+v"(s[3]), "+v"(s[4]), "+v"(s[5]), "+v"(s[6]), "+v"(s[7])
-               : "n"(K)
-               : "memory");
-}
-template <int K>
-__device__ __forceinline__ void vm_wait_in(f32x4 (&l)[2][2], int& flag, float& gate) {
-  asm volatile("s_waitcnt vmcnt(%6)"
-               : "+v"(l[0][0]), "+v"(l[0][1]), "+v"(l[1][0]), "+v"(l[1][1]), "+v"(flag), "+v"(gate)
-               : "n"(K)
-               : "memory");
-}
-template <int K>
 __device__ __forceinline__ void vm_wait_plain() {
   asm volatile("s_waitcnt vmcnt(%0)" ::"n"(K) : "memory");
 }
 
 }  // namespace
 
-// The instruction stream of a pair-step is the same every time -- where there is nothing to store or to fetch, the
-// instruction goes to a scratch bin of the workspace or reads what is at hand -- so every wait below counts against a
-// fixed number of younger operations (anything the compiler adds on top only makes a wait stricter).  Per pair-step,
-// in issue order:
-//   slot 0        4 loads of the previous state, 1 of the next pair-step's gates, 1 of its flags          (6 loads)
-//   slots 1..6    the stores of the previous pair-step: 2 exchange, 4 history, [2 record, 4 operand copy] (NST)
-//   slot 8        wait for the six loads: vmcnt(NST); slots 8..11: the next pair-step's operand          (8 loads)
-//   after the products: wait for the two exchange stores: vmcnt(NST - 2 + 8), then the flag store         (1 store)
-//   [first step only: 4 stores of the operand copy's slot 0]
-//   staging of the next operand: wait for the 8 loads: vmcnt(1)
+// ------------------------------------------------------------------------------------------------
+// The kernel: two waves per SIMD.
+//
+// A wave that issues a store stands still until the store's data has left the register file (some 150 cycles for
+// 16 bytes per lane, with four waves going through the compute unit's one store path), and a wave in the vector-ALU
+// epilogue feeds the matrix pipe nothing: with one wave per SIMD a pair-step is the SUM of its products, its
+// epilogue and its stores.  Here the workgroup has eight waves.  Wave (v, h) owns ONE column tile, the 16 neurons
+// 128 m + 16 (2 v + h) .. + 15 (its slices of the gated matrices fill its 128 accumulation registers), and the two
+// halves h = 0 / 1 run half a pair-step apart:
+//        half 0:   products(s)     epilogue(s)   | staging(s+1) |  products(s+1)   epilogue(s+1)
+//        half 1:   epilogue(s-1)   products(s)   |              |  epilogue(s)     products(s+1)
+// so each SIMD always has one wave on the matrix pipe and one in the epilogue or its stores.  The staged operand of
+// pair-step s serves both halves and is replaced between two workgroup barriers.  (A cluster with a single pair has
+// nothing to run ahead of: the next pair-step needs this one's state, and both halves run in phase.)
+// ------------------------------------------------------------------------------------------------
+namespace {
+#ifndef C8_PRIO
+#define C8_PRIO 2
+#endif
+constexpr int C8_WFR = C_KCH - 1;                 // Wo fragments of a wave kept in LDS
+constexpr int C8_WSLOTS = 8 * C8_WFR * 64;
+constexpr size_t C8_LDS_BYTES = (size_t)(C8_WSLOTS + C_XSLOTS) * 16 + 2 * 256 + 64;
+}  // namespace
+
 template <int ACT, bool SAVE>
-__global__ __launch_bounds__(256) void ring_fwd_cluster_full_kernel(RingFwdArgs p, RingClusterArgs c) {
+__global__ __launch_bounds__(512) void ring_fwd_cluster8_kernel(RingFwdArgs p, RingClusterArgs c) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
   bf16x8* wlds = reinterpret_cast<bf16x8*>(smem);
-  bf16x8* xs = wlds + C_WSLOTS;
-  float* gl = reinterpret_cast<float*>(xs + C_XSLOTS);   // [32 rows][2] action gates of the current pair-step
-  int* misc = reinterpret_cast<int*>(gl + 64);           // [0]: abort
+  bf16x8* xs = wlds + C8_WSLOTS;
+  float* gl = reinterpret_cast<float*>(xs + C_XSLOTS);   // [2][32 rows][2] action gates, by pair-step parity
+  int* misc = reinterpret_cast<int*>(gl + 128);          // [0]: abort
   char* const xchg = reinterpret_cast<char*>(c.xchg);
-  constexpr int NST = SAVE ? 12 : 6;
+  constexpr int NSTE = SAVE ? 6 : 4;                     // stores of every epilogue: 2 exchange, 2 history, 2 record (+ 2 at even steps)
 
-  const int tid = threadIdx.x, v = tid >> 6, lane = tid & 63, q = lane >> 4, n = lane & 15, g4 = n >> 2, j4 = n & 3;
+  const int tid = threadIdx.x, w8 = tid >> 6, v = w8 & 3, h = w8 >> 2, lane = tid & 63, q = lane >> 4, n = lane & 15,
+            g4 = n >> 2, j4 = n & 3;
+  const int ct = 2 * v + h;
   const int blk = blockIdx.x, xcd = blk & 7, gi = blk >> 3, m = gi & 3, cl = (gi >> 2) * 8 + xcd;
   if (cl >= c.nclusters) return;
   const int B = p.B, T = p.T, nbt = p.nbt;
   constexpr int N = 512;
   const int my_ppc = (c.npairs - cl + c.nclusters - 1) / c.nclusters;
-  const int vu = __builtin_amdgcn_readfirstlane(v);
+  const int w8u = __builtin_amdgcn_readfirstlane(w8);
+  const bool skew = __builtin_amdgcn_readfirstlane(h) == 1 && my_ppc >= 2;   // this wave's epilogue runs a phase late
 
   if (tid == 0) misc[0] = 0;
-  if (v == 0) {
+  if (w8 == 0) {
     const int mine = (__builtin_amdgcn_s_getreg(20 | (0 << 6) | (3 << 11)) & 15) + 1;   // XCC_ID + 1
     if (lane == 0) flag_store(c.hello + cl * 4 + m, mine);
-    int bad = 0;
-    for (int spins = 0;; ++spins) {
-      const int h = lane < 4 ? flag_load(c.hello + cl * 4 + lane) : mine;
-      if (__ballot(h == 0) == 0) {
-        bad = __ballot(h != mine) != 0 ? 1 : 0;
+    int bad = c.spin_max < 0 ? 2 : 0;   // (a negative limit gives up at once: the host's way to exercise this exit)
+    for (int spins = 0; !bad; ++spins) {
+      const int hh = lane < 4 ? flag_load(c.hello + cl * 4 + lane) : mine;
+      if (__ballot(hh == 0) == 0) {
+        bad = __ballot(hh != mine) != 0 ? 1 : 0;
         break;
       }
       if (spins > c.spin_max) {
@@ -586,128 +179,58 @@ __global__ __launch_bounds__(256) void ring_fwd_cluster_full_kernel(RingFwdArgs 
     }
   }
 
-  bf16x8 wreg[2][2][C_KCH];
+  bf16x8 wreg[2][C_KCH];
   bf16x8 wo_last;
-  bf16x8* wl = wlds + (size_t)(v * C_WFR) * 64 + lane;
+  bf16x8* wl = wlds + (size_t)(w8 * C8_WFR) * 64 + lane;
   {
     const bf16x8* Wp = reinterpret_cast<const bf16x8*>(p.Wpack);
 #pragma unroll
-    for (int cc = 0; cc < 2; ++cc)
+    for (int kc = 0; kc < C_KCH; ++kc) {
+      wreg[0][kc] = Wp[((size_t)((1 * 4 + m) * C_NC + ct) * C_KCH + kc) * 64 + lane];
+      wreg[1][kc] = Wp[((size_t)((2 * 4 + m) * C_NC + ct) * C_KCH + kc) * 64 + lane];
+    }
 #pragma unroll
-      for (int kc = 0; kc < C_KCH; ++kc) {
-        const int ct = 2 * v + cc;
-        wreg[0][cc][kc] = Wp[((size_t)((1 * 4 + m) * C_NC + ct) * C_KCH + kc) * 64 + lane];
-        wreg[1][cc][kc] = Wp[((size_t)((2 * 4 + m) * C_NC + ct) * C_KCH + kc) * 64 + lane];
+    for (int k8 = 0; k8 < C_KCH; k8 += 8) {
+      bf16x8 f[8];
+#pragma unroll
+      for (int x = 0; x < 8; ++x) f[x] = Wp[((size_t)((0 * 4 + m) * C_NC + ct) * C_KCH + k8 + x) * 64 + lane];
+#pragma unroll
+      for (int x = 0; x < 8; ++x) {
+        if (k8 + x < C8_WFR) wl[(k8 + x) * 64] = f[x];
+        else wo_last = f[x];
       }
+    }
 #pragma unroll
-    for (int cc = 0; cc < 2; ++cc)
-#pragma unroll
-      for (int k8 = 0; k8 < C_KCH; k8 += 8) {
-        bf16x8 f[8];
-#pragma unroll
-        for (int x = 0; x < 8; ++x) f[x] = Wp[((size_t)((0 * 4 + m) * C_NC + 2 * v + cc) * C_KCH + k8 + x) * 64 + lane];
-#pragma unroll
-        for (int x = 0; x < 8; ++x) {
-          if (cc * C_KCH + k8 + x < C_WFR) wl[(cc * C_KCH + k8 + x) * 64] = f[x];
-          else wo_last = f[x];
-        }
-      }
-#pragma unroll
-    for (int cc = 0; cc < 2; ++cc)
-#pragma unroll
-      for (int kc = 0; kc < C_KCH; ++kc) {
-        asm volatile("" : "+a"(wreg[0][cc][kc]));
-        asm volatile("" : "+a"(wreg[1][cc][kc]));
-      }
+    for (int kc = 0; kc < C_KCH; ++kc) {
+      asm volatile("" : "+a"(wreg[0][kc]));
+      asm volatile("" : "+a"(wreg[1][kc]));
+    }
   }
 
   const float oma = 1.f - p.alpha;
   const ActScale asc = act_scale_make(p.alpha);
-  const int lane_c = (lane & 48) | (4 * v + g4), c0 = 2 * j4;
   const size_t xhalf_bytes = (size_t)2 * c.npairs * C_TILE_UNITS * 16;
-  char* const bin = xchg + 2 * xhalf_bytes;   // where stores go that have nothing to store (C_BIN_BYTES)
-  // lane-constant byte offsets (what varies with step and tile is wave-uniform and goes into the scalar base)
-  const unsigned row_lane = (unsigned)(((4 * q + j4) * N + 128 * m + 32 * v + 8 * g4) * 4);   // fp32 [16 rows][N]: row 4q+j4, eight neurons
-  const unsigned xq_lane = (unsigned)(((((4 * m + v) * 4 + g4) * 16) + 4 * q + j4) * 16);     // exchange unit (own K chunk, g4, row 4q+j4)
-  const unsigned d_lane = (unsigned)(lane_c * 64 + 8 * c0);
-  const unsigned r_lane = (unsigned)((c0 * 64 + lane_c) * 16);
-  const unsigned x_lane = (unsigned)(lane * 16), x_lane_hi = x_lane + 4096;
+  char* const bin = xchg + 2 * xhalf_bytes;
+  // lane-constant byte offsets
+  const unsigned row_lane = (unsigned)(((4 * q + j4) * N + 128 * m + 16 * ct + 4 * g4) * 4);   // fp32 [16 rows][N]: row 4q+j4, four neurons
+  const unsigned xq_lane = (unsigned)(((((4 * m + (ct >> 1)) * 4 + 2 * (ct & 1) + (g4 >> 1)) * 16) + 4 * q + j4) * 16 + 8 * (g4 & 1));
+  const int lane_c = (lane & 48) | (2 * ct + (n >> 3)), cp = n & 7;   // the neuron's place in the common tile order
+  const unsigned d_lane = (unsigned)(lane_c * 64 + 8 * cp);
+  const unsigned r_lane = (unsigned)((cp * 64 + lane_c) * 16);
+  const unsigned x_lane = (unsigned)(lane * 16);
   const unsigned g_lane = (unsigned)(((lane >> 1) * T * 2 + (lane & 1)) * 4);
-  const unsigned f_lane = (unsigned)(n * 4);
-
-  // deferred stores of the last finished pair-step
-  f32x4 dh[2][2], dd16[2], dx[2];
-  f32x2 dr[2][2];
-  {
-    const f32x4 z = {0.f, 0.f, 0.f, 0.f};
-    dh[0][0] = dh[0][1] = dh[1][0] = dh[1][1] = dd16[0] = dd16[1] = dx[0] = dx[1] = z;
-    dr[0][0] = dr[0][1] = dr[1][0] = dr[1][1] = f32x2{0.f, 0.f};
-  }
-  bool dreal = false, dmore = false;
-  int dt = 0, dpr = 0, dpl = 0;
+  const unsigned f_lane = (unsigned)((lane & 31) * 4);
 
   auto hist_base = [&](int t, int bt) { return reinterpret_cast<const char*>(p.hist) + ((size_t)t * B + 16 * bt) * N * 4; };
-  auto emit = [&](auto iv) {
-    constexpr int i = decltype(iv)::value;
-    if constexpr (i < 2) {
-      const char* base = xchg + (size_t)((dt + 1) & 1) * xhalf_bytes + (size_t)(2 * dpr + i) * C_TILE_UNITS * 16;
-      sstore16<0>(dreal ? base : bin, xq_lane, dx[i]);
-    } else if constexpr (i < 6) {
-      constexpr int tl = (i - 2) >> 1, hf = (i - 2) & 1;
-      const char* base = hist_base(dt, 2 * dpr + tl);
-#ifdef CL_KNOCK_BIN
-      sstore16<16 * hf>(bin, row_lane, dh[tl][hf]);
-#else
-      sstore16<16 * hf>(dreal ? base : bin, row_lane, dh[tl][hf]);
-#endif
-    } else if constexpr (i < 8) {
-      if constexpr (SAVE) {
-        constexpr int tl = i - 6;
-        const char* base = reinterpret_cast<const char*>(p.dfrag) + ((((size_t)dt * nbt + 2 * dpr + tl) * 4 + m) * 64) * 64;
-#ifdef CL_KNOCK_BIN
-        sstore16<0>(bin, d_lane, dd16[tl]);
-#else
-        sstore16<0>(dreal ? base : bin, d_lane, dd16[tl]);
-#endif
-      }
-    } else {
-      if constexpr (SAVE) {
-        constexpr int tl = (i - 8) >> 1, cc = (i - 8) & 1;
-        // slot t+1 of the operand copy; past the last step there is none (an odd length's is the zero tail)
-        const char* base = reinterpret_cast<const char*>(p.rfrag) +
-                           (((size_t)((dt + 1) >> 1) * nbt + 2 * dpr + tl) * 32 + 8 * m) * 64 * 16 + ((dt + 1) & 1) * 8;
-        const bool there = dreal && (dmore || (T & 1));
-#ifdef CL_KNOCK_BIN
-        sstore8<1024 * cc>(there ? bin : bin, r_lane, dmore ? dr[tl][cc] : f32x2{0.f, 0.f});
-#else
-        sstore8<1024 * cc>(there ? base : bin, r_lane, dmore ? dr[tl][cc] : f32x2{0.f, 0.f});
-#endif
-      }
-    }
-  };
-  auto emit_all = [&]() {
-    emit(std::integral_constant<int, 0>{});
-    emit(std::integral_constant<int, 1>{});
-    emit(std::integral_constant<int, 2>{});
-    emit(std::integral_constant<int, 3>{});
-    emit(std::integral_constant<int, 4>{});
-    emit(std::integral_constant<int, 5>{});
-    emit(std::integral_constant<int, 6>{});
-    emit(std::integral_constant<int, 7>{});
-    emit(std::integral_constant<int, 8>{});
-    emit(std::integral_constant<int, 9>{});
-    emit(std::integral_constant<int, 10>{});
-    emit(std::integral_constant<int, 11>{});
-  };
-  auto flag_base = [&](int pl) { return reinterpret_cast<const char*>(c.flags) + ((size_t)cl * c.ppc + pl) * 16 * 4; };
+  auto flag_base = [&](int pl) { return reinterpret_cast<const char*>(c.flags) + ((size_t)cl * c.ppc + pl) * 32 * 4; };
   auto x_base = [&](int t, int pr) {
-    return xchg + (size_t)(t & 1) * xhalf_bytes + ((size_t)(2 * pr) * C_TILE_UNITS + vu * 512) * 16;
+    return xchg + (size_t)(t & 1) * xhalf_bytes + ((size_t)(2 * pr) * C_TILE_UNITS + w8u * 256) * 16;
   };
   auto gate_base = [&](int t, int pr) { return reinterpret_cast<const char*>(p.A) + ((size_t)(32 * pr) * T + t) * 8; };
   auto stage_from_r_init = [&](int pr) {
 #pragma unroll
-    for (int jj = 0; jj < 8; ++jj) {
-      const int u = v * 512 + jj * 64 + lane;
+    for (int jj = 0; jj < 4; ++jj) {
+      const int u = w8 * 256 + jj * 64 + lane;
       const int tl = u >> 10, kc = (u >> 6) & 15, qq = (u >> 4) & 3, row = u & 15;
       const f32x4* src = reinterpret_cast<const f32x4*>(p.r_init + (size_t)(32 * pr + 16 * tl + row) * N + 32 * kc + 8 * qq);
       const f32x4 lo = src[0], hi = src[1];
@@ -721,14 +244,106 @@ __global__ __launch_bounds__(256) void ring_fwd_cluster_full_kernel(RingFwdArgs 
     }
   };
 
+  int pf_pl = -1, pf_val = 0;   // exchange stores issued, flag not yet up: pair (local) and state number
+  f32x4 P[2][3];           // products of the pair-step in hand: [tile][matrix]
+  f32x4 Lr[2];             // previous state of its rows (row 4q+j4, four neurons), per tile
+  // the pair-step whose products are in P and whose epilogue is still to run (skewed half)
+  int et = 0, epr = 0, epl = 0, eit = 0;
+  bool epending = false;
+
+  // Epilogue of pair-step (t, pr, pl), number `it` in this cluster's order, in two parts: the arithmetic on P and Lr
+  // (its products and previous state) leaves everything in the form it is stored in; the stores follow.
+  struct EpiOut {
+    unsigned xe[2][2];
+    f32x4 hv[2];
+    f32x2 dk[2], rk[2], r0k[2];
+  };
+  auto epi_math = [&](int it, const f32x4 (&Lp)[2], EpiOut& o) {
+    const float* gb = gl + (it & 1) * 64;
+#pragma unroll
+    for (int tl = 0; tl < 2; ++tl) {
+      unsigned ro[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float e0 = Lp[tl][i];
+        ro[i] = __builtin_bit_cast(unsigned, e0);
+      }
+      quad_transpose(ro, j4);   // -> rows 4q+e of the lane's own neuron
+      const f32x4 ga = *reinterpret_cast<const f32x4*>(gb + (16 * tl + 4 * q) * 2);
+      const f32x4 gc = *reinterpret_cast<const f32x4*>(gb + (16 * tl + 4 * q + 2) * 2);
+      float rn[4], dv[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const float g0 = e < 2 ? ga[2 * e] : gc[2 * (e - 2)], g1 = e < 2 ? ga[2 * e + 1] : gc[2 * (e - 2) + 1];
+        const float p0 = P[tl][0][e], p1 = P[tl][1][e], p2 = P[tl][2][e];
+        const float x = fmaf(g1, p2, fmaf(g0, p1, p0));
+        float aF, aD;
+        act_scaled<ACT>(x, asc, aF, aD);
+        rn[e] = fmaf(oma, __builtin_bit_cast(float, ro[e]), aF);
+        dv[e] = aD;
+      }
+      if constexpr (SAVE) {
+        const f16x4 d4 = {(_Float16)dv[0], (_Float16)dv[1], (_Float16)dv[2], (_Float16)dv[3]};
+        o.dk[tl] = __builtin_bit_cast(f32x2, d4);
+        const bf16x4 r4 = {(__bf16)rn[0], (__bf16)rn[1], (__bf16)rn[2], (__bf16)rn[3]};
+        o.rk[tl] = __builtin_bit_cast(f32x2, r4);
+        const bf16x4 o4 = {(__bf16)__builtin_bit_cast(float, ro[0]), (__bf16)__builtin_bit_cast(float, ro[1]),
+                           (__bf16)__builtin_bit_cast(float, ro[2]), (__bf16)__builtin_bit_cast(float, ro[3])};
+        o.r0k[tl] = __builtin_bit_cast(f32x2, o4);
+      }
+      unsigned hh[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) hh[e] = __builtin_bit_cast(unsigned, rn[e]);
+      quad_transpose(hh, j4);   // -> row 4q+j4, neurons 4 g4 + i
+      o.hv[tl] = f32x4{__builtin_bit_cast(float, hh[0]), __builtin_bit_cast(float, hh[1]), __builtin_bit_cast(float, hh[2]),
+                     __builtin_bit_cast(float, hh[3])};
+      const float h0 = o.hv[tl][0], h1 = o.hv[tl][1], h2 = o.hv[tl][2], h3 = o.hv[tl][3];
+      const bf16x2 b01 = {(__bf16)h0, (__bf16)h1}, b23 = {(__bf16)h2, (__bf16)h3};
+      o.xe[tl][0] = __builtin_bit_cast(unsigned, b01);
+      o.xe[tl][1] = __builtin_bit_cast(unsigned, b23);
+    }
+  };
+  auto epi_stores = [&](int t, int pr, int pl, const EpiOut& o) {
+    const bool more = t + 1 < T;
+    // the exchange first: its flag goes up as soon as the two stores have landed
+    {
+      const char* xb = xchg + (size_t)((t + 1) & 1) * xhalf_bytes + (size_t)(2 * pr) * C_TILE_UNITS * 16;
+      const f32x2 x0 = {__builtin_bit_cast(float, o.xe[0][0]), __builtin_bit_cast(float, o.xe[0][1])};
+      const f32x2 x1 = {__builtin_bit_cast(float, o.xe[1][0]), __builtin_bit_cast(float, o.xe[1][1])};
+      sstore8<0>(more ? xb : bin, xq_lane, x0);
+      sstore8<0>(more ? xb + C_TILE_UNITS * 16 : bin, xq_lane, x1);
+    }
+    sstore16<0>(hist_base(t, 2 * pr), row_lane, o.hv[0]);
+    sstore16<0>(hist_base(t, 2 * pr + 1), row_lane, o.hv[1]);
+    if constexpr (SAVE) {
+      const char* db = reinterpret_cast<const char*>(p.dfrag) + ((((size_t)t * nbt + 2 * pr) * 4 + m) * 64) * 64;
+      sstore8<0>(db, d_lane, o.dk[0]);
+      sstore8<0>(db + 4 * 64 * 64, d_lane, o.dk[1]);
+      // The operand copy keeps steps 2j and 2j+1 side by side in one 16-byte slot per lane.  An even step has both
+      // halves at hand -- the state before it (slot t) and after it (slot t+1; past an odd length's end: the zero
+      // tail) -- and stores the slot whole; an odd step stores nothing.  (Eight bytes at a time would be partial
+      // 32-byte sectors, which cost a store five times what a whole one costs.)
+      if ((t & 1) == 0) {
+        const char* rb = reinterpret_cast<const char*>(p.rfrag) + (((size_t)(t >> 1) * nbt + 2 * pr) * 32 + 8 * m) * 64 * 16;
+        const f32x2 z = {0.f, 0.f};
+        const f32x2 n0 = more ? o.rk[0] : z, n1 = more ? o.rk[1] : z;
+        sstore16<0>(rb, r_lane, f32x4{o.r0k[0][0], o.r0k[0][1], n0[0], n0[1]});
+        sstore16<0>(rb + 32 * 64 * 16, r_lane, f32x4{o.r0k[1][0], o.r0k[1][1], n1[0], n1[1]});
+      }
+    }
+    // the flag of these two exchange stores goes up behind this wave's next full wait (fetch_decide, or the slow
+    // path of the staging): by then they have long landed, and nothing stands still for their acknowledgement
+    pf_pl = more ? pl : -1;
+    pf_val = t + 1;
+  };
+
   // the first pair-step's operand and gates
   stage_from_r_init(cl);
-  if (v == 0) gl[lane] = *reinterpret_cast<const float*>(gate_base(0, cl) + g_lane);
+  if (w8 == 0) gl[lane] = *reinterpret_cast<const float*>(gate_base(0, cl) + g_lane);
   lds_barrier();
   if (misc[0]) return;
 
-  int t = 0, pl = 0;
-  CL2_DECL();
+  int t = 0, pl = 0, it = 0;
   for (;;) {
     const int pr = cl + c.nclusters * pl;
     int nt = t, npl = pl + 1;
@@ -740,203 +355,141 @@ __global__ __launch_bounds__(256) void ring_fwd_cluster_full_kernel(RingFwdArgs 
     const bool look = have_next && nt >= 1;
     const int npr = cl + c.nclusters * npl;
 
-    f32x4 P[2][2][3];
-    {
-      const f32x4 z = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int tl = 0; tl < 2; ++tl)
-#pragma unroll
-        for (int cc = 0; cc < 2; ++cc) P[tl][cc][0] = P[tl][cc][1] = P[tl][cc][2] = z;
-    }
-    f32x4 L[2][2];      // previous state: eight neurons of the lane's row 4q+j4, per tile
-    f32x4 sreg[8];      // this wave's quarter of the next pair-step's operand
+    f32x4 sreg[4];      // this wave's eighth of the next pair-step's operand
     int nflag;
     float gnext;
     bool up = false;
-    // what goes out between the MFMA groups of K chunk kc
-    auto slot = [&](auto kcv) {
-      constexpr int kc = decltype(kcv)::value;
-      if constexpr (kc == 0) {
-        const char* pb = t == 0 ? reinterpret_cast<const char*>(p.r_init) + (size_t)(32 * pr) * N * 4 : hist_base(t - 1, 2 * pr);
-        L[0][0] = sload16<0>(pb, row_lane);
-        L[0][1] = sload16<16>(pb, row_lane);
-        L[1][0] = sload16<0>(pb + 16 * N * 4, row_lane);
-        L[1][1] = sload16<16>(pb + 16 * N * 4, row_lane);
-        gnext = sload4(have_next ? gate_base(nt, npr) : gate_base(t, pr), g_lane);
-        nflag = sload4_dev(flag_base(look ? npl : pl), f_lane);
-      } else if constexpr (kc >= 1 && kc <= 6) {
-        emit(std::integral_constant<int, 2 * (kc - 1)>{});
-        emit(std::integral_constant<int, 2 * (kc - 1) + 1>{});
-      } else if constexpr (kc == 8) {
-        vm_wait_in<NST>(L, nflag, gnext);
-        up = look && __ballot(nflag < nt) == 0;
-      }
-      if constexpr (kc >= 8 && kc <= 11) {
-        const char* xb = look ? x_base(nt, npr) : x_base(t, pr);
-        constexpr int jj = 2 * (kc - 8);
-        sreg[jj] = sload16_dev<1024 * (jj & 3)>(xb, jj < 4 ? x_lane : x_lane_hi);
-        sreg[jj + 1] = sload16_dev<1024 * ((jj + 1) & 3)>(xb, jj < 4 ? x_lane : x_lane_hi);
-      }
+    auto fetch_issue = [&]() {
+      gnext = sload4(have_next ? gate_base(nt, npr) : gate_base(t, pr), g_lane);
+      nflag = sload4_dev(flag_base(look ? npl : pl), f_lane);
     };
-    bf16x8 af[2][2], wf[2][2];
+    auto fetch_decide = [&]() {
+      asm volatile("s_waitcnt vmcnt(0)" : "+v"(nflag), "+v"(gnext)::"memory");
+      up = look && __ballot(nflag < nt) == 0;
+      sstore4_dev(pf_pl >= 0 ? flag_base(pf_pl) : bin, (unsigned)((8 * m + w8u) * 4), pf_val);   // (every lane the same word)
+      pf_pl = -1;
+    };
+    auto fetch_x = [&](auto iv) {
+      constexpr int i = decltype(iv)::value;
+      const char* xb = look ? x_base(nt, npr) : x_base(t, pr);
+      sreg[i] = sload16_dev<1024 * i>(xb, x_lane);
+    };
+
+    const bool thin = skew && !epending;   // no epilogue (and none of its stores) behind this pair-step's fetches
+    if (skew) {
+      // the late half: the previous pair-step's epilogue comes first, and the fetches for the next pair-step go out
+      // around it (its products follow at once, and the operand must have landed when they end)
+      EpiOut o = {};
+      fetch_issue();
+      if (epending) epi_math(eit, Lr, o);
+      fetch_decide();
+      fetch_x(std::integral_constant<int, 0>{});
+      fetch_x(std::integral_constant<int, 1>{});
+      fetch_x(std::integral_constant<int, 2>{});
+      fetch_x(std::integral_constant<int, 3>{});
+      if (epending) epi_stores(et, epr, epl, o);
+    }
+
+    // ---- products ----
+    {
+      const f32x4 z = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int tl = 0; tl < 2; ++tl) P[tl][0] = P[tl][1] = P[tl][2] = z;
+    }
+    // previous state of this pair-step's rows
+    const char* const pb = t == 0 ? reinterpret_cast<const char*>(p.r_init) + (size_t)(32 * pr) * N * 4 : hist_base(t - 1, 2 * pr);
+    bf16x8 af[2][2], wf[2];
     auto frag_fetch = [&](auto kcv, int stg) {
       constexpr int kc = decltype(kcv)::value;
       af[stg][0] = xs[(0 * C_KCH + kc) * 64 + lane];
       af[stg][1] = xs[(1 * C_KCH + kc) * 64 + lane];
-      wf[stg][0] = wl[(0 * C_KCH + kc) * 64];
-      if constexpr (C_KCH + kc < C_WFR) wf[stg][1] = wl[(1 * C_KCH + kc) * 64];
-      else wf[stg][1] = wo_last;
+      if constexpr (kc < C8_WFR) wf[stg] = wl[kc * 64];
+      else wf[stg] = wo_last;
     };
-    auto body = [&](auto kcv) {
+    auto body = [&](auto kcv, auto slotsv) {
       constexpr int kc = decltype(kcv)::value, stg = kc & 1;
       if constexpr (kc + 1 < C_KCH) frag_fetch(std::integral_constant<int, kc + 1>{}, stg ^ 1);
       __builtin_amdgcn_sched_barrier(0);
-      slot(kcv);
-      __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-      for (int cc = 0; cc < 2; ++cc) {
-        P[0][cc][1] = mfma16(af[stg][0], wreg[0][cc][kc], P[0][cc][1]);
-        P[1][cc][1] = mfma16(af[stg][1], wreg[0][cc][kc], P[1][cc][1]);
-        P[0][cc][2] = mfma16(af[stg][0], wreg[1][cc][kc], P[0][cc][2]);
-        P[1][cc][2] = mfma16(af[stg][1], wreg[1][cc][kc], P[1][cc][2]);
-        P[0][cc][0] = mfma16(af[stg][0], wf[stg][cc], P[0][cc][0]);
-        P[1][cc][0] = mfma16(af[stg][1], wf[stg][cc], P[1][cc][0]);
+      if constexpr (decltype(slotsv)::value) {
+        if constexpr (kc == 0) fetch_issue();
+        if constexpr (kc == 12) fetch_decide();
+        if constexpr (kc >= 12) fetch_x(std::integral_constant<int, kc - 12>{});
+        __builtin_amdgcn_sched_barrier(0);
       }
+      P[0][1] = mfma16(af[stg][0], wreg[0][kc], P[0][1]);
+      P[1][1] = mfma16(af[stg][1], wreg[0][kc], P[1][1]);
+      P[0][2] = mfma16(af[stg][0], wreg[1][kc], P[0][2]);
+      P[1][2] = mfma16(af[stg][1], wreg[1][kc], P[1][2]);
+      P[0][0] = mfma16(af[stg][0], wf[stg], P[0][0]);
+      P[1][0] = mfma16(af[stg][1], wf[stg], P[1][0]);
       __builtin_amdgcn_sched_barrier(0);
     };
-    CL2_STAMP(0);
-    frag_fetch(std::integral_constant<int, 0>{}, 0);
-    __builtin_amdgcn_s_setprio(1);
-    body(std::integral_constant<int, 0>{});
-    body(std::integral_constant<int, 1>{});
-    body(std::integral_constant<int, 2>{});
-    body(std::integral_constant<int, 3>{});
-    body(std::integral_constant<int, 4>{});
-    body(std::integral_constant<int, 5>{});
-    body(std::integral_constant<int, 6>{});
-    body(std::integral_constant<int, 7>{});
-    CL2_STAMP(1);
-    body(std::integral_constant<int, 8>{});
-    CL2_STAMP(2);
-    body(std::integral_constant<int, 9>{});
-    body(std::integral_constant<int, 10>{});
-    body(std::integral_constant<int, 11>{});
-    body(std::integral_constant<int, 12>{});
-    body(std::integral_constant<int, 13>{});
-    body(std::integral_constant<int, 14>{});
-    body(std::integral_constant<int, 15>{});
-    __builtin_amdgcn_s_setprio(0);
-    CL2_STAMP(3);
-    // the exchange stores of the previous pair-step went out in slot 1: once they have landed, publish them
-    vm_wait_plain<NST - 2 + 8>();
-    sstore4_dev((dreal && dmore) ? flag_base(dpl) : bin, (unsigned)((4 * m + vu) * 4), dt + 1);   // (every lane the same word)
-
-    CL2_STAMP(4);
-    // ---- epilogue ----
-    const bool more = t + 1 < T;
-#pragma unroll
-    for (int tl = 0; tl < 2; ++tl) {
-      // previous state: the lane loaded eight neurons of row 4q+j4; the quad turns that into rows 4q+e of its own two
-      unsigned pl0[4], pl1[4];
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        // (through named floats: a bit cast applied directly to a vector element reads the wrong lanes)
-        const float e0 = L[tl][i >> 1][(i & 1) * 2 + 0], e1 = L[tl][i >> 1][(i & 1) * 2 + 1];
-        pl0[i] = __builtin_bit_cast(unsigned, e0);
-        pl1[i] = __builtin_bit_cast(unsigned, e1);
-      }
-      quad_transpose(pl0, j4);
-      quad_transpose(pl1, j4);
-      float rn[4][2], dv[4][2];
-      const f32x4 ga = *reinterpret_cast<const f32x4*>(gl + (16 * tl + 4 * q) * 2);       // rows 4q, 4q+1
-      const f32x4 gb = *reinterpret_cast<const f32x4*>(gl + (16 * tl + 4 * q + 2) * 2);   // rows 4q+2, 4q+3
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const float g0 = e < 2 ? ga[2 * e] : gb[2 * (e - 2)], g1 = e < 2 ? ga[2 * e + 1] : gb[2 * (e - 2) + 1];
-#pragma unroll
-        for (int cc = 0; cc < 2; ++cc) {
-          const float x = fmaf(g1, P[tl][cc][2][e], fmaf(g0, P[tl][cc][1][e], P[tl][cc][0][e]));
-          float aF, aD;
-          act_scaled<ACT>(x, asc, aF, aD);
-          const float ro = __builtin_bit_cast(float, cc ? pl1[e] : pl0[e]);
-          rn[e][cc] = fmaf(oma, ro, aF);
-          dv[e][cc] = aD;
-        }
-      }
-      if (SAVE && t == 0) {
-        // slot 0 of the operand copy is the initial state
-        const char* base = reinterpret_cast<const char*>(p.rfrag) + (((size_t)0 * nbt + 2 * pr + tl) * 32 + 8 * m) * 64 * 16;
-        const bf16x4 k0 = {(__bf16)__builtin_bit_cast(float, pl0[0]), (__bf16)__builtin_bit_cast(float, pl0[1]),
-                           (__bf16)__builtin_bit_cast(float, pl0[2]), (__bf16)__builtin_bit_cast(float, pl0[3])};
-        const bf16x4 k1 = {(__bf16)__builtin_bit_cast(float, pl1[0]), (__bf16)__builtin_bit_cast(float, pl1[1]),
-                           (__bf16)__builtin_bit_cast(float, pl1[2]), (__bf16)__builtin_bit_cast(float, pl1[3])};
-        sstore8<0>(base, r_lane, __builtin_bit_cast(f32x2, k0));
-        sstore8<1024>(base, r_lane, __builtin_bit_cast(f32x2, k1));
-      }
-      // hold the results back in the form they are stored in
-      {
-        unsigned h0[4], h1[4], xe[4];
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          h0[e] = __builtin_bit_cast(unsigned, rn[e][0]);
-          h1[e] = __builtin_bit_cast(unsigned, rn[e][1]);
-          const bf16x2 pk = {(__bf16)rn[e][0], (__bf16)rn[e][1]};
-          xe[e] = __builtin_bit_cast(unsigned, pk);
-        }
-        quad_transpose(h0, j4);
-        quad_transpose(h1, j4);
-        quad_transpose(xe, j4);
-        dh[tl][0] = f32x4{__builtin_bit_cast(float, h0[0]), __builtin_bit_cast(float, h1[0]), __builtin_bit_cast(float, h0[1]),
-                          __builtin_bit_cast(float, h1[1])};
-        dh[tl][1] = f32x4{__builtin_bit_cast(float, h0[2]), __builtin_bit_cast(float, h1[2]), __builtin_bit_cast(float, h0[3]),
-                          __builtin_bit_cast(float, h1[3])};
-        dx[tl] = f32x4{__builtin_bit_cast(float, xe[0]), __builtin_bit_cast(float, xe[1]), __builtin_bit_cast(float, xe[2]),
-                       __builtin_bit_cast(float, xe[3])};
-      }
-      if constexpr (SAVE) {
-        typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
-        const f16x8 dk = {(_Float16)dv[0][0], (_Float16)dv[1][0], (_Float16)dv[2][0], (_Float16)dv[3][0],
-                          (_Float16)dv[0][1], (_Float16)dv[1][1], (_Float16)dv[2][1], (_Float16)dv[3][1]};
-        dd16[tl] = __builtin_bit_cast(f32x4, dk);
-#pragma unroll
-        for (int cc = 0; cc < 2; ++cc) {
-          const bf16x4 pk = {(__bf16)rn[0][cc], (__bf16)rn[1][cc], (__bf16)rn[2][cc], (__bf16)rn[3][cc]};
-          dr[tl][cc] = __builtin_bit_cast(f32x2, pk);
-        }
-      }
-      __builtin_amdgcn_sched_barrier(0);
+    auto products = [&](auto slotsv) {
+      frag_fetch(std::integral_constant<int, 0>{}, 0);
+      __builtin_amdgcn_s_setprio(C8_PRIO);
+      body(std::integral_constant<int, 0>{}, slotsv);
+      body(std::integral_constant<int, 1>{}, slotsv);
+      body(std::integral_constant<int, 2>{}, slotsv);
+      body(std::integral_constant<int, 3>{}, slotsv);
+      body(std::integral_constant<int, 4>{}, slotsv);
+      body(std::integral_constant<int, 5>{}, slotsv);
+      body(std::integral_constant<int, 6>{}, slotsv);
+      body(std::integral_constant<int, 7>{}, slotsv);
+      body(std::integral_constant<int, 8>{}, slotsv);
+      body(std::integral_constant<int, 9>{}, slotsv);
+      body(std::integral_constant<int, 10>{}, slotsv);
+      body(std::integral_constant<int, 11>{}, slotsv);
+      body(std::integral_constant<int, 12>{}, slotsv);
+      body(std::integral_constant<int, 13>{}, slotsv);
+      body(std::integral_constant<int, 14>{}, slotsv);
+      body(std::integral_constant<int, 15>{}, slotsv);
+      __builtin_amdgcn_s_setprio(0);
+    };
+    if (skew) {
+      // (ordinary loads: they are read in the next pair-step's first phase, and the compiler waits for them there)
+      Lr[0] = *reinterpret_cast<const f32x4*>(pb + row_lane);
+      Lr[1] = *reinterpret_cast<const f32x4*>(pb + 16 * N * 4 + row_lane);
+      products(std::false_type{});
+      et = t;
+      epr = pr;
+      epl = pl;
+      eit = it;
+      epending = true;
+    } else {
+      // the early half reads them right behind its products: seven operations younger (gates, flags, the flag
+      // store, four operand loads) are still allowed to be out when it does
+      f32x4 La[2];
+      La[0] = sload16<0>(pb, row_lane);
+      La[1] = sload16<0>(pb + 16 * N * 4, row_lane);
+      products(std::true_type{});
+      asm volatile("s_waitcnt vmcnt(7)" : "+v"(La[0]), "+v"(La[1])::"memory");
+      EpiOut o;
+      epi_math(it, La, o);
+      epi_stores(t, pr, pl, o);
     }
-    dreal = true;
-    dmore = more;
-    dt = t;
-    dpr = pr;
-    dpl = pl;
 
-    CL2_STAMP(5);
     // ---- the next pair-step's operand and gates into LDS ----
-    lds_barrier();
-    CL2_STAMP(6);   // every wave has finished with the operand and the gates of this pair-step
-    // Whatever the slots fetched has landed after this wait, wanted or not.  (One wait, in straight-line code: a wait
-    // inside the branches below would have the compiler copy the registers into place in front of it, in flight.)
-    vm_wait_x<1>(sreg);
-    CL2_STAMP(7);
+    lds_barrier();   // every wave has finished with this pair-step's operand (and the late half with the gates before it)
+    // the four operand loads are older than the epilogue's stores, which every wave has issued since; the late
+    // half's first pair-step has no epilogue in front of it, and a plain vmcnt(0) covers that one time
+    if (thin) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NSTE) : "memory");
     if (!have_next) break;
     if (nt == 0) {
       stage_from_r_init(npr);
     } else {
       if (up) {
 #pragma unroll
-        for (int jj = 0; jj < 8; ++jj) xs[v * 512 + jj * 64 + lane] = __builtin_bit_cast(bf16x8, sreg[jj]);
+        for (int jj = 0; jj < 4; ++jj) xs[w8 * 256 + jj * 64 + lane] = __builtin_bit_cast(bf16x8, sreg[jj]);
       } else {
-        // nothing valid was fetched ahead (the producers of this operand were not done when slot 8 looked, or
-        // this is the cluster's only pair): publish what is still held back, then wait for the flags
-        emit_all();
+        // nothing valid was fetched ahead: put up the flag still held back (the producers of what is waited for may
+        // be waiting for it in turn), wait for the flags, then ordinary loads behind a device-scope acquire
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        if (dmore) sstore4_dev(flag_base(dpl), (unsigned)((4 * m + vu) * 4), dt + 1);
-        dreal = false;
+        if (pf_pl >= 0) sstore4_dev(flag_base(pf_pl), (unsigned)((8 * m + w8u) * 4), pf_val);
+        pf_pl = -1;
         bool ok = false;
         for (int spins = 0; spins <= c.spin_max; ++spins) {
-          const int f = flag_load(c.flags + ((size_t)cl * c.ppc + npl) * 16 + n);
+          const int f = flag_load(c.flags + ((size_t)cl * c.ppc + npl) * 32 + (lane & 31));
           if ((ok = (__ballot(f < nt) == 0))) break;
           __builtin_amdgcn_s_sleep(2);
         }
@@ -944,23 +497,24 @@ __global__ __launch_bounds__(256) void ring_fwd_cluster_full_kernel(RingFwdArgs 
           misc[0] = 1;
           *c.host_err = RING_CLUSTER_ERR_WAIT;
         }
-        // ordinary loads behind a device-scope acquire (which drops the vector L1's lines): the compiler waits for them
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
         const bf16x8* xb = reinterpret_cast<const bf16x8*>(x_base(nt, npr));
 #pragma unroll
-        for (int jj = 0; jj < 8; ++jj) xs[v * 512 + jj * 64 + lane] = xb[jj * 64 + lane];
+        for (int jj = 0; jj < 4; ++jj) xs[w8 * 256 + jj * 64 + lane] = xb[jj * 64 + lane];
       }
     }
-    if (v == 0) gl[lane] = gnext;
-    CL2_STAMP(8);
+    if (w8 == 0) gl[((it + 1) & 1) * 64 + lane] = gnext;
     lds_barrier();
-    CL2_STAMP(9);
-    CL2_FLUSH();
     if (misc[0]) return;
     t = nt;
     pl = npl;
+    ++it;
   }
-  emit_all();   // the last pair-step's results (its state is nobody's operand)
+  if (skew && epending) {
+    EpiOut o;
+    epi_math(eit, Lr, o);
+    epi_stores(et, epr, epl, o);
+  }
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -982,7 +536,7 @@ ClusterGeo cluster_geo(int nbt) {
   g.nclusters = (g.npairs + g.ppc - 1) / g.ppc;
   g.grid = 32 * ((g.nclusters + 7) / 8);
   g.xchg_bytes = c_align((size_t)2 * 2 * g.npairs * C_TILE_UNITS * 16 + C_BIN_BYTES);
-  g.flag_bytes = c_align((size_t)g.nclusters * g.ppc * 16 * sizeof(int));
+  g.flag_bytes = c_align((size_t)g.nclusters * g.ppc * 32 * sizeof(int));   // (the eight-wave kernel: 32 per pair)
   g.hello_bytes = c_align((size_t)g.nclusters * 4 * sizeof(int));
   return g;
 }
@@ -1010,7 +564,7 @@ hipError_t host_err_word(int** dev) {
 
 }  // namespace
 
-bool ring_cluster_applicable(int N, int k) { return N > 256 && N <= 512 && k == 2; }
+bool ring_cluster_applicable(int N, int k) { return N == 512 && k == 2; }
 
 size_t ring_cluster_workspace_bytes(int nbt) {
   const ClusterGeo g = cluster_geo(nbt);
@@ -1019,11 +573,27 @@ size_t ring_cluster_workspace_bytes(int nbt) {
 
 int ring_cluster_error() { return g_host_err ? *(volatile int*)g_host_err : 0; }
 
-// RINGATTR_CLUSTER=1 / 0 switches the cluster kernel on / off where it applies.
-bool ring_uses_cluster(int N, int k, int nbt) {
-  if (!ring_cluster_applicable(N, k)) return false;
+// The error word, the first time it is found set (0 afterwards): the caller reports it once; from then on the cluster
+// kernel stays switched off (ring_uses_cluster) and the streaming kernels do the work.
+int ring_cluster_take_error() {
+  static bool reported = false;
+  const int e = ring_cluster_error();
+  if (e == 0 || reported) return 0;
+  reported = true;
+  return e;
+}
+
+// Where the cluster kernel runs.  It wins where every cluster has at least four batch-tile pairs to rotate through
+// (B >= 6176 or so: 17 to 25 % at B = 8192 and 16384); with fewer, a pair-step waits for the state its siblings are
+// still computing and the streaming kernels are several times faster.  RINGATTR_CLUSTER=0 switches it off, =1 on
+// wherever the shape allows (tests of the short rotations).  Unasked, it also wants the device it was measured on
+// (256 compute units in 8 XCDs); the placement check in the kernel is what it relies on elsewhere.
+bool ring_uses_cluster(int N, int k, int B, int T) {
+  if (!ring_cluster_applicable(N, k) || B % 32 != 0 || T > (1 << 20)) return false;   // whole pairs of batch tiles
+  const int nbt = B / 16;
   const char* v = getenv("RINGATTR_CLUSTER");
-  if (!(v && v[0] == '1')) return false;
+  if (v && v[0] == '0') return false;
+  const bool forced = v && v[0] == '1';
   if (ring_cluster_error()) return false;
   static int cus = 0;
   if (cus == 0) {
@@ -1032,28 +602,27 @@ bool ring_uses_cluster(int N, int k, int nbt) {
         hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = -1;
     cus = n;
   }
-  return cluster_geo(nbt).grid <= cus;   // every workgroup needs a compute unit of its own, all at once
+  const ClusterGeo g = cluster_geo(nbt);
+  if (g.grid > cus) return false;   // every workgroup needs a compute unit of its own, all at once
+  return forced || (cus == 256 && g.ppc >= 4 && T >= 16);
 }
+
+int ring_cluster_pack_order(int, int, int) { return 3; }
 
 template <int ACT>
 static hipError_t launch_fwd_cluster_act(const RingFwdArgs& a, const RingClusterArgs& c, int grid, hipStream_t st) {
-  const bool full = a.N == 512 && a.B % 32 == 0;
   auto go = [&](auto kern) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       (int)C_LDS_BYTES);
+                                       (int)C8_LDS_BYTES);
     if (e != hipSuccess) return e;
-    RING_LAUNCH(kern, dim3(grid), dim3(256), C_LDS_BYTES, st, a, c);
+    RING_LAUNCH(kern, dim3(grid), dim3(512), C8_LDS_BYTES, st, a, c);
     return hipGetLastError();
   };
-  static const bool burst = [] { const char* v = getenv("RINGATTR_CLUSTER_BURST"); return v && v[0] == '1'; }();
-  if (full && !burst && a.T <= (1 << 20))
-    return a.dfrag ? go(ring_fwd_cluster_full_kernel<ACT, true>) : go(ring_fwd_cluster_full_kernel<ACT, false>);
-  if (a.dfrag) return full ? go(ring_fwd_cluster_kernel<ACT, true, true>) : go(ring_fwd_cluster_kernel<ACT, true, false>);
-  return full ? go(ring_fwd_cluster_kernel<ACT, false, true>) : go(ring_fwd_cluster_kernel<ACT, false, false>);
+  return a.dfrag ? go(ring_fwd_cluster8_kernel<ACT, true>) : go(ring_fwd_cluster8_kernel<ACT, false>);
 }
 
 hipError_t ring_launch_fwd_cluster(const RingFwdArgs& a, hipStream_t st) {
-  if (!a.cluster_ws || !ring_cluster_applicable(a.N, a.k) || !a.hist) return hipErrorInvalidValue;
+  if (!a.cluster_ws || !ring_cluster_applicable(a.N, a.k) || a.B % 32 != 0 || !a.hist) return hipErrorInvalidValue;
   const ClusterGeo g = cluster_geo(a.nbt);
   RingClusterArgs c;
   char* ws = static_cast<char*>(a.cluster_ws);
@@ -1068,7 +637,7 @@ hipError_t ring_launch_fwd_cluster(const RingFwdArgs& a, hipStream_t st) {
   c.spin_max = 4000000;
   if (const char* v = getenv("RINGATTR_CLUSTER_SPIN")) {
     const long s = atol(v);
-    if (s >= 0 && s <= 100000000L) c.spin_max = (int)s;
+    if (s >= -1 && s <= 100000000L) c.spin_max = (int)s;
   }
   const int nclear = (int)((g.flag_bytes + g.hello_bytes) / sizeof(int));
   hipLaunchKernelGGL(ring_cluster_clear_kernel, dim3((nclear + 255) / 256), dim3(256), 0, st, c.flags, nclear);

@@ -19,7 +19,9 @@
 //   split_k = 1 (NC = 4 only): contraction position kappa stands for neuron split_k_neuron(kappa) and output
 //   column n of tile c for neuron 64*w + 32*(c/2) + 2*n + c%2: the pipelined weight-resident forward's order.
 //   split_k = 2 (NC = 8 only): the same column order (neuron 128*w + 32*(c/2) + 2*n + c%2) with the contraction in
-//   neuron order: the cluster forward's.
+//   neuron order: the cluster forward's (four waves).
+//   split_k = 3 (NC = 8 only): tile c of wave group w holds the 16 consecutive neurons 128*w + 16*c + n, contraction
+//   in neuron order: the eight-wave cluster forward's.
 // ------------------------------------------------------------------------------------------------
 __device__ __forceinline__ bf16x8 pack_fragment(const float* __restrict__ Wo, const float* __restrict__ Wa, size_t u,
                                                 int N, int NC, int transposed, int split_k, float scale0, float shift0) {
@@ -34,7 +36,8 @@ __device__ __forceinline__ bf16x8 pack_fragment(const float* __restrict__ Wo, co
   const int mm = (int)(v >> 2);
   const int q = lane >> 4, n = lane & 15;
   // split_k: the output columns follow the pipelined forward's ownership as well (tile c = 2*h + cc of wave w)
-  const int col = split_k ? 16 * NC * w + 32 * (c >> 1) + 2 * n + (c & 1) : 16 * NC * w + NC * n + c;
+  const int col = split_k == 3 ? 16 * NC * w + 16 * c + n
+                               : (split_k ? 16 * NC * w + 32 * (c >> 1) + 2 * n + (c & 1) : 16 * NC * w + NC * n + c);
   const int k0 = 32 * kc + 8 * q;
   const float* W = (mm == 0) ? Wo : Wa + (size_t)(mm - 1) * N * N;
   bf16x8 pk;
@@ -1143,7 +1146,7 @@ hipError_t ring_profile_collect(double* ms, long long* launches) {
 hipError_t ring_launch_pack2(const float* Wo, const float* Wa, int N, int k, int NC, void* out, int transposed,
                              int split_k, float scale0, float shift0, void* out2, int transposed2, int split_k2,
                              float scale2, float shift2, hipStream_t st) {
-  auto order_ok = [&](int sk) { return sk == 0 || (sk == 1 && NC == 4) || (sk == 2 && NC == 8); };
+  auto order_ok = [&](int sk) { return sk == 0 || (sk == 1 && NC == 4) || ((sk == 2 || sk == 3) && NC == 8); };
   if (!order_ok(split_k) || (out2 && !order_ok(split_k2))) return hipErrorInvalidValue;
   const size_t total = (size_t)(1 + k) * 4 * NC * 2 * NC * 64 * (out2 ? 2 : 1);
   const int blocks = (int)((total + 255) / 256 < 4096 ? (total + 255) / 256 : 4096);
@@ -1252,6 +1255,7 @@ hipError_t ring_launch_fwd(const RingFwdArgs& a, int NCv, hipStream_t st) {
   ProfScope prof(1, st);
   if (ring_uses_step_kernels(a.N, a.k, NCv, a.nbt))
     return step_prefers_wide(NCv, a.nbt, a.k) ? ring_launch_wide_fwd(a, NCv, false, 4, st) : ring_launch_block_fwd(a, NCv, false, st);
+  if (a.cluster_ws) return ring_launch_fwd_cluster(a, st);   // (the caller's choice: ring_uses_cluster)
   // A forward that keeps nothing for a backward, on few batch tiles, with weights too large to stay on chip: the
   // persistent kernels would pull every weight byte through a handful of compute units once per step.  One launch per
   // step with the output columns split over workgroups spreads that over the device (a launch costs a few
@@ -1264,7 +1268,6 @@ hipError_t ring_launch_fwd(const RingFwdArgs& a, int NCv, hipStream_t st) {
     }
   }
   if (ring_uses_resident(a.N, a.k)) return ring_launch_fwd_res256(a, st);
-  if (a.cluster_ws) return ring_launch_fwd_cluster(a, st);
   const int rt = stream_row_tiles(NCv, a.nbt, false);
   hipError_t e = hipErrorInvalidValue;
   if (weights_fit_lds(NCv, a.k, 8 * 1024)) {

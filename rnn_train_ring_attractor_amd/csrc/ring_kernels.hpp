@@ -75,10 +75,10 @@ bool ring_uses_resident(int N, int k);   // applicable and not disabled by RINGA
 hipError_t ring_launch_fwd_res256(const RingFwdArgs& a, hipStream_t st);
 hipError_t ring_launch_bptt_res256(const RingBpttArgs& a, hipStream_t st);
 
-// Weight-resident forward over clusters of four compute units for 256 < N <= 512, a_dim == 2 (ring_cluster.hip).
+// Weight-resident forward over clusters of four compute units for N == 512, a_dim == 2 (ring_cluster.hip).
 struct RingClusterArgs {
   void* xchg;        // [2][2 * npairs][16 K chunks][4][16 rows] x 16 bytes: the state in MFMA A-operand order
-  int* flags;        // [nclusters][ppc][16]: last state number published per (pair, member, wave)
+  int* flags;        // [nclusters][ppc][32]: last state number published per (pair, member, wave)
   int* hello;        // [nclusters][4]: XCC_ID + 1 of each member
   int* host_err;     // word in pinned host memory, RING_CLUSTER_ERR_* when a wait ran out
   int npairs, nclusters, ppc, spin_max;
@@ -86,8 +86,10 @@ struct RingClusterArgs {
 enum { RING_CLUSTER_ERR_XCD = 1, RING_CLUSTER_ERR_START = 2, RING_CLUSTER_ERR_WAIT = 3 };
 bool ring_cluster_applicable(int N, int k);               // the shape alone
 size_t ring_cluster_workspace_bytes(int nbt);
-bool ring_uses_cluster(int N, int k, int nbt);            // applicable, switched on, and the device has the compute units
+bool ring_uses_cluster(int N, int k, int B, int T);       // applicable, switched on, whole pairs of batch tiles, and the device has the compute units
 int ring_cluster_error();                                 // the host word: non-zero once a cluster kernel gave up waiting
+int ring_cluster_take_error();                            // the same, the first time it is found set; 0 afterwards
+int ring_cluster_pack_order(int N, int B, int T);        // the column order (ring_pack_weights_kernel's split_k) its kernel for that shape reads
 hipError_t ring_launch_fwd_cluster(const RingFwdArgs& a, hipStream_t st);
 
 // Step-per-launch kernels for 512 < N <= 2048, NC in {16, 24, 32} (ring_bign.hip).

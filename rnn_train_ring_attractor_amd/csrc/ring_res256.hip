@@ -264,11 +264,15 @@ __global__ __launch_bounds__(512) void ring_fwd_res256_kernel(RingFwdArgs p) {
         if (okf[e][1] != 0.f) dst[1] = r[e][1];
       }
     } else if (slot < 6) {
-      if (SAVE) {
-        const int cc = slot - 4;
+      // the lane's two tiles lie side by side in the record: one 16-byte store (slot 4), whole 32-byte sectors per
+      // lane pair; two 8-byte stores would each write every other 8 bytes, and a store of partial sectors costs the
+      // wave several times what a whole one costs
+      if (SAVE && slot == 4) {
+        typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
         char* base = reinterpret_cast<char*>(p.dfrag + side_offset<R_NC>(t, p.nbt, bt, wu, 0));
-        const f16x4 pk = {(_Float16)d[0][cc], (_Float16)d[1][cc], (_Float16)d[2][cc], (_Float16)d[3][cc]};
-        *reinterpret_cast<f16x4*>(base + d_lane + cc * 8) = pk;
+        const f16x8 pk = {(_Float16)d[0][0], (_Float16)d[1][0], (_Float16)d[2][0], (_Float16)d[3][0],
+                          (_Float16)d[0][1], (_Float16)d[1][1], (_Float16)d[2][1], (_Float16)d[3][1]};
+        *reinterpret_cast<f16x8*>(base + d_lane) = pk;
       }
     } else if (SAVE) {
       const int cc = slot - 6;   // r after step t is the operand of step t+1

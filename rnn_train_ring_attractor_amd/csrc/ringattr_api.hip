@@ -240,11 +240,11 @@ static int fwd_impl(const void* A, const void* Wa, float J0, float J1, const voi
     return fail(RINGATTR_ERR_WORKSPACE, "ringattr_fwd: workspace of %zu bytes needed, %zu given", g.wpack_bytes,
                 workspace ? workspace_bytes : (size_t)0);
   hipStream_t st = static_cast<hipStream_t>(stream);
-  if (const int ce = ring_cluster_error())
+  if (const int ce = ring_cluster_take_error())
     return fail(RINGATTR_ERR_HIP,
                 "an earlier cluster forward gave up waiting for a sibling workgroup (code %d: 1 members on different "
-                "XCDs, 2 members not resident together, 3 a published state never arrived); its results are invalid. "
-                "Set RINGATTR_CLUSTER=0 and restart the process",
+                "XCDs, 2 members not resident together, 3 a published state never arrived) and its results are "
+                "invalid; this is reported once, and the streaming kernels run N = 512 from here on",
                 ce);
 
   // With a saved buffer the same launch also writes the transposed copy the backward will need behind the saved
@@ -252,12 +252,13 @@ static int fwd_impl(const void* A, const void* Wa, float J0, float J1, const voi
   // in its own copy and leaves the plain transposed one the streaming BPTT expects.
   const int resident = ring_uses_resident(N, a_dim) ? 1 : 0;
   const size_t cluster_bytes = ring_cluster_applicable(N, a_dim) ? ring_cluster_workspace_bytes(g.nbt) : 0;
-  const bool cluster = !resident && ring_uses_cluster(N, a_dim, g.nbt) && !ring_uses_step_kernels(N, a_dim, g.NC, g.nbt) &&
+  const bool cluster = !resident && ring_uses_cluster(N, a_dim, batch_size, seq_len) && !ring_uses_step_kernels(N, a_dim, g.NC, g.nbt) &&
                        workspace_bytes >= g.wpack_bytes + cluster_bytes;
   void* wpack_t = saved ? (char*)saved + g.side_bytes + g.pair_bytes : nullptr;
   const float s0 = (resident || cluster) ? J1 : 1.f, h0 = (resident || cluster) ? J0 : 0.f;
   const float s2 = resident ? J1 : 1.f, h2 = resident ? J0 : 0.f;
-  hipError_t e = ring_launch_pack2((const float*)Wo, (const float*)Wa, N, a_dim, g.NC, workspace, 0, cluster ? 2 : resident,
+  hipError_t e = ring_launch_pack2((const float*)Wo, (const float*)Wa, N, a_dim, g.NC, workspace, 0,
+                                   cluster ? ring_cluster_pack_order(N, batch_size, seq_len) : resident,
                                    s0, h0, wpack_t, 1, 0, s2, h2, st);
   if (e != hipSuccess) return hip_fail(e, "pack weights");
   if (saved)

@@ -105,3 +105,70 @@ def test_hot_kernels_use_no_scratch(res256_asm):
             seen += 1
             assert int(m.group(1)) == 0, f"{name} spills {m.group(1)} bytes per lane"
     assert seen >= 12
+
+
+# ------------------------------------------------------------------------------------------------
+# The N = 512 cluster forward issues its flag, gate, previous-state and operand loads with inline assembly as
+# well and waits for them with counted s_waitcnt.  Same proof on its emitted code: between such a load and the first
+# wait that covers it nothing reads or writes its destination registers (a copy "into place" ahead of the wait would
+# copy a register that is still being filled), and no variant uses scratch memory.
+# ------------------------------------------------------------------------------------------------
+@pytest.fixture(scope="module")
+def cluster_asm(tmp_path_factory):
+    out = tmp_path_factory.mktemp("isa") / "cluster.s"
+    cmd = [HIPCC, "--offload-arch=gfx950", "-O3", "-std=c++17", "-S", "--cuda-device-only", f"-I{ROOT}/include",
+           f"-I{CSRC}", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+           *PER_SOURCE_FLAGS.get("ring_cluster.hip", []),
+           "-Rpass-analysis=kernel-resource-usage", os.path.join(CSRC, "ring_cluster.hip"), "-o", str(out)]
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    return out.read_text(), proc.stderr
+
+
+@pytest.mark.parametrize("save", [0, 1], ids=["history_only", "with_record"])
+@pytest.mark.parametrize("act", [0, 1, 2, 3], ids=["relu", "gelu", "tanh", "silu"])
+def test_cluster_forward_leaves_in_flight_registers_alone(cluster_asm, act, save):
+    asm, _ = cluster_asm
+    name = f"_Z24ring_fwd_cluster8_kernelILi{act}ELb{save}EEv11RingFwdArgs15RingClusterArgs"
+    i = asm.index(name + ":")
+    body = asm[i:asm.index(".Lfunc_end", i)].split("\n")
+    fifo, in_asm, loads = [], False, 0
+    for ln in body + body:                      # second pass models the loop back edge
+        t = ln.strip()
+        if t.startswith(";;#ASMSTART"):
+            in_asm = True
+            continue
+        if t.startswith(";;#ASMEND"):
+            in_asm = False
+            continue
+        if not t or t[0] in ";.":
+            continue
+        if in_asm and t.startswith("global_load"):
+            fifo.append(_regs(t.split()[1].rstrip(",")))
+            loads += 1
+            continue
+        if t.startswith("s_waitcnt") and "vmcnt" in t:
+            k = int(re.search(r"vmcnt\((\d+)\)", t).group(1))
+            del fifo[:max(0, len(fifo) - k)]
+            continue
+        # every other vector-memory instruction occupies a slot of the same in-order counter
+        if t.startswith(("global_store", "global_load", "buffer_", "scratch_")):
+            fifo.append(set())
+            continue
+        pending = set().union(*fifo) if fifo else set()
+        ops = t.split(None, 1)
+        used = _regs(ops[1]) if len(ops) > 1 else set()
+        assert not (used & pending), f"in-flight registers {sorted(used & pending)} touched by: {t}"
+    assert loads == 2 * 14          # early half: 2 previous-state, gates, flags, 4 operand; late half: gates, flags, 4 operand
+
+
+def test_cluster_forward_uses_no_scratch(cluster_asm):
+    _, remarks = cluster_asm
+    seen = 0
+    for b in re.split(r"remark: Function Name: ", remarks)[1:]:
+        name = b.split()[0]
+        if name.startswith("_Z24ring_fwd_cluster8_kernel"):
+            seen += 1
+            m = re.search(r"ScratchSize \[bytes/lane\]: (\d+)", b)
+            assert int(m.group(1)) == 0, f"{name} spills {m.group(1)} bytes per lane"
+    assert seen == 8
