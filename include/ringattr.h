@@ -63,6 +63,9 @@ RINGATTR_API size_t ringattr_saved_bytes(int N, int a_dim, int seq_len, int batc
 /* Scratch bytes needed by ringattr_fwd / ringattr_bwd.  have_saved = 1 when the
  * forward's saved buffer will be handed to the backward, 0 when the backward
  * must rebuild it from bump_history (then the workspace also holds it).
+ * At N = 512 with two action channels the forward's figure includes the exchange area of the
+ * kernel that spreads the weights over four compute units; a forward handed less than that (but at
+ * least the packed weights) runs the weight-streaming kernel instead.
  * Replaces the fixed workspace list of cpp/ring_rnn_cuda.py:108-114. */
 RINGATTR_API size_t ringattr_fwd_workspace_bytes(int N, int a_dim, int seq_len, int batch_size);
 RINGATTR_API size_t ringattr_bwd_workspace_bytes(int N, int a_dim, int seq_len, int batch_size, int have_saved);
