@@ -66,6 +66,8 @@ RINGATTR_API size_t ringattr_saved_bytes(int N, int a_dim, int seq_len, int batc
  * At N = 512 with two action channels the forward's figure includes the exchange area of the
  * kernel that spreads the weights over four compute units; a forward handed less than that (but at
  * least the packed weights) runs the weight-streaming kernel instead.
+ * The backward's figure at that width includes the scratch area of the BPTT on the same clusters
+ * (switched on by RINGATTR_CLUSTER_BPTT=1), whether it is on or not.
  * Replaces the fixed workspace list of cpp/ring_rnn_cuda.py:108-114. */
 RINGATTR_API size_t ringattr_fwd_workspace_bytes(int N, int a_dim, int seq_len, int batch_size);
 RINGATTR_API size_t ringattr_bwd_workspace_bytes(int N, int a_dim, int seq_len, int batch_size, int have_saved);

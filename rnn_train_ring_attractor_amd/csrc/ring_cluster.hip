@@ -1,5 +1,5 @@
-// Weight-resident forward for N = 512 (NC = 8), a_dim = 2: the weights stay on chip, spread over a cluster of four
-// compute units.
+// Weight-resident forward (and, further down, BPTT) for N = 512 (NC = 8), a_dim = 2: the weights stay on chip, spread
+// over a cluster of four compute units.
 //
 // [Wo|Wl|Wr] in bf16 is 1.5 MiB at N = 512, four times what one compute unit can hold (the streaming kernels
 // therefore pull all of it from L2 once per step and batch-tile pair, and a step is bound by that stream).  Here
@@ -70,16 +70,26 @@ __device__ __forceinline__ void quad_transpose(unsigned (&a)[4], int j) {
 }
 
 // scalar base + 32-bit lane offset + immediate
+// (A store of more than 8 bytes per lane reads its data registers over the cycles after it issues; a vector-ALU write
+// to one of them in the next two wait states changes what is stored.  The compiler keeps that distance for the stores
+// it knows, not for one inside an asm statement, hence the s_nop.)
 template <int IMM>
 __device__ __forceinline__ void sstore16(const void* sbase, unsigned voff, f32x4 v) {
-  asm volatile("global_store_dwordx4 %0, %1, %2 offset:%3" ::"v"(voff), "v"(v), "s"(sbase), "n"(IMM) : "memory");
+  asm volatile("global_store_dwordx4 %0, %1, %2 offset:%3\n\ts_nop 1" ::"v"(voff), "v"(v), "s"(sbase), "n"(IMM) : "memory");
 }
 template <int IMM>
 __device__ __forceinline__ void sstore8(const void* sbase, unsigned voff, f32x2 v) {
   asm volatile("global_store_dwordx2 %0, %1, %2 offset:%3" ::"v"(voff), "v"(v), "s"(sbase), "n"(IMM) : "memory");
 }
+// (A base the compiler cannot prove wave-uniform would be handed over in vector registers, which the instruction does
+// not take: the two halves go through readfirstlane, which costs nothing where the value is scalar already.)
+__device__ __forceinline__ const void* uniform_ptr(const void* ptr) {
+  const unsigned long long a = reinterpret_cast<unsigned long long>(ptr);
+  const unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)a), hi = __builtin_amdgcn_readfirstlane((unsigned)(a >> 32));
+  return reinterpret_cast<const void*>(((unsigned long long)hi << 32) | lo);
+}
 __device__ __forceinline__ void sstore4_dev(const void* sbase, unsigned voff, int v) {
-  asm volatile("global_store_dword %0, %1, %2 sc1" ::"v"(voff), "v"(v), "s"(sbase) : "memory");
+  asm volatile("global_store_dword %0, %1, %2 sc1" ::"v"(voff), "v"(v), "s"(uniform_ptr(sbase)) : "memory");
 }
 template <int IMM>
 __device__ __forceinline__ f32x4 sload16(const void* sbase, unsigned voff) {
@@ -91,6 +101,12 @@ template <int IMM>
 __device__ __forceinline__ f32x4 sload16_dev(const void* sbase, unsigned voff) {
   f32x4 v;
   asm volatile("global_load_dwordx4 %0, %1, %2 offset:%3 sc1" : "=&v"(v) : "v"(voff), "s"(sbase), "n"(IMM) : "memory");
+  return v;
+}
+template <int IMM>
+__device__ __forceinline__ f32x2 sload8(const void* sbase, unsigned voff) {
+  f32x2 v;
+  asm volatile("global_load_dwordx2 %0, %1, %2 offset:%3" : "=&v"(v) : "v"(voff), "s"(sbase), "n"(IMM) : "memory");
   return v;
 }
 __device__ __forceinline__ int sload4_dev(const void* sbase, unsigned voff) {
@@ -518,6 +534,424 @@ __global__ __launch_bounds__(512) void ring_fwd_cluster8_kernel(RingFwdArgs p, R
 }
 
 // ------------------------------------------------------------------------------------------------
+// BPTT on the same clusters.  Visit s = 0 .. T-1 of a pair produces g of step t = T-1-s:
+//     carry_t = (1 - alpha) G_{t+1} + [g_{t+1} (J1 Wo + J0)] + sum_c A_c(t+1) [g_{t+1} Wa_c]     (0 at t = T-1)
+//     G_t = grad_output_t + carry_t,      g_t = (alpha F'(re_t)) G_t                              (the record carries alpha)
+// with the products in brackets taken over all N neurons of g_{t+1}: that is what the members exchange, by the
+// forward's protocol with s in the place of its t (state s = g_{t+1}; a pair's first visit has no products).  Wpack holds
+// the transposed matrices in this kernel's column order, J1 Wo^T + J0 as matrix 0.  What a pair carries from one
+// visit to the next besides the exchanged g lives in a private scratch record per lane: (1 - alpha) G_t for its four
+// rows (fp32) and, behind odd steps, the bf16 g of those rows: the copy of g for the weight-gradient kernel keeps
+// steps 2j and 2j+1 side by side in one 16-byte slot, and the even step that follows stores the slot whole.
+// One more visit (t = -1) forms dL/dr_init when it is asked for.  No dL/dA and no fused loss head here: the caller
+// runs those on the streaming kernel.
+// ------------------------------------------------------------------------------------------------
+template <bool GRI>
+__global__ __launch_bounds__(512) void ring_bptt_cluster8_kernel(RingBpttArgs p, RingClusterArgs c) {
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  bf16x8* wlds = reinterpret_cast<bf16x8*>(smem);
+  bf16x8* xs = wlds + C8_WSLOTS;
+  float* gl = reinterpret_cast<float*>(xs + C_XSLOTS);   // [2][32 rows][2] action gates, by pair-step parity
+  int* misc = reinterpret_cast<int*>(gl + 128);          // [0]: abort
+  char* const xchg = reinterpret_cast<char*>(c.xchg);
+  constexpr int NSTE = 6;                                // stores of every epilogue: per tile exchange, carry record, g
+
+  const int tid = threadIdx.x, w8 = tid >> 6, v = w8 & 3, h = w8 >> 2, lane = tid & 63, q = lane >> 4, n = lane & 15,
+            g4 = n >> 2, j4 = n & 3;
+  const int ct = 2 * v + h;
+  const int blk = blockIdx.x, xcd = blk & 7, gi = blk >> 3, m = gi & 3, cl = (gi >> 2) * 8 + xcd;
+  if (cl >= c.nclusters) return;
+  const int B = p.B, T = p.T, nbt = p.nbt;
+  constexpr int N = 512;
+  const int S = T + (GRI ? 1 : 0);   // visits per pair
+  const int my_ppc = (c.npairs - cl + c.nclusters - 1) / c.nclusters;
+  const int w8u = __builtin_amdgcn_readfirstlane(w8);
+  const bool skew = __builtin_amdgcn_readfirstlane(h) == 1 && my_ppc >= 2;
+
+  if (tid == 0) misc[0] = 0;
+  if (w8 == 0) {
+    const int mine = (__builtin_amdgcn_s_getreg(20 | (0 << 6) | (3 << 11)) & 15) + 1;   // XCC_ID + 1
+    if (lane == 0) flag_store(c.hello + cl * 4 + m, mine);
+    int bad = c.spin_max < 0 ? 2 : 0;
+    for (int spins = 0; !bad; ++spins) {
+      const int hh = lane < 4 ? flag_load(c.hello + cl * 4 + lane) : mine;
+      if (__ballot(hh == 0) == 0) {
+        bad = __ballot(hh != mine) != 0 ? 1 : 0;
+        break;
+      }
+      if (spins > c.spin_max) {
+        bad = 2;
+        break;
+      }
+      __builtin_amdgcn_s_sleep(8);
+    }
+    if (bad && lane == 0) {
+      misc[0] = 1;
+      *c.host_err = bad == 1 ? RING_CLUSTER_ERR_XCD : RING_CLUSTER_ERR_START;
+    }
+  }
+
+  bf16x8 wreg[2][C_KCH];
+  bf16x8 wo_last;
+  bf16x8* wl = wlds + (size_t)(w8 * C8_WFR) * 64 + lane;
+  {
+    const bf16x8* Wp = reinterpret_cast<const bf16x8*>(p.Wpack);
+#pragma unroll
+    for (int kc = 0; kc < C_KCH; ++kc) {
+      wreg[0][kc] = Wp[((size_t)((1 * 4 + m) * C_NC + ct) * C_KCH + kc) * 64 + lane];
+      wreg[1][kc] = Wp[((size_t)((2 * 4 + m) * C_NC + ct) * C_KCH + kc) * 64 + lane];
+    }
+#pragma unroll
+    for (int k8 = 0; k8 < C_KCH; k8 += 8) {
+      bf16x8 f[8];
+#pragma unroll
+      for (int x = 0; x < 8; ++x) f[x] = Wp[((size_t)((0 * 4 + m) * C_NC + ct) * C_KCH + k8 + x) * 64 + lane];
+#pragma unroll
+      for (int x = 0; x < 8; ++x) {
+        if (k8 + x < C8_WFR) wl[(k8 + x) * 64] = f[x];
+        else wo_last = f[x];
+      }
+    }
+#pragma unroll
+    for (int kc = 0; kc < C_KCH; ++kc) {
+      asm volatile("" : "+a"(wreg[0][kc]));
+      asm volatile("" : "+a"(wreg[1][kc]));
+    }
+  }
+
+  const float oma = 1.f - p.alpha;
+  const size_t xhalf_bytes = (size_t)2 * c.npairs * C_TILE_UNITS * 16;
+  char* const bin = xchg + 2 * xhalf_bytes;
+  char* const carry = reinterpret_cast<char*>(c.carry);     // [batch tile][member][wave][lane] x 16 bytes
+  char* const ghalf = reinterpret_cast<char*>(c.ghalf);     // the same, first 8 bytes: bf16 g of the last odd step
+  // lane-constant byte offsets
+  const unsigned row_lane = (unsigned)(((4 * q + j4) * N + 128 * m + 16 * ct + 4 * g4) * 4);   // fp32 [16 rows][N]: row 4q+j4, four neurons
+  const unsigned xq_lane = (unsigned)(((((4 * m + (ct >> 1)) * 4 + 2 * (ct & 1) + (g4 >> 1)) * 16) + 4 * q + j4) * 16 + 8 * (g4 & 1));
+  const int lane_c = (lane & 48) | (2 * ct + (n >> 3)), cp = n & 7;   // the neuron's place in the common tile order
+  const unsigned d_lane = (unsigned)(lane_c * 64 + 8 * cp);
+  const unsigned r_lane = (unsigned)((cp * 64 + lane_c) * 16);
+  const unsigned x_lane = (unsigned)(lane * 16);
+  const unsigned g_lane = (unsigned)(((lane >> 1) * T * 2 + (lane & 1)) * 4);
+  const unsigned f_lane = (unsigned)((lane & 31) * 4);
+  const unsigned c_lane = (unsigned)(((m * 8 + w8) * 64 + lane) * 16);
+
+  auto rows_base = [&](const float* base, int t, int bt) { return reinterpret_cast<const char*>(base) + ((size_t)t * B + 16 * bt) * N * 4; };
+  auto flag_base = [&](int pl) { return reinterpret_cast<const char*>(c.flags) + ((size_t)cl * c.ppc + pl) * 32 * 4; };
+  auto x_base = [&](int s, int pr) {
+    return xchg + (size_t)(s & 1) * xhalf_bytes + ((size_t)(2 * pr) * C_TILE_UNITS + w8u * 256) * 16;
+  };
+  // gates of visit s: those of step t+1 = T - s, the step whose g is multiplied (the first visit multiplies zeros)
+  auto gate_base = [&](int s, int pr) {
+    const int tg = s == 0 ? T - 1 : T - s;
+    return reinterpret_cast<const char*>(p.A) + ((size_t)(32 * pr) * T + tg) * 8;
+  };
+
+  int pf_pl = -1, pf_val = 0;   // exchange stores issued, flag not yet up: pair (local) and state number
+  f32x4 P[2][3];                // products of the visit in hand: [tile][matrix]
+  // what the epilogue of a visit reads besides P: grad_output rows (row 4q+j4, four neurons), the carry record, F', the held g half
+  struct EpiIn {
+    f32x4 go[2], cp[2];
+    f32x2 fd[2], gh[2];
+  };
+  EpiIn Lr;
+  int es = 0, epr = 0, epl = 0, eit = 0;   // the visit whose products are in P and whose epilogue is still to run (late half)
+  bool epending = false;
+
+  // Epilogue of visit (s, pr, pl), number `it` in this cluster's order, one batch tile at a time: the arithmetic on P
+  // and the loaded inputs, then the tile's three stores (exchange, carry record, g copy).  The count of stores is the
+  // same on every path -- the staging of the next operand counts on it -- so what has no place to go goes to the bin.
+  struct EpiT {
+    f32x2 xe;
+    f32x4 cv, gvv;
+  };
+  auto epi_tile_math = [&](auto tlv, int s, int it, const EpiIn& in, EpiT& o) {
+    constexpr int tl = decltype(tlv)::value;
+    const float* gb = gl + (it & 1) * 64;
+    const int t = T - 1 - s;
+    const bool last = GRI && t < 0;       // the visit that forms dL/dr_init
+    unsigned gr[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float e0 = in.go[tl][i];
+      gr[i] = __builtin_bit_cast(unsigned, e0);
+    }
+    quad_transpose(gr, j4);   // -> rows 4q+e of the lane's own neuron
+    const f32x4 ga = *reinterpret_cast<const f32x4*>(gb + (16 * tl + 4 * q) * 2);
+    const f32x4 gc = *reinterpret_cast<const f32x4*>(gb + (16 * tl + 4 * q + 2) * 2);
+    const f16x4 d4 = __builtin_bit_cast(f16x4, in.fd[tl]);
+    float gv[4], cn[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const float g0 = e < 2 ? ga[2 * e] : gc[2 * (e - 2)], g1 = e < 2 ? ga[2 * e + 1] : gc[2 * (e - 2) + 1];
+      const float p0 = P[tl][0][e], p1 = P[tl][1][e], p2 = P[tl][2][e];
+      const float cprev = in.cp[tl][e];
+      // (a pair's first visit has no step behind it: whatever operand was staged for it, its products are dropped)
+      const float carry_t = s > 0 ? cprev + fmaf(g1, p2, fmaf(g0, p1, p0)) : 0.f;
+      const float G = last ? carry_t : __builtin_bit_cast(float, gr[e]) + carry_t;
+      const float dF = (float)d4[e];
+      gv[e] = last ? G : dF * G;          // (last: the rows of dL/dr_init travel in gv)
+      cn[e] = oma * G;
+    }
+    const bf16x4 g4b = {(__bf16)gv[0], (__bf16)gv[1], (__bf16)gv[2], (__bf16)gv[3]};
+    const f32x2 gk = __builtin_bit_cast(f32x2, g4b);
+    unsigned hh[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) hh[e] = __builtin_bit_cast(unsigned, gv[e]);
+    quad_transpose(hh, j4);   // -> row 4q+j4, neurons 4 g4 + i
+    const float h0 = __builtin_bit_cast(float, hh[0]), h1 = __builtin_bit_cast(float, hh[1]), h2 = __builtin_bit_cast(float, hh[2]),
+                h3 = __builtin_bit_cast(float, hh[3]);
+    const bf16x2 b01 = {(__bf16)h0, (__bf16)h1}, b23 = {(__bf16)h2, (__bf16)h3};
+    o.xe = f32x2{__builtin_bit_cast(float, b01), __builtin_bit_cast(float, b23)};
+    // (the dL/dr_init visit stores its fp32 rows where the others store the carry record)
+    o.cv = f32x4{last ? h0 : cn[0], last ? h1 : cn[1], last ? h2 : cn[2], last ? h3 : cn[3]};
+    const bool tail = t + 1 < T;
+    o.gvv = f32x4{gk[0], gk[1], tail ? in.gh[tl][0] : 0.f, tail ? in.gh[tl][1] : 0.f};   // (an odd length's last slot: zero tail)
+  };
+  auto epi_tile_stores = [&](auto tlv, int s, int pr, const EpiT& o) {
+    constexpr int tl = decltype(tlv)::value;
+    const int t = T - 1 - s;
+    const bool last = GRI && t < 0;
+    const bool more = s + 1 < S;
+    // 1: the exchange (a pair's last visit: nobody reads it)
+    {
+      const char* xb = xchg + (size_t)((s + 1) & 1) * xhalf_bytes + (size_t)(2 * pr + tl) * C_TILE_UNITS * 16;
+      sstore8<0>(more ? xb : bin, xq_lane, o.xe);
+    }
+    // 2: the carry record, or the rows of dL/dr_init
+    {
+      const char* cb = carry + (size_t)(2 * pr + tl) * 32768;
+      const char* ib = reinterpret_cast<const char*>(p.grad_r_init) + (size_t)(32 * pr + 16 * tl) * N * 4;
+      sstore16<0>(last ? ib : cb, last ? row_lane : c_lane, o.cv);
+    }
+    // 3: the copy of g for the weight gradient: an odd step's half is held in the private record until the even step
+    // that follows stores the slot whole
+    {
+      const char* hb = ghalf + (size_t)(2 * pr + tl) * 32768;
+      const int tt = t < 0 ? 0 : t;
+      const char* rb = reinterpret_cast<const char*>(p.gfrag) + (((size_t)(tt >> 1) * nbt + 2 * pr + tl) * 32 + 8 * m) * 64 * 16;
+      const bool whole = !last && (t & 1) == 0;
+      // (the half goes out as a whole 16-byte record too: one form of store on both paths)
+      sstore16<0>(last ? bin : whole ? rb : hb, whole ? r_lane : c_lane, o.gvv);
+    }
+  };
+  auto epi_done = [&](int s, int pl) {
+    pf_pl = s + 1 < S ? pl : -1;
+    pf_val = s + 1;
+  };
+
+  // the first visit has nothing to multiply (its products are dropped); zeros keep the matrix pipe's inputs tame
+  {
+    const bf16x8 z8 = {(__bf16)0.f, (__bf16)0.f, (__bf16)0.f, (__bf16)0.f, (__bf16)0.f, (__bf16)0.f, (__bf16)0.f, (__bf16)0.f};
+#pragma unroll
+    for (int jj = 0; jj < 4; ++jj) xs[w8 * 256 + jj * 64 + lane] = z8;
+  }
+  if (w8 == 0) gl[lane] = *reinterpret_cast<const float*>(gate_base(0, cl) + g_lane);
+  lds_barrier();
+  if (misc[0]) return;
+
+  // The two halves run different loops (one body, compiled twice): what the late half carries from one visit to the
+  // next -- its products and the loaded inputs of the epilogue still to run -- would otherwise occupy registers on the
+  // early half's path as well.
+  auto run = [&](auto skv) {
+    constexpr bool SK = decltype(skv)::value;
+    int s = 0, pl = 0, it = 0;
+    for (;;) {
+      const int pr = cl + c.nclusters * pl;
+      int ns = s, npl = pl + 1;
+      if (npl == my_ppc) {
+        npl = 0;
+        ns = s + 1;
+      }
+      const bool have_next = ns < S;
+      const bool look = have_next && ns >= 1;
+      const int npr = cl + c.nclusters * npl;
+      const int tc = T - 1 - s < 0 ? 0 : T - 1 - s;   // the step whose inputs this visit's epilogue reads (the last visit: none)
+
+      f32x4 sreg[4];      // this wave's eighth of the next visit's operand
+      int nflag;
+      float gnext;
+      bool up = false;
+      auto fetch_issue = [&]() {
+        gnext = sload4(have_next ? gate_base(ns, npr) : gate_base(s, pr), g_lane);
+        nflag = sload4_dev(flag_base(look ? npl : pl), f_lane);
+      };
+      auto fetch_decide = [&]() {
+        asm volatile("s_waitcnt vmcnt(0)" : "+v"(nflag), "+v"(gnext)::"memory");
+        up = look && __ballot(nflag < ns) == 0;
+        sstore4_dev(pf_pl >= 0 ? flag_base(pf_pl) : bin, (unsigned)((8 * m + w8u) * 4), pf_val);   // (every lane the same word)
+        pf_pl = -1;
+      };
+      auto fetch_x = [&](auto iv) {
+        constexpr int i = decltype(iv)::value;
+        const char* xb = look ? x_base(ns, npr) : x_base(s, pr);
+        sreg[i] = sload16_dev<1024 * i>(xb, x_lane);
+      };
+
+      const bool thin = SK && !epending;
+      if constexpr (SK) {
+        EpiT o = {};
+        fetch_issue();
+        if (epending) epi_tile_math(std::integral_constant<int, 0>{}, es, eit, Lr, o);
+        fetch_decide();
+        fetch_x(std::integral_constant<int, 0>{});
+        fetch_x(std::integral_constant<int, 1>{});
+        fetch_x(std::integral_constant<int, 2>{});
+        fetch_x(std::integral_constant<int, 3>{});
+        if (epending) {
+          epi_tile_stores(std::integral_constant<int, 0>{}, es, epr, o);
+          epi_tile_math(std::integral_constant<int, 1>{}, es, eit, Lr, o);
+          epi_tile_stores(std::integral_constant<int, 1>{}, es, epr, o);
+          epi_done(es, epl);
+        }
+      }
+
+      // ---- products ----
+      {
+        const f32x4 z = {0.f, 0.f, 0.f, 0.f};
+  #pragma unroll
+        for (int tl = 0; tl < 2; ++tl) P[tl][0] = P[tl][1] = P[tl][2] = z;
+      }
+      const char* const gob = rows_base(p.grad_out, tc, 2 * pr);
+      const char* const fdb = reinterpret_cast<const char*>(p.dfrag) + ((((size_t)tc * nbt + 2 * pr) * 4 + m) * 64) * 64;
+      const char* const cpb = carry + (size_t)(2 * pr) * 32768;
+      const char* const ghb = ghalf + (size_t)(2 * pr) * 32768;
+      bf16x8 af[2][2], wf[2];
+      auto frag_fetch = [&](auto kcv, int stg) {
+        constexpr int kc = decltype(kcv)::value;
+        af[stg][0] = xs[(0 * C_KCH + kc) * 64 + lane];
+        af[stg][1] = xs[(1 * C_KCH + kc) * 64 + lane];
+        if constexpr (kc < C8_WFR) wf[stg] = wl[kc * 64];
+        else wf[stg] = wo_last;
+      };
+      auto body = [&](auto kcv, auto slotsv) {
+        constexpr int kc = decltype(kcv)::value, stg = kc & 1;
+        if constexpr (kc + 1 < C_KCH) frag_fetch(std::integral_constant<int, kc + 1>{}, stg ^ 1);
+        __builtin_amdgcn_sched_barrier(0);
+        if constexpr (decltype(slotsv)::value) {
+          if constexpr (kc == 0) fetch_issue();
+          if constexpr (kc == 12) fetch_decide();
+          if constexpr (kc >= 12) fetch_x(std::integral_constant<int, kc - 12>{});
+          __builtin_amdgcn_sched_barrier(0);
+        }
+        P[0][1] = mfma16(af[stg][0], wreg[0][kc], P[0][1]);
+        P[1][1] = mfma16(af[stg][1], wreg[0][kc], P[1][1]);
+        P[0][2] = mfma16(af[stg][0], wreg[1][kc], P[0][2]);
+        P[1][2] = mfma16(af[stg][1], wreg[1][kc], P[1][2]);
+        P[0][0] = mfma16(af[stg][0], wf[stg], P[0][0]);
+        P[1][0] = mfma16(af[stg][1], wf[stg], P[1][0]);
+        __builtin_amdgcn_sched_barrier(0);
+      };
+      auto products = [&](auto slotsv) {
+        frag_fetch(std::integral_constant<int, 0>{}, 0);
+        __builtin_amdgcn_s_setprio(C8_PRIO);
+        body(std::integral_constant<int, 0>{}, slotsv);
+        body(std::integral_constant<int, 1>{}, slotsv);
+        body(std::integral_constant<int, 2>{}, slotsv);
+        body(std::integral_constant<int, 3>{}, slotsv);
+        body(std::integral_constant<int, 4>{}, slotsv);
+        body(std::integral_constant<int, 5>{}, slotsv);
+        body(std::integral_constant<int, 6>{}, slotsv);
+        body(std::integral_constant<int, 7>{}, slotsv);
+        body(std::integral_constant<int, 8>{}, slotsv);
+        body(std::integral_constant<int, 9>{}, slotsv);
+        body(std::integral_constant<int, 10>{}, slotsv);
+        body(std::integral_constant<int, 11>{}, slotsv);
+        body(std::integral_constant<int, 12>{}, slotsv);
+        body(std::integral_constant<int, 13>{}, slotsv);
+        body(std::integral_constant<int, 14>{}, slotsv);
+        body(std::integral_constant<int, 15>{}, slotsv);
+        __builtin_amdgcn_s_setprio(0);
+      };
+      if constexpr (SK) {
+        // (ordinary loads: they are read in the next visit's first phase, and the compiler waits for them there)
+        Lr.go[0] = *reinterpret_cast<const f32x4*>(gob + row_lane);
+        Lr.go[1] = *reinterpret_cast<const f32x4*>(gob + 16 * N * 4 + row_lane);
+        Lr.cp[0] = *reinterpret_cast<const f32x4*>(cpb + c_lane);
+        Lr.cp[1] = *reinterpret_cast<const f32x4*>(cpb + 32768 + c_lane);
+        Lr.fd[0] = *reinterpret_cast<const f32x2*>(fdb + d_lane);
+        Lr.fd[1] = *reinterpret_cast<const f32x2*>(fdb + 4 * 64 * 64 + d_lane);
+        Lr.gh[0] = *reinterpret_cast<const f32x2*>(ghb + c_lane);
+        Lr.gh[1] = *reinterpret_cast<const f32x2*>(ghb + 32768 + c_lane);
+        products(std::false_type{});
+        es = s;
+        epr = pr;
+        epl = pl;
+        eit = it;
+        epending = true;
+      } else {
+        // the early half reads them right behind its products: seven operations younger (gates, flags, the flag
+        // store, four operand loads) are still allowed to be out when it does
+        EpiIn La;
+        La.go[0] = sload16<0>(gob, row_lane);
+        La.go[1] = sload16<0>(gob + 16 * N * 4, row_lane);
+        La.cp[0] = sload16<0>(cpb, c_lane);
+        La.cp[1] = sload16<0>(cpb + 32768, c_lane);
+        La.fd[0] = sload8<0>(fdb, d_lane);
+        La.fd[1] = sload8<0>(fdb + 4 * 64 * 64, d_lane);
+        La.gh[0] = sload8<0>(ghb, c_lane);
+        La.gh[1] = sload8<0>(ghb + 32768, c_lane);
+        products(std::true_type{});
+        asm volatile("s_waitcnt vmcnt(7)"
+                     : "+v"(La.go[0]), "+v"(La.go[1]), "+v"(La.cp[0]), "+v"(La.cp[1]), "+v"(La.fd[0]), "+v"(La.fd[1]), "+v"(La.gh[0]),
+                       "+v"(La.gh[1])::"memory");
+        EpiT o;
+        epi_tile_math(std::integral_constant<int, 0>{}, s, it, La, o);
+        epi_tile_stores(std::integral_constant<int, 0>{}, s, pr, o);
+        epi_tile_math(std::integral_constant<int, 1>{}, s, it, La, o);
+        epi_tile_stores(std::integral_constant<int, 1>{}, s, pr, o);
+        epi_done(s, pl);
+      }
+
+      // ---- the next visit's operand and gates into LDS ----
+      lds_barrier();
+      if (thin) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NSTE) : "memory");
+      if (!have_next) break;
+      if (up) {
+  #pragma unroll
+        for (int jj = 0; jj < 4; ++jj) xs[w8 * 256 + jj * 64 + lane] = __builtin_bit_cast(bf16x8, sreg[jj]);
+      } else {
+        // nothing valid was fetched ahead: put up the flag still held back (the producers of what is waited for may
+        // be waiting for it in turn), wait for the flags, then ordinary loads behind a device-scope acquire
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        if (pf_pl >= 0) sstore4_dev(flag_base(pf_pl), (unsigned)((8 * m + w8u) * 4), pf_val);
+        pf_pl = -1;
+        bool ok = false;
+        for (int spins = 0; spins <= c.spin_max; ++spins) {
+          const int f = flag_load(c.flags + ((size_t)cl * c.ppc + npl) * 32 + (lane & 31));
+          if ((ok = (__ballot(f < ns) == 0))) break;
+          __builtin_amdgcn_s_sleep(2);
+        }
+        if (!ok && lane == 0) {
+          misc[0] = 1;
+          *c.host_err = RING_CLUSTER_ERR_WAIT;
+        }
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+        const bf16x8* xb = reinterpret_cast<const bf16x8*>(x_base(ns, npr));
+  #pragma unroll
+        for (int jj = 0; jj < 4; ++jj) xs[w8 * 256 + jj * 64 + lane] = xb[jj * 64 + lane];
+      }
+      if (w8 == 0) gl[((it + 1) & 1) * 64 + lane] = gnext;
+      lds_barrier();
+      if (misc[0]) return;
+      s = ns;
+      pl = npl;
+      ++it;
+    }
+    if (SK && epending) {
+      EpiT o;
+      epi_tile_math(std::integral_constant<int, 0>{}, es, eit, Lr, o);
+      epi_tile_stores(std::integral_constant<int, 0>{}, es, epr, o);
+      epi_tile_math(std::integral_constant<int, 1>{}, es, eit, Lr, o);
+      epi_tile_stores(std::integral_constant<int, 1>{}, es, epr, o);
+    }
+
+  };
+  if (skew) run(std::true_type{});
+  else run(std::false_type{});
+}
+
+// ------------------------------------------------------------------------------------------------
 // Host side.
 // ------------------------------------------------------------------------------------------------
 namespace {
@@ -588,12 +1022,11 @@ int ring_cluster_take_error() {
 // still computing and the streaming kernels are several times faster.  RINGATTR_CLUSTER=0 switches it off, =1 on
 // wherever the shape allows (tests of the short rotations).  Unasked, it also wants the device it was measured on
 // (256 compute units in 8 XCDs); the placement check in the kernel is what it relies on elsewhere.
-bool ring_uses_cluster(int N, int k, int B, int T) {
+// (1: the cluster kernels can run this shape here; 0: not; ppc: batch-tile pairs per cluster)
+static bool cluster_can_run(int N, int k, int B, int T, int* ppc, int* cus_out) {
   if (!ring_cluster_applicable(N, k) || B % 32 != 0 || T > (1 << 20)) return false;   // whole pairs of batch tiles
-  const int nbt = B / 16;
   const char* v = getenv("RINGATTR_CLUSTER");
   if (v && v[0] == '0') return false;
-  const bool forced = v && v[0] == '1';
   if (ring_cluster_error()) return false;
   static int cus = 0;
   if (cus == 0) {
@@ -602,12 +1035,39 @@ bool ring_uses_cluster(int N, int k, int B, int T) {
         hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = -1;
     cus = n;
   }
-  const ClusterGeo g = cluster_geo(nbt);
+  const ClusterGeo g = cluster_geo(B / 16);
   if (g.grid > cus) return false;   // every workgroup needs a compute unit of its own, all at once
-  return forced || (cus == 256 && g.ppc >= 4 && T >= 16);
+  *ppc = g.ppc;
+  *cus_out = cus;
+  return true;
+}
+
+bool ring_uses_cluster(int N, int k, int B, int T) {
+  int ppc = 0, cus = 0;
+  if (!cluster_can_run(N, k, B, T, &ppc, &cus)) return false;
+  const char* v = getenv("RINGATTR_CLUSTER");
+  const bool forced = v && v[0] == '1';
+  return forced || (cus == 256 && ppc >= 4 && T >= 16);
+}
+
+// The cluster BPTT runs only where it is asked for (RINGATTR_CLUSTER_BPTT=1): at N = 512, B = 8192, T = 512 it takes
+// 10.5 to 10.9 ms against the streaming kernel's 10.6, and the weight-gradient kernel behind it runs 0.5 ms slower.
+// Unlike the forward, a visit has per-lane state to carry (fp32, 32 bytes per lane and pair) that fits neither the
+// registers nor LDS beside the weights; its loads and stores, and the misses they cause in an L2 that also holds the
+// exchange buffer, cost what keeping the weights on chip gains.
+bool ring_uses_cluster_bptt(int N, int k, int B, int T) {
+  const char* v = getenv("RINGATTR_CLUSTER_BPTT");
+  if (!v || v[0] != '1') return false;
+  int ppc = 0, cus = 0;
+  return cluster_can_run(N, k, B, T, &ppc, &cus);
 }
 
 int ring_cluster_pack_order(int, int, int) { return 3; }
+
+size_t ring_cluster_bptt_workspace_bytes(int nbt) {
+  const ClusterGeo g = cluster_geo(nbt);
+  return ring_cluster_workspace_bytes(nbt) + (size_t)2 * g.npairs * (32768 + 32768);   // + carry records, held g halves
+}
 
 template <int ACT>
 static hipError_t launch_fwd_cluster_act(const RingFwdArgs& a, const RingClusterArgs& c, int grid, hipStream_t st) {
@@ -621,14 +1081,15 @@ static hipError_t launch_fwd_cluster_act(const RingFwdArgs& a, const RingCluster
   return a.dfrag ? go(ring_fwd_cluster8_kernel<ACT, true>) : go(ring_fwd_cluster8_kernel<ACT, false>);
 }
 
-hipError_t ring_launch_fwd_cluster(const RingFwdArgs& a, hipStream_t st) {
-  if (!a.cluster_ws || !ring_cluster_applicable(a.N, a.k) || a.B % 32 != 0 || !a.hist) return hipErrorInvalidValue;
-  const ClusterGeo g = cluster_geo(a.nbt);
-  RingClusterArgs c;
-  char* ws = static_cast<char*>(a.cluster_ws);
+// The scratch area's parts, the flags cleared (on the stream, by a small kernel: the launch may be under graph capture).
+static hipError_t cluster_args(void* cluster_ws, int nbt, RingClusterArgs& c, int& grid, hipStream_t st) {
+  const ClusterGeo g = cluster_geo(nbt);
+  char* ws = static_cast<char*>(cluster_ws);
   c.xchg = ws;
   c.flags = reinterpret_cast<int*>(ws + g.xchg_bytes);
   c.hello = reinterpret_cast<int*>(ws + g.xchg_bytes + g.flag_bytes);
+  c.carry = reinterpret_cast<float*>(ws + g.xchg_bytes + g.flag_bytes + g.hello_bytes);
+  c.ghalf = ws + g.xchg_bytes + g.flag_bytes + g.hello_bytes + (size_t)2 * g.npairs * 32768;
   hipError_t e = host_err_word(&c.host_err);
   if (e != hipSuccess) return e;
   c.npairs = g.npairs;
@@ -639,15 +1100,41 @@ hipError_t ring_launch_fwd_cluster(const RingFwdArgs& a, hipStream_t st) {
     const long s = atol(v);
     if (s >= -1 && s <= 100000000L) c.spin_max = (int)s;
   }
+  grid = g.grid;
   const int nclear = (int)((g.flag_bytes + g.hello_bytes) / sizeof(int));
   hipLaunchKernelGGL(ring_cluster_clear_kernel, dim3((nclear + 255) / 256), dim3(256), 0, st, c.flags, nclear);
-  e = hipGetLastError();
+  return hipGetLastError();
+}
+
+hipError_t ring_launch_bptt_cluster(const RingBpttArgs& a, hipStream_t st) {
+  if (!a.cluster_ws || !ring_cluster_applicable(a.N, a.k) || a.B % 32 != 0 || a.grad_A || a.loss_coef || !a.grad_out ||
+      !a.dfrag || !a.gfrag)
+    return hipErrorInvalidValue;
+  RingClusterArgs c;
+  int grid = 0;
+  hipError_t e = cluster_args(a.cluster_ws, a.nbt, c, grid, st);
+  if (e != hipSuccess) return e;
+  auto go = [&](auto kern) {
+    hipError_t e2 = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                        (int)C8_LDS_BYTES);
+    if (e2 != hipSuccess) return e2;
+    RING_LAUNCH(kern, dim3(grid), dim3(512), C8_LDS_BYTES, st, a, c);
+    return hipGetLastError();
+  };
+  return a.grad_r_init ? go(ring_bptt_cluster8_kernel<true>) : go(ring_bptt_cluster8_kernel<false>);
+}
+
+hipError_t ring_launch_fwd_cluster(const RingFwdArgs& a, hipStream_t st) {
+  if (!a.cluster_ws || !ring_cluster_applicable(a.N, a.k) || a.B % 32 != 0 || !a.hist) return hipErrorInvalidValue;
+  RingClusterArgs c;
+  int grid = 0;
+  hipError_t e = cluster_args(a.cluster_ws, a.nbt, c, grid, st);
   if (e != hipSuccess) return e;
   switch (a.act) {
-    case ACT_RELU: return launch_fwd_cluster_act<ACT_RELU>(a, c, g.grid, st);
-    case ACT_GELU: return launch_fwd_cluster_act<ACT_GELU>(a, c, g.grid, st);
-    case ACT_TANH: return launch_fwd_cluster_act<ACT_TANH>(a, c, g.grid, st);
-    case ACT_SILU: return launch_fwd_cluster_act<ACT_SILU>(a, c, g.grid, st);
+    case ACT_RELU: return launch_fwd_cluster_act<ACT_RELU>(a, c, grid, st);
+    case ACT_GELU: return launch_fwd_cluster_act<ACT_GELU>(a, c, grid, st);
+    case ACT_TANH: return launch_fwd_cluster_act<ACT_TANH>(a, c, grid, st);
+    case ACT_SILU: return launch_fwd_cluster_act<ACT_SILU>(a, c, grid, st);
     default: return hipErrorInvalidValue;
   }
 }

@@ -1330,6 +1330,7 @@ static hipError_t launch_bptt_stream(const RingBpttArgs& a, dim3 grid, size_t dy
 hipError_t ring_launch_bptt(const RingBpttArgs& a, int NCv, hipStream_t st) {
   ProfScope prof(3, st);
   hipError_t e = hipErrorInvalidValue;
+  if (a.cluster_ws) return ring_launch_bptt_cluster(a, st);   // (the caller's choice: ring_uses_cluster_bptt)
   if (ring_uses_step_kernels(a.N, a.k, NCv, a.nbt)) {
     if (a.grad_A || !a.wide_carry) return hipErrorInvalidValue;   // (dL/dA comes from a pass of its own, see the C ABI)
     return step_prefers_wide(NCv, a.nbt, a.k) ? ring_launch_wide_bptt(a, NCv, a.wide_carry, st)

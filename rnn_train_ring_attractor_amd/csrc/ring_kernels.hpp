@@ -42,6 +42,7 @@ struct RingBpttArgs {
   float* wide_carry;     // N > 512 only: 2 x [16*nbt][NPAD] fp32 scratch for the carried gradient between step launches
   float J0, J1, alpha;
   int N, k, T, B, nbt;
+  void* cluster_ws = nullptr;   // non-null: the cluster kernel (ring_cluster.hip), ring_cluster_bptt_workspace_bytes(nbt) bytes
 };
 
 struct RingDwArgs {
@@ -81,16 +82,21 @@ struct RingClusterArgs {
   int* flags;        // [nclusters][ppc][32]: last state number published per (pair, member, wave)
   int* hello;        // [nclusters][4]: XCC_ID + 1 of each member
   int* host_err;     // word in pinned host memory, RING_CLUSTER_ERR_* when a wait ran out
+  void* ghalf;       // BPTT: the same order x 16 bytes, the first 8: bf16 g of the last odd step
+  float* carry;      // BPTT: [2 * npairs][4 members][8 waves][64 lanes] x 16 bytes, (1 - alpha) G of the lane's four rows
   int npairs, nclusters, ppc, spin_max;
 };
 enum { RING_CLUSTER_ERR_XCD = 1, RING_CLUSTER_ERR_START = 2, RING_CLUSTER_ERR_WAIT = 3 };
 bool ring_cluster_applicable(int N, int k);               // the shape alone
 size_t ring_cluster_workspace_bytes(int nbt);
 bool ring_uses_cluster(int N, int k, int B, int T);       // applicable, switched on, whole pairs of batch tiles, and the device has the compute units
+bool ring_uses_cluster_bptt(int N, int k, int B, int T);  // the BPTT on clusters: the same conditions, and only when asked for (RINGATTR_CLUSTER_BPTT=1)
 int ring_cluster_error();                                 // the host word: non-zero once a cluster kernel gave up waiting
 int ring_cluster_take_error();                            // the same, the first time it is found set; 0 afterwards
 int ring_cluster_pack_order(int N, int B, int T);        // the column order (ring_pack_weights_kernel's split_k) its kernel for that shape reads
 hipError_t ring_launch_fwd_cluster(const RingFwdArgs& a, hipStream_t st);
+size_t ring_cluster_bptt_workspace_bytes(int nbt);
+hipError_t ring_launch_bptt_cluster(const RingBpttArgs& a, hipStream_t st);   // a.cluster_ws; Wpack transposed, in ring_cluster_pack_order, J1 * Wo^T + J0 as matrix 0
 
 // Step-per-launch kernels for 512 < N <= 2048, NC in {16, 24, 32} (ring_bign.hip).
 bool ring_wide_applicable(int NC);

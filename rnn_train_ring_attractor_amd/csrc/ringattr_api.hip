@@ -184,6 +184,8 @@ size_t ringattr_bwd_workspace_bytes(int N, int a_dim, int seq_len, int batch_siz
   if (make_geo(N, a_dim, seq_len, batch_size, g) != RINGATTR_OK) return 0;
   size_t s = g.wpack_bytes + g.pair_bytes + g.partial_bytes + g.carry_bytes + g.trig_bytes;
   if (!have_saved) s += g.wpack_bytes + g.side_bytes + g.pair_bytes;
+  // (the cluster BPTT's scratch area is asked for wherever its shape applies, switched on or not)
+  if (ring_cluster_applicable(N, a_dim)) s += ring_cluster_bptt_workspace_bytes(g.nbt);
   return s;
 }
 
@@ -425,6 +427,11 @@ static int bwd_impl(const char* who, const void* grad_output, const void* loss_w
     rfrag = r;
   }
 
+  // The cluster BPTT (N = 512, where ring_uses_cluster_bptt says so; no dL/dA, no fused loss head) packs its own
+  // transposed copy, in its column order with J1 * Wo^T + J0 as matrix 0; its scratch area is the workspace's tail.
+  const bool bptt_cluster = !step_family && !grad_A && !loss_workspace && ring_uses_cluster_bptt(N, a_dim, batch_size, seq_len) &&
+                            !ring_uses_resident(N, a_dim);
+  void* const cluster_ws = bptt_cluster ? (char*)workspace + need - ring_cluster_bptt_workspace_bytes(g.nbt) : nullptr;
   // the weight-resident BPTT kernel takes J1 * Wo + J0 in the transposed Wo fragments
   const bool resident = ring_uses_resident(N, a_dim);
   const bool bptt_resident = resident;
@@ -435,7 +442,11 @@ static int bwd_impl(const char* who, const void* grad_output, const void* loss_w
   if (noted != 0 && (noted == 3) != (family == 3))
     return fail(RINGATTR_ERR_INVALID, "%s: the saved buffer was filled by the other kernel family (its derivative record "
                 "has a different layout); run forward and backward under the same RINGATTR_BLOCK setting", who);
-  if (saved && saved_note_matches(note, family, N, a_dim, seq_len, batch_size, J0, J1, Wo, Wa)) {
+  if (bptt_cluster) {
+    e = ring_launch_pack((const float*)Wo, (const float*)Wa, wb, N, a_dim, g.NC, 1,
+                         ring_cluster_pack_order(N, batch_size, seq_len), J1, J0, st);
+    if (e != hipSuccess) return hip_fail(e, "pack transposed weights");
+  } else if (saved && saved_note_matches(note, family, N, a_dim, seq_len, batch_size, J0, J1, Wo, Wa)) {
     // the forward left the transposed copy, in the form this BPTT kernel expects, behind the saved activations
     wb = (char*)const_cast<void*>(saved) + g.side_bytes + g.pair_bytes;
   } else {
@@ -473,6 +484,7 @@ static int bwd_impl(const char* who, const void* grad_output, const void* loss_w
   b.T = seq_len;
   b.B = batch_size;
   b.nbt = g.nbt;
+  b.cluster_ws = cluster_ws;
   e = ring_launch_bptt(b, g.NC, st);
   if (e != hipSuccess) return hip_fail(e, "BPTT launch");
   if (step_family && grad_A) {

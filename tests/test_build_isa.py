@@ -125,24 +125,38 @@ def cluster_asm(tmp_path_factory):
     return out.read_text(), proc.stderr
 
 
-@pytest.mark.parametrize("save", [0, 1], ids=["history_only", "with_record"])
-@pytest.mark.parametrize("act", [0, 1, 2, 3], ids=["relu", "gelu", "tanh", "silu"])
-def test_cluster_forward_leaves_in_flight_registers_alone(cluster_asm, act, save):
-    asm, _ = cluster_asm
-    name = f"_Z24ring_fwd_cluster8_kernelILi{act}ELb{save}EEv11RingFwdArgs15RingClusterArgs"
+def _sregs(tok):
+    out = set()
+    for m in re.finditer(r"\bs\[(\d+):(\d+)\]", tok):
+        out |= set(range(int(m.group(1)), int(m.group(2)) + 1))
+    for m in re.finditer(r"\bs(\d+)\b", tok):
+        out.add(int(m.group(1)))
+    return out
+
+
+def _function_body(asm, name):
     i = asm.index(name + ":")
-    body = asm[i:asm.index(".Lfunc_end", i)].split("\n")
-    fifo, in_asm, loads = [], False, 0
-    for ln in body + body:                      # second pass models the loop back edge
+    return asm[i:asm.index(".Lfunc_end", i)].split("\n")
+
+
+def _instructions(body):
+    """(inside an asm statement?, instruction text) for every instruction of a function body."""
+    in_asm = False
+    for ln in body:
         t = ln.strip()
         if t.startswith(";;#ASMSTART"):
             in_asm = True
-            continue
-        if t.startswith(";;#ASMEND"):
+        elif t.startswith(";;#ASMEND"):
             in_asm = False
-            continue
-        if not t or t[0] in ";.":
-            continue
+        elif t and t[0] not in ";.":
+            yield in_asm, t
+
+
+def _check_in_flight(body):
+    """Asserts that nothing touches the destination of an asm-issued load before a wait covers it; returns the
+    number of such loads seen (over two passes of the body: the second models the loop back edge)."""
+    fifo, loads = [], 0
+    for in_asm, t in list(_instructions(body)) * 2:
         if in_asm and t.startswith("global_load"):
             fifo.append(_regs(t.split()[1].rstrip(",")))
             loads += 1
@@ -159,16 +173,65 @@ def test_cluster_forward_leaves_in_flight_registers_alone(cluster_asm, act, save
         ops = t.split(None, 1)
         used = _regs(ops[1]) if len(ops) > 1 else set()
         assert not (used & pending), f"in-flight registers {sorted(used & pending)} touched by: {t}"
+    return loads
+
+
+CLUSTER_KERNELS = [f"_Z24ring_fwd_cluster8_kernelILi{act}ELb{save}EEv11RingFwdArgs15RingClusterArgs"
+                   for act in range(4) for save in (0, 1)] + \
+                  [f"_Z25ring_bptt_cluster8_kernelILb{gri}EEv12RingBpttArgs15RingClusterArgs" for gri in (0, 1)]
+
+
+@pytest.mark.parametrize("save", [0, 1], ids=["history_only", "with_record"])
+@pytest.mark.parametrize("act", [0, 1, 2, 3], ids=["relu", "gelu", "tanh", "silu"])
+def test_cluster_forward_leaves_in_flight_registers_alone(cluster_asm, act, save):
+    asm, _ = cluster_asm
+    loads = _check_in_flight(_function_body(asm, f"_Z24ring_fwd_cluster8_kernelILi{act}ELb{save}EEv11RingFwdArgs15RingClusterArgs"))
     assert loads == 2 * 14          # early half: 2 previous-state, gates, flags, 4 operand; late half: gates, flags, 4 operand
 
 
-def test_cluster_forward_uses_no_scratch(cluster_asm):
+@pytest.mark.parametrize("gri", [0, 1], ids=["weights_only", "with_grad_r_init"])
+def test_cluster_bptt_leaves_in_flight_registers_alone(cluster_asm, gri):
+    asm, _ = cluster_asm
+    loads = _check_in_flight(_function_body(asm, f"_Z25ring_bptt_cluster8_kernelILb{gri}EEv12RingBpttArgs15RingClusterArgs"))
+    assert loads == 2 * 20          # early half: 8 epilogue inputs, gates, flags, 4 operand; late half: gates, flags, 4 operand
+
+
+@pytest.mark.parametrize("name", CLUSTER_KERNELS)
+def test_cluster_asm_memory_instructions_keep_their_hazard_distances(cluster_asm, name):
+    """The compiler's hazard recognizer does not look inside asm statements.  Two hazards of gfx950 concern the
+    vector-memory instructions issued there: a store of more than 8 bytes per lane reads its data registers during
+    the two wait states after it issues (a vector-ALU write to them in that window changes what is stored: the store
+    carries its own s_nop 1), and a vector-ALU write of a scalar register (v_readfirstlane, v_cmp) needs five wait
+    states before a vector-memory instruction reads it."""
+    asm, _ = cluster_asm
+    ins = list(_instructions(_function_body(asm, name)))
+    wide = 0
+    for k, (in_asm, t) in enumerate(ins):
+        if not (in_asm and t.startswith(("global_load", "global_store"))):
+            continue
+        if t.startswith(("global_store_dwordx4", "global_store_dwordx3")):
+            wide += 1
+            assert ins[k + 1] == (True, "s_nop 1"), f"no wait states behind: {t}"
+        need = _sregs(t)
+        ws = 0
+        for _, pt in reversed(ins[max(0, k - 8):k]):
+            if ws >= 5:
+                break
+            op = pt.split()[0]
+            if op.startswith("v_"):
+                dst = pt.split(None, 1)[1].split(",")[0]
+                assert not (_sregs(dst) & need), f"{pt} writes a scalar register {ws} wait states before: {t}"
+            ws += int(pt.split()[1]) + 1 if op == "s_nop" else 1
+    assert wide >= 4
+
+
+def test_cluster_kernels_use_no_scratch(cluster_asm):
     _, remarks = cluster_asm
     seen = 0
     for b in re.split(r"remark: Function Name: ", remarks)[1:]:
         name = b.split()[0]
-        if name.startswith("_Z24ring_fwd_cluster8_kernel"):
+        if name.startswith(("_Z24ring_fwd_cluster8_kernel", "_Z25ring_bptt_cluster8_kernel")):
             seen += 1
             m = re.search(r"ScratchSize \[bytes/lane\]: (\d+)", b)
             assert int(m.group(1)) == 0, f"{name} spills {m.group(1)} bytes per lane"
-    assert seen == 8
+    assert seen == 10

@@ -4,7 +4,9 @@ agreement with the streaming kernels, run-to-run reproducibility (a race between
 difference between two runs), the choice of kernel by shape, and the exit taken when a wait runs out.
 
 RINGATTR_CLUSTER=1 makes the kernel run on every shape it can (whole pairs of batch tiles); left alone it only takes
-shapes with at least four pairs per cluster, where it is ahead."""
+shapes with at least four pairs per cluster, where it is ahead.  The BPTT on the same clusters runs only under
+RINGATTR_CLUSTER_BPTT=1 (it is not ahead of the streaming kernel anywhere); its tests compare it with that kernel on
+the same saved record, with the fp64 oracle where the CPU can afford the batch, and run to run."""
 import os
 import subprocess
 import sys
@@ -153,6 +155,89 @@ def test_kernel_choice_by_shape(gpu_device, monkeypatch):
     p = make_problem(314, 8192, 16, K, 512, action="lr")
     _forward(p, "tanh", gpu_device, saved=False)
     assert "cluster" not in _fwd_kernel_name()
+
+
+# name, B, T, act, grad_r_init asked for
+BPTT_CASES = [
+    ("one_pair_odd_length",  32,  9, "tanh", True),
+    ("one_pair_even_length", 32,  8, "tanh", False),
+    ("one_step",             64,  1, "gelu", True),
+    ("pairs_over_xcds",     416,  6, "silu", True),
+    ("two_per_cluster",    2112,  5, "tanh", False),
+    ("four_per_cluster",   8192,  6, "gelu", True),
+    ("uneven_rotation",    6400,  7, "tanh", True),
+]
+
+
+def _backward_full(p, act, dev, hist, sv, want_r_init):
+    from rnn_train_ring_attractor_amd import rnn_cuda
+    A, Wa, Wo, r0, G = (_t(p[k], dev) for k in ("A", "Wa", "Wo", "r0", "G"))
+    gWa, gWo = torch.zeros_like(Wa), torch.zeros_like(Wo)
+    gr = torch.full_like(r0, float("nan")) if want_r_init else None
+    rnn_cuda._Bwd.bwd(G, A, Wa, -0.1, 0.1, Wo, hist, r_init=r0, grad_Wa=gWa, grad_Wo=gWo, alpha=0.15,
+                      activation_type=ACTS[act], saved=sv, grad_r_init=gr)
+    torch.cuda.synchronize()
+    return gWa.cpu().numpy().astype(np.float64), gWo.cpu().numpy().astype(np.float64), \
+        (gr.cpu().numpy().astype(np.float64) if want_r_init else None)
+
+
+def _bptt_kernel_name():
+    from rnn_train_ring_attractor_amd import _lib
+    return _lib.last_kernel_names().get("bptt", "")
+
+
+@pytest.mark.parametrize("case", BPTT_CASES, ids=[c[0] for c in BPTT_CASES])
+def test_cluster_bptt_against_the_streaming_kernel_and_the_oracle(case, gpu_device, monkeypatch):
+    from rnn_train_ring_attractor_amd import rnn_cuda
+    name, B, T, act, want_r_init = case
+    print(f"[case] cluster bptt {name} B={B} T={T} {act} grad_r_init={want_r_init}", flush=True)
+    p = make_problem(411, B, T, K, N, action="dense")
+    monkeypatch.setenv("RINGATTR_CLUSTER", "0")
+    hist, sv = _forward(p, act, gpu_device)
+    ga_s, go_s, gr_s = _backward_full(p, act, gpu_device, hist, sv, want_r_init)
+    assert "cluster" not in _bptt_kernel_name()
+    # the cluster kernel's scratch (carry records, held halves, the exchange, the copy of g with its zero tail) starts
+    # out as NaN patterns: whatever it read before writing it would show
+    plain_workspace = rnn_cuda._workspace
+    monkeypatch.setattr(rnn_cuda, "_workspace",
+                        lambda nbytes, device, stream: plain_workspace(nbytes, device, stream).fill_(0xFF))
+    monkeypatch.setenv("RINGATTR_CLUSTER", "1")
+    monkeypatch.setenv("RINGATTR_CLUSTER_BPTT", "1")
+    ga, go, gr = _backward_full(p, act, gpu_device, hist, sv, want_r_init)
+    assert "ring_bptt_cluster8_kernel" in _bptt_kernel_name()
+    ga2, go2, gr2 = _backward_full(p, act, gpu_device, hist, sv, want_r_init)
+    assert np.isfinite(ga).all() and np.isfinite(go).all()
+    errs = [O.max_rel_err(ga, ga_s), O.max_rel_err(go, go_s)]
+    if want_r_init:
+        assert np.isfinite(gr).all()
+        errs.append(O.max_rel_err(gr, gr_s))
+    print(f"[measured] {name}: vs the streaming BPTT " + ", ".join(f"{e:.2e}" for e in errs), flush=True)
+    assert max(errs) <= 1e-2
+    # one order of arithmetic, flags in memory between the members: a read of an incomplete operand would differ run to run
+    assert np.array_equal(ga, ga2) and np.array_equal(go, go2) and (not want_r_init or np.array_equal(gr, gr2))
+    if B <= 512:
+        ref_h, _ = O.forward_dense(p["A"], p["Wa"], -0.1, 0.1, p["Wo"], p["r0"], 0.15, act)
+        g = O.backward_dense(p["G"], p["A"], p["Wa"], -0.1, 0.1, p["Wo"], ref_h, p["r0"], 0.15, act)
+        assert O.cosine(go, g["grad_Wo"]) >= GRAD_COS and O.cosine(ga, g["grad_Wa"]) >= GRAD_COS
+        assert O.max_rel_err(go, g["grad_Wo"]) <= GRAD_TOL and O.max_rel_err(ga, g["grad_Wa"]) <= GRAD_TOL
+        if want_r_init:
+            assert O.max_rel_err(gr, g["grad_r_init"]) <= GRAD_TOL
+
+
+def test_cluster_bptt_runs_only_where_asked_for(gpu_device, monkeypatch):
+    monkeypatch.delenv("RINGATTR_CLUSTER", raising=False)
+    monkeypatch.delenv("RINGATTR_CLUSTER_BPTT", raising=False)
+    p = make_problem(412, 8192, 16, K, N, action="lr")
+    hist, sv = _forward(p, "tanh", gpu_device)
+    assert "cluster" in _fwd_kernel_name()
+    _backward_full(p, "tanh", gpu_device, hist, sv, False)
+    assert "cluster" not in _bptt_kernel_name(), _bptt_kernel_name()
+    monkeypatch.setenv("RINGATTR_CLUSTER_BPTT", "1")
+    _backward_full(p, "tanh", gpu_device, hist, sv, False)
+    assert "ring_bptt_cluster8_kernel" in _bptt_kernel_name()
+    monkeypatch.setenv("RINGATTR_CLUSTER", "0")          # the forward's switch turns both off
+    _backward_full(p, "tanh", gpu_device, hist, sv, False)
+    assert "cluster" not in _bptt_kernel_name()
 
 
 _GIVE_UP_SCRIPT = r"""
