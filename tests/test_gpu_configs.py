@@ -173,15 +173,20 @@ def test_widest_ring_at_a_training_batch(gpu_device):
     assert O.max_rel_err(part[2].cpu().numpy(), g["grad_Wo"]) <= GRAD_TOL
 
 
-@pytest.mark.parametrize("forward", ["cluster", "streaming"])
+@pytest.mark.parametrize("forward", ["cluster", "streaming", "cluster_with_bptt"])
 def test_long_sequence_shape_at_full_size(gpu_device, monkeypatch, forward):
     """N=512, B=8192, T=512, tanh at its real size (inputs generated on the device): bitwise repeatable, a 32-row
     slice run alone reproduces its rows of the full batch bit for bit and agrees with the fp64 oracle, the
     gradient is linear in grad_output, two half-batch shards add up to the full batch.  Once per forward kernel of
     this width (left alone the library runs the full batch on the cluster kernel and the small shards on the
-    streaming ones, which round Wo differently; the row-for-row identities hold inside one family)."""
+    streaming ones, which round Wo differently; the row-for-row identities hold inside one family), and once more with
+    the BPTT on the clusters as well (off unless asked for)."""
     from rnn_train_ring_attractor_amd import ring_rnn_cuda_func
-    monkeypatch.setenv("RINGATTR_CLUSTER", "1" if forward == "cluster" else "0")
+    monkeypatch.setenv("RINGATTR_CLUSTER", "0" if forward == "streaming" else "1")
+    if forward == "cluster_with_bptt":
+        monkeypatch.setenv("RINGATTR_CLUSTER_BPTT", "1")
+    else:
+        monkeypatch.delenv("RINGATTR_CLUSTER_BPTT", raising=False)
     print(f"[case] long sequence N=512 B=8192 T=512 tanh (full size), {forward} forward", flush=True)
     B, T, k, N = 8192, 512, 2, 512
     # J1 = 0.5 here: at the configuration's own J1 = 1 the dynamics are marginally stable and the bf16 rounding of Wo
