@@ -142,6 +142,31 @@ def test_cluster_forward_is_reproducible_run_to_run(gpu_device, monkeypatch):
             assert torch.equal(h, h0) and torch.equal(s, s0)
 
 
+def test_cluster_forwards_on_two_streams(gpu_device, monkeypatch):
+    """Every cluster kernel wants all compute units for its own workgroups.  Two of them launched back to back on two
+    streams still both finish with the right result (the second one's workgroups become resident as the first one's
+    leave; every wait for a sibling is bounded in any case)."""
+    from rnn_train_ring_attractor_amd import rnn_cuda
+    monkeypatch.setenv("RINGATTR_CLUSTER", "1")
+    B, T, act = 8192, 48, "tanh"
+    print(f"[case] two cluster forwards on two streams B={B} T={T}", flush=True)
+    p = make_problem(316, B, T, K, N, action="lr")
+    A, Wa, Wo, r0 = (_t(p[k], gpu_device) for k in ("A", "Wa", "Wo", "r0"))
+    ref, _ = _forward(p, act, gpu_device, saved=False)
+    assert "ring_fwd_cluster8_kernel" in _fwd_kernel_name()
+    streams = [torch.cuda.Stream(device=gpu_device) for _ in range(2)]
+    out = [torch.full((T, B, N), float("nan"), device=gpu_device) for _ in range(2)]
+    torch.cuda.synchronize()
+    for _ in range(3):
+        for st, h in zip(streams, out):
+            with torch.cuda.stream(st):
+                rnn_cuda._Fwd.fwd(A, Wa, -0.1, 0.1, Wo, r0, h, 0.15, ACTS[act])
+        torch.cuda.synchronize()
+        assert torch.equal(out[0], ref) and torch.equal(out[1], ref)
+    _forward(p, act, gpu_device, saved=False)      # (a member that had given up would be reported by this call)
+    assert "ring_fwd_cluster8_kernel" in _fwd_kernel_name()
+
+
 def test_kernel_choice_by_shape(gpu_device, monkeypatch):
     """Unasked, the cluster kernel takes shapes with at least four batch-tile pairs per cluster; RINGATTR_CLUSTER=0
     keeps it off, and shapes it cannot run (ragged batch, other widths) never see it."""
