@@ -177,6 +177,10 @@ def main():
     ap.add_argument("--precise-wo", action="store_true",
                     help="Wo enters the contraction as two bf16 operands (hi + lo), one more matrix per step: the "
                          "accuracy option for long, marginally stable sequences (never the metric's configuration)")
+    ap.add_argument("--cluster-bptt", action="store_true",
+                    help="N = 512 workloads: run the BPTT on the compute-unit clusters as well (sets "
+                         "RINGATTR_CLUSTER_BPTT=1; off by default because it is not faster; never the metric's "
+                         "configuration)")
     ap.add_argument("--event-stride", type=int, default=0,
                     help="bracket every n-th launch of each kernel with HIP events inside the timed region "
                          "(0: steps // 4 clamped to 1..8)")
@@ -195,6 +199,8 @@ def main():
     from rnn_train_ring_attractor_amd import _lib, ring_rnn_cuda_func
     from rnn_train_ring_attractor_amd import ring_rnn_cuda as _op
     _op.RECOMPUTE_IN_BACKWARD = bool(args.recompute)
+    if args.cluster_bptt:
+        os.environ["RINGATTR_CLUSTER_BPTT"] = "1"
     _op.PRECISE_WO = bool(args.precise_wo)
     if not torch.cuda.is_available():
         sys.exit("bench.py: no GPU visible; the HIP path has no CPU fallback")
@@ -319,7 +325,7 @@ def main():
         "value": value, "unit": "sample-steps/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": args.workload + ("_recompute" if args.recompute else "") + ("_precise_wo" if args.precise_wo else ""), "N": N, "B": B, "T": T, "a_dim": k, "activation": cfg["act"],
+        "config": {"workload": args.workload + ("_recompute" if args.recompute else "") + ("_precise_wo" if args.precise_wo else "") + ("_cluster_bptt" if args.cluster_bptt else ""), "N": N, "B": B, "T": T, "a_dim": k, "activation": cfg["act"],
                    "mode": {"train": "forward + backward", "infer": "forward only (no saved activations)",
                             "gain": "gain MLPs + forward + backward (MLP gradients through dL/d action_signal)"}[mode],
                    "grad_output": "gradient of the cos-sim + 0.2*bump-amplitude loss pair, precomputed" if train else None},

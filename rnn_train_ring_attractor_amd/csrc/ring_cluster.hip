@@ -1028,13 +1028,10 @@ static bool cluster_can_run(int N, int k, int B, int T, int* ppc, int* cus_out) 
   const char* v = getenv("RINGATTR_CLUSTER");
   if (v && v[0] == '0') return false;
   if (ring_cluster_error()) return false;
-  static int cus = 0;
-  if (cus == 0) {
-    int dev = 0, n = 0;
-    if (hipGetDevice(&dev) != hipSuccess ||
-        hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = -1;
-    cus = n;
-  }
+  int dev = 0, cus = 0;   // (of the current device: asked every time, a process may hold several kinds)
+  if (hipGetDevice(&dev) != hipSuccess ||
+      hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+    return false;
   const ClusterGeo g = cluster_geo(B / 16);
   if (g.grid > cus) return false;   // every workgroup needs a compute unit of its own, all at once
   *ppc = g.ppc;
