@@ -538,11 +538,12 @@ __global__ __launch_bounds__(512) void ring_fwd_cluster8_kernel(RingFwdArgs p, R
 //     carry_t = (1 - alpha) G_{t+1} + [g_{t+1} (J1 Wo + J0)] + sum_c A_c(t+1) [g_{t+1} Wa_c]     (0 at t = T-1)
 //     G_t = grad_output_t + carry_t,      g_t = (alpha F'(re_t)) G_t                              (the record carries alpha)
 // with the products in brackets taken over all N neurons of g_{t+1}: that is what the members exchange, by the
-// forward's protocol with s in the place of its t (state s = g_{t+1}; a pair's first visit has no products).  Wpack holds
-// the transposed matrices in this kernel's column order, J1 Wo^T + J0 as matrix 0.  What a pair carries from one
-// visit to the next besides the exchanged g lives in a private scratch record per lane: (1 - alpha) G_t for its four
-// rows (fp32) and, behind odd steps, the bf16 g of those rows: the copy of g for the weight-gradient kernel keeps
-// steps 2j and 2j+1 side by side in one 16-byte slot, and the even step that follows stores the slot whole.
+// forward's protocol with s in the place of its t (state s = g_{t+1}; a pair's first visit has no products).  Wpack
+// holds the transposed matrices in this kernel's column order, J1 Wo^T + J0 as matrix 0.  What a pair carries from
+// one visit to the next besides the exchanged g lives in a private scratch record per lane (registers and LDS are
+// full of weights): (1 - alpha) G_t for its four rows (fp32) and, behind odd steps, the bf16 g of those rows -- the
+// copy of g for the weight-gradient kernel keeps steps 2j and 2j+1 side by side in one 16-byte slot, and the even
+// step that follows stores the slot whole.
 // One more visit (t = -1) forms dL/dr_init when it is asked for.  No dL/dA and no fused loss head here: the caller
 // runs those on the streaming kernel.
 // ------------------------------------------------------------------------------------------------
