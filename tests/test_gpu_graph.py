@@ -12,17 +12,24 @@ from tests.ring_cases import make_problem
 pytestmark = pytest.mark.gpu
 
 CASES = [
-    # name,        B,  T, k,   N, act
-    ("resident",  48, 10, 2, 256, "gelu"),
-    ("streaming", 40, 12, 2, 120, "tanh"),
-    ("step",      24,  5, 3, 640, "silu"),
+    # name,        B,  T, k,   N, act, environment
+    ("resident",  48, 10, 2, 256, "gelu", {}),
+    ("streaming", 40, 12, 2, 120, "tanh", {}),
+    ("step",      24,  5, 3, 640, "silu", {}),
+    # the N = 512 kernels on clusters of compute units: their flags are cleared by a kernel of the captured stream
+    ("cluster_forward", 96, 7, 2, 512, "tanh", {"RINGATTR_CLUSTER": "1"}),
+    ("cluster_forward_and_bptt", 64, 6, 2, 512, "gelu", {"RINGATTR_CLUSTER": "1", "RINGATTR_CLUSTER_BPTT": "1"}),
 ]
 
 
 @pytest.mark.parametrize("case", CASES, ids=[c[0] for c in CASES])
-def test_forward_backward_replays_from_a_graph(case, gpu_device):
-    from rnn_train_ring_attractor_amd import ring_rnn_cuda_func
-    name, B, T, k, N, act = case
+def test_forward_backward_replays_from_a_graph(case, gpu_device, monkeypatch):
+    from rnn_train_ring_attractor_amd import ring_rnn_cuda_func, _lib
+    name, B, T, k, N, act, env = case
+    for key in ("RINGATTR_CLUSTER", "RINGATTR_CLUSTER_BPTT"):
+        monkeypatch.delenv(key, raising=False)
+    for key, val in env.items():
+        monkeypatch.setenv(key, val)
     print(f"[case] graph {name} B={B} T={T} k={k} N={N} {act}", flush=True)
     J0, J1 = -0.05, 0.4
     problems = [make_problem(900 + i, B, T, k, N, action="dense") for i in range(3)]
@@ -68,6 +75,9 @@ def test_forward_backward_replays_from_a_graph(case, gpu_device):
         assert torch.equal(got[1], eWa.grad), f"replay {rep}: grad_Wa differs from the eager run"
         assert torch.equal(got[2], eWo.grad), f"replay {rep}: grad_Wo differs from the eager run"
         assert float(got[1].abs().max()) > 0
+    names = _lib.last_kernel_names()
+    assert ("cluster" in names.get("fwd", "")) == ("RINGATTR_CLUSTER" in env)
+    assert ("cluster" in names.get("bptt", "")) == ("RINGATTR_CLUSTER_BPTT" in env)
 
 
 def test_device_counted_optimizer_matches_the_host_counted_one(gpu_device):
